@@ -1,0 +1,178 @@
+/*
+ * libmsamp_hip.so -- C ABI of the MI355X (gfx950) FP8 hot path.
+ *
+ * Every entry point borrows raw device pointers for the duration of the enqueue, allocates
+ * nothing, enqueues on the caller's stream and returns without synchronising.  Return value:
+ * 0 on success, negative on error (MSAMP_ERR_*); msamp_last_error() gives a thread-local
+ * message.  Data-type codes are the reference's QType values
+ * (msamp/common/dtype/dtypes.py:30-36).
+ *
+ * The functions replace, one for one, the native calls the reference makes for this path:
+ * the five TransformerEngine extension calls behind
+ * msamp/common/utils/transformer_engine_wrapper.py:93-176, the jit-scripted scale rule
+ * (msamp/common/tensor/meta.py:37-56), the amax-window update
+ * (msamp/optim/optimizer.py:83-108) and the msamp_adamw extension
+ * (msamp/optim/adamw.cu:77-153).
+ */
+#ifndef MSAMP_HIP_H_
+#define MSAMP_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* stream handle: a hipStream_t passed as an opaque pointer (NULL = the null stream) */
+typedef void* msamp_stream_t;
+
+enum {
+    MSAMP_DT_BYTE = 0,
+    MSAMP_DT_INT32 = 1,
+    MSAMP_DT_F32 = 2,
+    MSAMP_DT_F16 = 3,
+    MSAMP_DT_BF16 = 4,
+    MSAMP_DT_E4M3 = 5,
+    MSAMP_DT_E5M2 = 6
+};
+
+enum {
+    MSAMP_OK = 0,
+    MSAMP_ERR_DTYPE = -1,     /* unsupported data type code            */
+    MSAMP_ERR_SHAPE = -2,     /* bad size, shape or alignment          */
+    MSAMP_ERR_NULL = -3,      /* required pointer is NULL              */
+    MSAMP_ERR_WORKSPACE = -4, /* workspace missing or too small        */
+    MSAMP_ERR_HIP = -100      /* -100 - hipError_t of the failing call */
+};
+
+/* flags of msamp_cast_to_fp8_intime / msamp_cast_transpose_intime */
+enum {
+    MSAMP_FLAG_NAN_TO_INF = 1 /* amax: NaN/+Inf -> +Inf before the scale rule (cast.py:37-40, sync=True) */
+};
+
+/* bytes of zero-initialised device workspace the *_intime and fused-AdamW entry points need;
+ * the library leaves it zeroed again when each call's kernels finish.  Calls that share one
+ * workspace must be ordered on one stream. */
+#define MSAMP_WORKSPACE_BYTES 256
+
+int msamp_hip_version(void);
+const char* msamp_last_error(void);
+
+/* amax[0] = max|x| over n elements, NaN propagating (torch abs().max(), cast.py:34).
+ * dtype: F32/F16/BF16.  workspace: MSAMP_WORKSPACE_BYTES. */
+int msamp_amax(const void* x, int dtype, size_t n, float* amax, void* workspace, msamp_stream_t stream);
+
+/* out[i] = rule(amax[i], fallback scale_in[i]) for i < n; the pow-2 scale rule of
+ * ScalingMeta.compute_scaling_factor (meta.py:37-56).  scale_in may have 1 element
+ * (scale_in_n == 1, broadcast) or n.  out may alias scale_in. */
+int msamp_compute_scaling_factor(const float* amax, const float* scale_in, int scale_in_n, float* scale_out, int n,
+                                 float fp_max, int margin, msamp_stream_t stream);
+
+/* Delayed-scaling cast: tex.cast_to_fp8 (transformer_engine_wrapper.py:106-120).
+ * out[i] = fp8_sat_rne(float(x[i]) * *scale); if amax != NULL: *amax = atomic-max(*amax, max|x|)
+ * (NaN elements skipped); if scale_inv != NULL: *scale_inv = 1 / *scale. */
+int msamp_cast_to_fp8(const void* x, int in_dtype, size_t n, const float* scale, float* amax, float* scale_inv,
+                      uint8_t* out, int fp8_type, msamp_stream_t stream);
+
+/* In-time cast: the whole of TypeCast.cast_to_fp8's in-time branch (cast.py:33-62) --
+ * amax[0] = max|x|, *scale = rule(amax[0], *scale, fp_max(fp8_type), margin), quantize,
+ * *scale_inv = 1 / *scale.  Two passes over x; the second runs back to front so that it
+ * meets the cache lines the first pass left behind. */
+int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
+                             uint8_t* out, int fp8_type, int margin, int flags, void* workspace,
+                             msamp_stream_t stream);
+
+/* tex.cast_from_fp8 (transformer_engine_wrapper.py:123-137): out[i] = otype(float(q[i]) * *scale_inv). */
+int msamp_cast_from_fp8(const uint8_t* q, int fp8_type, size_t n, const float* scale_inv, void* out, int out_dtype,
+                        msamp_stream_t stream);
+
+/* tex.fused_cast_transpose (transformer_engine_wrapper.py:140-162), any rows/cols (the reference
+ * pads to multiples of 16 and slices; the result is the same): out[r][c] and out_t[c][r]. */
+int msamp_cast_transpose(const void* x, int in_dtype, int rows, int cols, const float* scale, float* amax,
+                         float* scale_inv, uint8_t* out, uint8_t* out_t, int fp8_type, msamp_stream_t stream);
+
+/* in-time variant of the above (cast.py:33-52 with fuse_transpose=True) */
+int msamp_cast_transpose_intime(const void* x, int in_dtype, int rows, int cols, float* scale, float* amax,
+                                float* scale_inv, uint8_t* out, uint8_t* out_t, int fp8_type, int margin, int flags,
+                                void* workspace, msamp_stream_t stream);
+
+/* tex.fp8_transpose (transformer_engine_wrapper.py:165-176): out[c][r] = q[r][c]. */
+int msamp_fp8_transpose(const uint8_t* q, int rows, int cols, uint8_t* out, msamp_stream_t stream);
+
+/* Scaled 16/32-bit "ScalingTensor" payloads (cast.py:68-95,122-136):
+ * out[i] = otype(float(x[i]) * *scale) with IEEE overflow (no saturation). */
+int msamp_scale_cast(const void* x, int in_dtype, size_t n, const float* scale, void* out, int out_dtype,
+                     msamp_stream_t stream);
+
+/* Device part of LBOptimizer._update_scaling_factors (optimizer.py:91-108) on flattened metas:
+ * scales (n), amaxs (n x window, row-major).  bad[i] (nullable, n bytes) = 1 where amaxs[i][0]
+ * was not finite (the caller resets that meta's host-side counter). */
+int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int n, int window, float fp_max, int margin,
+                       msamp_stream_t stream);
+
+/* tex.te_gemm as Gemm.fp8_gemm calls it (gemm.py:121-144; transa=True, transb=False):
+ * D[N][M] = (B[N][K] . A[M][K]^T) * *a_scale_inv * *b_scale_inv (+ bias[M]) (+ D if accumulate).
+ * A, B: FP8 bytes, row-major, K contiguous, K % 16 == 0, 16-byte aligned.  d_dtype: F32/F16/BF16.
+ * bias: nullable, bias_dtype F32/F16/BF16. */
+int msamp_fp8_gemm(const uint8_t* a, int a_type, const float* a_scale_inv, const uint8_t* b, int b_type,
+                   const float* b_scale_inv, void* d, int d_dtype, int m, int n, int k, int accumulate,
+                   const void* bias, int bias_dtype, msamp_stream_t stream);
+
+/* msamp_adamw.adamw_fp8_stage1_compute (adamw.cu:99-127): fp32 param/grad, quantized moments;
+ * updates param in place and atomically maxes |m'|, |v'| into the two amax cells.
+ * exp_avg_dtype: E4M3/E5M2/F16/F32, exp_avg_sq_dtype: F16/F32/E4M3/E5M2. */
+int msamp_adamw_fp8_stage1(float* param, const float* grad, size_t n, const void* exp_avg, int exp_avg_dtype,
+                           float exp_avg_factor, float* exp_avg_amax, float beta1, const void* exp_avg_sq,
+                           int exp_avg_sq_dtype, float exp_avg_sq_factor, float* exp_avg_sq_amax, float beta2,
+                           float eps, int step, float lr, int bias_correction, msamp_stream_t stream);
+
+/* msamp_adamw.adamw_fp8_stage2_compute (adamw.cu:129-153): rewrite the moments with new scales. */
+int msamp_adamw_fp8_stage2(const float* grad, size_t n, void* exp_avg, int exp_avg_dtype, float exp_avg_factor,
+                           float new_exp_avg_factor, float beta1, void* exp_avg_sq, int exp_avg_sq_dtype,
+                           float exp_avg_sq_factor, float new_exp_avg_sq_factor, float beta2, msamp_stream_t stream);
+
+/* One tensor of the fused multi-tensor step below.  The array of descriptors lives in DEVICE
+ * memory and is written by the kernels (acc/saved are scratch: zero-initialise acc once; the
+ * library leaves it zero). */
+typedef struct msamp_adamw_tensor {
+    void* weight;            /* weight_dtype payload (FP8 codes or scaled fp16), updated in place */
+    const uint8_t* grad;     /* FP8 codes (grad_dtype)                                            */
+    uint8_t* exp_avg;        /* E4M3 codes, updated in place                                      */
+    uint16_t* exp_avg_sq;    /* scaled fp16, updated in place                                     */
+    float* w_scale;          /* weight meta: scale, scale_inv, amax[0] -- read, then rewritten    */
+    float* w_scale_inv;
+    float* w_amax;
+    const float* g_scale_inv;
+    float* m_scale;          /* exp_avg meta                                                      */
+    float* m_scale_inv;
+    float* m_amax;
+    float* v_scale;          /* exp_avg_sq meta                                                   */
+    float* v_scale_inv;
+    float* v_amax;
+    uint64_t numel;
+    uint32_t acc[3];         /* scratch: running max bit patterns of |p'|, |m'|, |v'|             */
+    float saved[3];          /* scratch: dequantization factors in force before this step         */
+    uint32_t reserved[2];
+} msamp_adamw_tensor;
+
+/* The whole FP8 branch of LBAdamW.adamw_fn (adamw.py:148-199) for n_tensors tensors in three
+ * launches: (1) dequantize w/g/m/v, AdamW (or Adam-mode L2) update, fresh amax of p', m', v';
+ * (2) pow-2 scales (weight: fallback = old scale; moments: fallback 1.0; all moment scales 1 when
+ * tensor_scale == 0) and meta rewrite; (3) recompute and requantize w (weight_dtype), m (E4M3),
+ * v (scaled fp16), walking the blocks back to front so the re-read meets the cache.
+ * `tensors`: DEVICE array of descriptors; `block_map`: DEVICE array of n_blocks
+ * {tensor index, chunk index} int32 pairs (chunks of MSAMP_ADAMW_CHUNK elements) built by the
+ * caller once per parameter set.  weight_dtype: E4M3/E5M2/F16; grad_dtype: E4M3/E5M2.
+ * Hyper-parameters arrive as doubles and are narrowed the way the reference narrows them
+ * (adamw.cu:99-107, adamw.py:160-164). */
+#define MSAMP_ADAMW_CHUNK 16384
+int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int32_t* block_map, int n_blocks,
+                          int weight_dtype, int grad_dtype, double lr, double beta1, double beta2, double eps,
+                          double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
+                          int tensor_scale, msamp_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSAMP_HIP_H_ */

@@ -1,0 +1,643 @@
+// Cast group: amax, pow-2 scale rule, FP8 quantize / dequantize, cast+transpose, byte transpose,
+// amax-window update.  All bandwidth-bound: 16-byte lane-contiguous loads, packed FP8 converters,
+// wavefront shuffle reductions, one atomic per block.
+#include "common.cuh"
+
+namespace msamp {
+
+constexpr int kCastThreads = 256;
+constexpr int kCastUnroll = 4;
+
+template <typename IT>
+struct In16;    // one 16-byte load = EPT elements as float
+template <>
+struct In16<float> {
+    static constexpr int EPT = 4;
+    static __device__ __forceinline__ void load(const float* p, float* v) {
+        float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+    }
+};
+template <>
+struct In16<bf16_t> {
+    static constexpr int EPT = 8;
+    static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
+        uint4 t = *reinterpret_cast<const uint4*>(p);
+        v[0] = __uint_as_float(t.x << 16), v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16), v[3] = __uint_as_float(t.y & 0xffff0000u);
+        v[4] = __uint_as_float(t.z << 16), v[5] = __uint_as_float(t.z & 0xffff0000u);
+        v[6] = __uint_as_float(t.w << 16), v[7] = __uint_as_float(t.w & 0xffff0000u);
+    }
+};
+template <>
+struct In16<f16_t> {
+    static constexpr int EPT = 8;
+    static __device__ __forceinline__ void load(const f16_t* p, float* v) {
+        uint4 t = *reinterpret_cast<const uint4*>(p);
+        v[0] = f16_bits_to_float(t.x & 0xffffu), v[1] = f16_bits_to_float(t.x >> 16);
+        v[2] = f16_bits_to_float(t.y & 0xffffu), v[3] = f16_bits_to_float(t.y >> 16);
+        v[4] = f16_bits_to_float(t.z & 0xffffu), v[5] = f16_bits_to_float(t.z >> 16);
+        v[6] = f16_bits_to_float(t.w & 0xffffu), v[7] = f16_bits_to_float(t.w >> 16);
+    }
+};
+
+// issue an atomic max on a non-negative float cell only when it can change the cell
+__device__ __forceinline__ void amax_publish(float* amax, float v) {
+    int vb = __float_as_int(v);
+    int cur = __hip_atomic_load(reinterpret_cast<int*>(amax), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (vb > cur) atomicMax(reinterpret_cast<int*>(amax), vb);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Quantize with a given scale.  WITH_AMAX: also fold max|x| (NaN skipped) into *amax.
+// reverse != 0 walks the tiles back to front (second pass of the in-time cast).
+template <typename IT, int FMT, bool WITH_AMAX>
+__global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __restrict__ x,
+                                                                    uint8_t* __restrict__ out, size_t n,
+                                                                    const float* __restrict__ scale_p, float* amax,
+                                                                    float* scale_inv, int vec_ok, int reverse) {
+    constexpr int EPT = In16<IT>::EPT;
+    constexpr size_t TILE = static_cast<size_t>(kCastThreads) * EPT * kCastUnroll;
+    __shared__ uint32_t red[kCastThreads / kWave];
+    const float s = *scale_p;
+    const int tid = threadIdx.x;
+    float mx = 0.0f;
+    const size_t ntiles = (n + TILE - 1) / TILE;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t tile = reverse ? (ntiles - 1 - t) : t;
+        const size_t base = tile * TILE;
+        if (vec_ok && base + TILE <= n) {
+            float v[kCastUnroll][EPT];
+#pragma unroll
+            for (int u = 0; u < kCastUnroll; ++u)
+                In16<IT>::load(x + base + (static_cast<size_t>(u) * kCastThreads + tid) * EPT, v[u]);
+#pragma unroll
+            for (int u = 0; u < kCastUnroll; ++u) {
+                uint32_t w[EPT / 4];
+#pragma unroll
+                for (int j = 0; j < EPT / 4; ++j) {
+                    const float a = v[u][4 * j], b = v[u][4 * j + 1], c = v[u][4 * j + 2], d = v[u][4 * j + 3];
+                    if (WITH_AMAX) mx = fmaxf(fmaxf(mx, fabsf(a)), fmaxf(fmaxf(fabsf(b), fabsf(c)), fabsf(d)));
+                    w[j] = quant4<FMT>(a * s, b * s, c * s, d * s);
+                }
+                uint8_t* o = out + base + (static_cast<size_t>(u) * kCastThreads + tid) * EPT;
+                if constexpr (EPT == 4) {
+                    *reinterpret_cast<uint32_t*>(o) = w[0];
+                } else {
+                    *reinterpret_cast<uint2*>(o) = make_uint2(w[0], w[1]);
+                }
+            }
+        } else {
+            const size_t end = (base + TILE < n) ? base + TILE : n;
+            for (size_t i = base + tid; i < end; i += kCastThreads) {
+                const float a = Elem<IT>::load(x + i);
+                if (WITH_AMAX) mx = fmaxf(mx, fabsf(a));
+                out[i] = static_cast<uint8_t>(quant1<FMT>(a * s));
+            }
+        }
+    }
+    if (WITH_AMAX) {
+        uint32_t m = block_max_u32(__float_as_uint(mx), red);
+        if (tid == 0) amax_publish(amax, __uint_as_float(m));
+    }
+    if (scale_inv != nullptr && blockIdx.x == 0 && tid == 0) *scale_inv = 1.0f / s;
+}
+
+// ---------------------------------------------------------------------------------------------
+// NaN-propagating max|x| with the scale rule folded into the last block to finish.
+// ws[0]: arrival counter, ws[1]: running max of |x| bit patterns; both zero on entry and exit.
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
+template <typename IT>
+__global__ __launch_bounds__(kCastThreads) void amax_kernel(const IT* __restrict__ x, size_t n, uint32_t* ws,
+                                                             float* amax, float* scale, float* scale_inv,
+                                                             float fp_max, int margin, int flags, int update_scale,
+                                                             int vec_ok) {
+    constexpr int EPT = 16 / sizeof(IT);
+    constexpr int UNROLL = 8;
+    constexpr size_t TILE = static_cast<size_t>(kCastThreads) * EPT * UNROLL;
+    __shared__ uint32_t red[kCastThreads / kWave];
+    const int tid = threadIdx.x;
+    // running max of the |x| bit pattern; for 2-byte inputs kept in the high half-word
+    uint32_t m = 0;
+    const size_t ntiles = (n + TILE - 1) / TILE;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * TILE;
+        if (vec_ok && base + TILE <= n) {
+            uint4 v[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u)
+                v[u] = *reinterpret_cast<const uint4*>(x + base + (static_cast<size_t>(u) * kCastThreads + tid) * EPT);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if constexpr (sizeof(IT) == 4) {
+                        m = umax(m, w[j] & 0x7fffffffu);
+                    } else {
+                        m = umax(m, umax((w[j] << 16) & 0x7fff0000u, w[j] & 0x7fff0000u));
+                    }
+                }
+            }
+        } else {
+            const size_t end = (base + TILE < n) ? base + TILE : n;
+            for (size_t i = base + tid; i < end; i += kCastThreads) {
+                if constexpr (sizeof(IT) == 4) {
+                    m = umax(m, reinterpret_cast<const uint32_t*>(x)[i] & 0x7fffffffu);
+                } else {
+                    m = umax(m, (static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(x)[i]) << 16) & 0x7fff0000u);
+                }
+            }
+        }
+    }
+    m = block_max_u32(m, red);
+    if (tid == 0) {
+        // to a float32 bit pattern (order-preserving for bf16 already; fp16 needs widening)
+        if constexpr (sizeof(IT) == 2 && !__is_same(IT, bf16_t)) {
+            m = __float_as_uint(f16_bits_to_float(m >> 16));
+        }
+        if (m != 0u) atomicMax(&ws[1], m);
+        __threadfence();
+        const uint32_t ticket = atomicAdd(&ws[0], 1u);
+        if (ticket == gridDim.x - 1) {
+            __threadfence();
+            const uint32_t bits = atomicExch(&ws[1], 0u);
+            atomicExch(&ws[0], 0u);
+            float a = __uint_as_float(bits);
+            if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(a < __uint_as_float(0x7f800000u))) a = __uint_as_float(0x7f800000u);
+            *amax = a;
+            if (update_scale) {
+                const float s = scale_rule(a, *scale, fp_max, margin);
+                *scale = s;
+                *scale_inv = 1.0f / s;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int FMT, typename OT>
+__global__ __launch_bounds__(kCastThreads) void cast_from_fp8_kernel(const uint8_t* __restrict__ q,
+                                                                      OT* __restrict__ out, size_t n,
+                                                                      const float* __restrict__ scale_inv_p,
+                                                                      int vec_ok) {
+    constexpr int EPT = 16 / sizeof(OT);    // codes per thread per step: 4 (fp32 out) or 8
+    constexpr int UNROLL = 4;
+    constexpr size_t TILE = static_cast<size_t>(kCastThreads) * EPT * UNROLL;
+    const float si = *scale_inv_p;
+    const int tid = threadIdx.x;
+    const size_t ntiles = (n + TILE - 1) / TILE;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * TILE;
+        if (vec_ok && base + TILE <= n) {
+            uint32_t w[UNROLL][EPT / 4];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint8_t* p = q + base + (static_cast<size_t>(u) * kCastThreads + tid) * EPT;
+                if constexpr (EPT == 4) {
+                    w[u][0] = *reinterpret_cast<const uint32_t*>(p);
+                } else {
+                    uint2 t2 = *reinterpret_cast<const uint2*>(p);
+                    w[u][0] = t2.x, w[u][1] = t2.y;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                float f[EPT];
+#pragma unroll
+                for (int j = 0; j < EPT / 4; ++j) {
+                    dequant4<FMT>(w[u][j], f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]);
+                }
+#pragma unroll
+                for (int j = 0; j < EPT; ++j) f[j] *= si;
+                OT* o = out + base + (static_cast<size_t>(u) * kCastThreads + tid) * EPT;
+                if constexpr (sizeof(OT) == 4) {
+                    *reinterpret_cast<float4*>(o) = make_float4(f[0], f[1], f[2], f[3]);
+                } else {
+                    uint32_t pk[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if constexpr (__is_same(OT, bf16_t)) {
+                            pk[j] = float_to_bf16_bits(f[2 * j]) | (float_to_bf16_bits(f[2 * j + 1]) << 16);
+                        } else {
+                            pk[j] = float_to_f16_bits(f[2 * j]) | (float_to_f16_bits(f[2 * j + 1]) << 16);
+                        }
+                    }
+                    *reinterpret_cast<uint4*>(o) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                }
+            }
+        } else {
+            const size_t end = (base + TILE < n) ? base + TILE : n;
+            for (size_t i = base + tid; i < end; i += kCastThreads) {
+                Elem<OT>::store(out + i, dequant1<FMT>(q[i]) * si);
+            }
+        }
+    }
+}
+
+// out = OT(float(x) * scale), IEEE overflow
+template <typename IT, typename OT>
+__global__ __launch_bounds__(kCastThreads) void scale_cast_kernel(const IT* __restrict__ x, OT* __restrict__ out,
+                                                                   size_t n, const float* __restrict__ scale_p) {
+    const float s = *scale_p;
+    const size_t stride = static_cast<size_t>(gridDim.x) * kCastThreads;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kCastThreads + threadIdx.x; i < n; i += stride) {
+        Elem<OT>::store(out + i, Elem<IT>::load(x + i) * s);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// 64x64 tile: quantize (or pass bytes through), write the row-major copy, stage the packed words
+// in LDS, transpose 4x4 byte blocks in registers and write the transposed copy.
+template <typename IT>
+struct TileLoad {    // 4 consecutive elements of a row as floats
+    static __device__ __forceinline__ void load(const IT* p, int vec, int valid, float* v) {
+        if (vec && valid == 4) {
+            if constexpr (sizeof(IT) == 4) {
+                float4 t = *reinterpret_cast<const float4*>(p);
+                v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+            } else {
+                uint2 t = *reinterpret_cast<const uint2*>(p);
+                if constexpr (__is_same(IT, bf16_t)) {
+                    v[0] = __uint_as_float(t.x << 16), v[1] = __uint_as_float(t.x & 0xffff0000u);
+                    v[2] = __uint_as_float(t.y << 16), v[3] = __uint_as_float(t.y & 0xffff0000u);
+                } else {
+                    v[0] = f16_bits_to_float(t.x & 0xffffu), v[1] = f16_bits_to_float(t.x >> 16);
+                    v[2] = f16_bits_to_float(t.y & 0xffffu), v[3] = f16_bits_to_float(t.y >> 16);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = j < valid ? Elem<IT>::load(p + j) : 0.0f;
+        }
+    }
+};
+
+template <typename IT, int FMT, bool CAST, bool WITH_AMAX>
+__global__ __launch_bounds__(kCastThreads) void cast_transpose_kernel(const IT* __restrict__ x,
+                                                                       uint8_t* __restrict__ out,
+                                                                       uint8_t* __restrict__ out_t, int R, int C,
+                                                                       const float* __restrict__ scale_p,
+                                                                       float* amax, float* scale_inv, int vec_in,
+                                                                       int vec_out, int vec_t) {
+    __shared__ uint32_t tile[64][17];
+    __shared__ uint32_t red[kCastThreads / kWave];
+    const int tid = threadIdx.x;
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    float s = 1.0f;
+    if constexpr (CAST) s = *scale_p;
+    float mx = 0.0f;
+    const int wc = tid & 15;    // word column: columns c0 + 4*wc .. +3
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int lr = (tid >> 4) + 16 * i;
+        const int r = r0 + lr, c = c0 + 4 * wc;
+        uint32_t w = 0;
+        int valid = C - c;
+        valid = valid > 4 ? 4 : valid;
+        if (r < R && valid > 0) {
+            const size_t off = static_cast<size_t>(r) * C + c;
+            if constexpr (CAST) {
+                float v[4];
+                TileLoad<IT>::load(x + off, vec_in, valid, v);
+                if (WITH_AMAX) mx = fmaxf(fmaxf(mx, fabsf(v[0])), fmaxf(fmaxf(fabsf(v[1]), fabsf(v[2])), fabsf(v[3])));
+                w = quant4<FMT>(v[0] * s, v[1] * s, v[2] * s, v[3] * s);
+                if (out != nullptr) {
+                    if (vec_out && valid == 4) {
+                        *reinterpret_cast<uint32_t*>(out + off) = w;
+                    } else {
+                        for (int j = 0; j < valid; ++j) out[off + j] = static_cast<uint8_t>(w >> (8 * j));
+                    }
+                }
+            } else {
+                const uint8_t* p = reinterpret_cast<const uint8_t*>(x) + off;
+                if (vec_in && valid == 4) {
+                    w = *reinterpret_cast<const uint32_t*>(p);
+                } else {
+                    for (int j = 0; j < valid; ++j) w |= static_cast<uint32_t>(p[j]) << (8 * j);
+                }
+            }
+        }
+        tile[lr][wc] = w;
+    }
+    __syncthreads();
+    {
+        const int tr = tid & 15, tc = tid >> 4;    // rows 4*tr..+3 of the tile, word column tc
+        const uint32_t w0 = tile[4 * tr][tc], w1 = tile[4 * tr + 1][tc], w2 = tile[4 * tr + 2][tc],
+                       w3 = tile[4 * tr + 3][tc];
+        const int row = r0 + 4 * tr;
+        int rvalid = R - row;
+        rvalid = rvalid > 4 ? 4 : rvalid;
+        if (rvalid > 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int col = c0 + 4 * tc + i;
+                if (col < C) {
+                    const int sh = 8 * i;
+                    const uint32_t t = ((w0 >> sh) & 0xffu) | (((w1 >> sh) & 0xffu) << 8) |
+                                       (((w2 >> sh) & 0xffu) << 16) | (((w3 >> sh) & 0xffu) << 24);
+                    const size_t off = static_cast<size_t>(col) * R + row;
+                    if (vec_t && rvalid == 4) {
+                        *reinterpret_cast<uint32_t*>(out_t + off) = t;
+                    } else {
+                        for (int j = 0; j < rvalid; ++j) out_t[off + j] = static_cast<uint8_t>(t >> (8 * j));
+                    }
+                }
+            }
+        }
+    }
+    if constexpr (CAST && WITH_AMAX) {
+        uint32_t m = block_max_u32(__float_as_uint(mx), red);
+        if (tid == 0) amax_publish(amax, __uint_as_float(m));
+    }
+    if constexpr (CAST) {
+        if (scale_inv != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *scale_inv = 1.0f / s;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+__global__ void scaling_factor_kernel(const float* amax, const float* scale_in, int scale_in_n, float* scale_out, int n,
+                                      float fp_max, int margin) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) scale_out[i] = scale_rule(amax[i], scale_in[scale_in_n == 1 ? 0 : i], fp_max, margin);
+}
+
+__device__ __forceinline__ float nanmax(float a, float b) { return (a != a) ? a : ((b != b) ? b : fmaxf(a, b)); }
+
+__global__ void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad, int n, int window, float fp_max,
+                                    int margin) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float* row = amaxs + static_cast<size_t>(i) * window;
+    float a0 = row[0];
+    const bool is_bad = !(fabsf(a0) < __uint_as_float(0x7f800000u));
+    if (is_bad) a0 = 0.0f;
+    float mx = a0;
+    for (int j = 1; j < window; ++j) mx = nanmax(mx, row[j]);
+    const float sf = scale_rule(mx, scales[i], fp_max, margin);
+    for (int j = window - 1; j >= 2; --j) row[j] = row[j - 1];
+    if (window > 1) row[1] = a0;
+    row[0] = 0.0f;
+    scales[i] = sf;
+    if (bad != nullptr) bad[i] = is_bad ? 1 : 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+static int grid_for(size_t n, size_t tile) {
+    size_t tiles = (n + tile - 1) / tile;
+    size_t cap = static_cast<size_t>(cu_count()) * 8;
+    if (tiles < 1) tiles = 1;
+    return static_cast<int>(tiles < cap ? tiles : cap);
+}
+
+template <typename IT>
+static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, float* scale_inv, uint8_t* out,
+                       int fp8_type, int reverse, hipStream_t st) {
+    constexpr int EPT = In16<IT>::EPT;
+    const int vec_ok = aligned(x, 16) && aligned(out, EPT);
+    const int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * kCastUnroll);
+#define LAUNCH(FMT, AM) \
+    hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, AM>), dim3(grid), dim3(kCastThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, reverse)
+    if (fp8_type == MSAMP_DT_E4M3) {
+        if (amax) LAUNCH(MSAMP_DT_E4M3, true); else LAUNCH(MSAMP_DT_E4M3, false);
+    } else {
+        if (amax) LAUNCH(MSAMP_DT_E5M2, true); else LAUNCH(MSAMP_DT_E5M2, false);
+    }
+#undef LAUNCH
+    MSAMP_CHECK_LAUNCH("cast_to_fp8_kernel");
+    return MSAMP_OK;
+}
+
+template <typename IT>
+static int launch_amax(const IT* x, size_t n, uint32_t* ws, float* amax, float* scale, float* scale_inv, float fp_max,
+                       int margin, int flags, int update_scale, hipStream_t st) {
+    constexpr int EPT = 16 / sizeof(IT);
+    const int vec_ok = aligned(x, 16);
+    const int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * 8);
+    hipLaunchKernelGGL((amax_kernel<IT>), dim3(grid), dim3(kCastThreads), 0, st, x, n, ws, amax, scale, scale_inv, fp_max,
+                       margin, flags, update_scale, vec_ok);
+    MSAMP_CHECK_LAUNCH("amax_kernel");
+    return MSAMP_OK;
+}
+
+static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, float* amax, float* scale, float* scale_inv,
+                         float fp_max, int margin, int flags, int update_scale, hipStream_t st) {
+    uint32_t* w = static_cast<uint32_t*>(ws);
+    switch (dtype) {
+        case MSAMP_DT_F32:
+            return launch_amax(static_cast<const float*>(x), n, w, amax, scale, scale_inv, fp_max, margin, flags, update_scale, st);
+        case MSAMP_DT_F16:
+            return launch_amax(static_cast<const f16_t*>(x), n, w, amax, scale, scale_inv, fp_max, margin, flags, update_scale, st);
+        case MSAMP_DT_BF16:
+            return launch_amax(static_cast<const bf16_t*>(x), n, w, amax, scale, scale_inv, fp_max, margin, flags, update_scale, st);
+    }
+    set_error("unsupported input dtype %d", dtype);
+    return MSAMP_ERR_DTYPE;
+}
+
+static int dispatch_cast(const void* x, int dtype, size_t n, const float* scale, float* amax, float* scale_inv,
+                         uint8_t* out, int fp8_type, int reverse, hipStream_t st) {
+    switch (dtype) {
+        case MSAMP_DT_F32:
+            return launch_cast(static_cast<const float*>(x), n, scale, amax, scale_inv, out, fp8_type, reverse, st);
+        case MSAMP_DT_F16:
+            return launch_cast(static_cast<const f16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, reverse, st);
+        case MSAMP_DT_BF16:
+            return launch_cast(static_cast<const bf16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, reverse, st);
+    }
+    set_error("unsupported input dtype %d", dtype);
+    return MSAMP_ERR_DTYPE;
+}
+
+template <typename IT, bool CAST>
+static int launch_ct(const IT* x, int rows, int cols, const float* scale, float* amax, float* scale_inv, uint8_t* out,
+                     uint8_t* out_t, int fp8_type, hipStream_t st) {
+    const int esz = CAST ? static_cast<int>(sizeof(IT)) : 1;
+    const int vec_in = (cols % 4 == 0) && aligned(x, 4 * esz);
+    const int vec_out = (cols % 4 == 0) && (out == nullptr || aligned(out, 4));
+    const int vec_t = (rows % 4 == 0) && aligned(out_t, 4);
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    MSAMP_REQUIRE(grid.y <= 65535u, MSAMP_ERR_SHAPE, "too many rows for one launch: %d", rows);
+#define LAUNCH(FMT, AM) \
+    hipLaunchKernelGGL((cast_transpose_kernel<IT, FMT, CAST, AM>), grid, dim3(kCastThreads), 0, st, x, out, out_t, rows, cols, scale, amax, scale_inv, vec_in, vec_out, vec_t)
+    if (fp8_type == MSAMP_DT_E4M3) {
+        if (amax) LAUNCH(MSAMP_DT_E4M3, true); else LAUNCH(MSAMP_DT_E4M3, false);
+    } else {
+        if (amax) LAUNCH(MSAMP_DT_E5M2, true); else LAUNCH(MSAMP_DT_E5M2, false);
+    }
+#undef LAUNCH
+    MSAMP_CHECK_LAUNCH("cast_transpose_kernel");
+    return MSAMP_OK;
+}
+
+static int dispatch_ct(const void* x, int dtype, int rows, int cols, const float* scale, float* amax, float* scale_inv,
+                       uint8_t* out, uint8_t* out_t, int fp8_type, hipStream_t st) {
+    switch (dtype) {
+        case MSAMP_DT_F32:
+            return launch_ct<float, true>(static_cast<const float*>(x), rows, cols, scale, amax, scale_inv, out, out_t, fp8_type, st);
+        case MSAMP_DT_F16:
+            return launch_ct<f16_t, true>(static_cast<const f16_t*>(x), rows, cols, scale, amax, scale_inv, out, out_t, fp8_type, st);
+        case MSAMP_DT_BF16:
+            return launch_ct<bf16_t, true>(static_cast<const bf16_t*>(x), rows, cols, scale, amax, scale_inv, out, out_t, fp8_type, st);
+    }
+    set_error("unsupported input dtype %d", dtype);
+    return MSAMP_ERR_DTYPE;
+}
+
+template <typename IT>
+static int launch_scale_cast_out(const IT* x, size_t n, const float* scale, void* out, int out_dtype, hipStream_t st) {
+    const int grid = grid_for(n, kCastThreads * 4);
+    switch (out_dtype) {
+        case MSAMP_DT_F32:
+            hipLaunchKernelGGL((scale_cast_kernel<IT, float>), dim3(grid), dim3(kCastThreads), 0, st, x, static_cast<float*>(out), n, scale);
+            break;
+        case MSAMP_DT_F16:
+            hipLaunchKernelGGL((scale_cast_kernel<IT, f16_t>), dim3(grid), dim3(kCastThreads), 0, st, x, static_cast<f16_t*>(out), n, scale);
+            break;
+        case MSAMP_DT_BF16:
+            hipLaunchKernelGGL((scale_cast_kernel<IT, bf16_t>), dim3(grid), dim3(kCastThreads), 0, st, x, static_cast<bf16_t*>(out), n, scale);
+            break;
+        default:
+            set_error("unsupported output dtype %d", out_dtype);
+            return MSAMP_ERR_DTYPE;
+    }
+    MSAMP_CHECK_LAUNCH("scale_cast_kernel");
+    return MSAMP_OK;
+}
+
+}    // namespace msamp
+
+using namespace msamp;
+
+extern "C" {
+
+int msamp_amax(const void* x, int dtype, size_t n, float* amax, void* workspace, msamp_stream_t stream) {
+    MSAMP_REQUIRE(amax != nullptr && (x != nullptr || n == 0), MSAMP_ERR_NULL, "msamp_amax: null pointer");
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_amax: workspace required");
+    MSAMP_REQUIRE(is_hp(dtype), MSAMP_ERR_DTYPE, "msamp_amax: unsupported dtype %d", dtype);
+    return dispatch_amax(x, dtype, n, workspace, amax, nullptr, nullptr, 0.0f, 0, 0, 0, static_cast<hipStream_t>(stream));
+}
+
+int msamp_compute_scaling_factor(const float* amax, const float* scale_in, int scale_in_n, float* scale_out, int n,
+                                 float fp_max, int margin, msamp_stream_t stream) {
+    MSAMP_REQUIRE(n >= 0 && (scale_in_n == 1 || scale_in_n == n), MSAMP_ERR_SHAPE,
+                  "msamp_compute_scaling_factor: n=%d scale_in_n=%d", n, scale_in_n);
+    if (n == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(amax && scale_in && scale_out, MSAMP_ERR_NULL, "msamp_compute_scaling_factor: null pointer");
+    hipLaunchKernelGGL(scaling_factor_kernel, dim3((n + 127) / 128), dim3(128), 0, static_cast<hipStream_t>(stream), amax,
+                       scale_in, scale_in_n, scale_out, n, fp_max, margin);
+    MSAMP_CHECK_LAUNCH("scaling_factor_kernel");
+    return MSAMP_OK;
+}
+
+int msamp_cast_to_fp8(const void* x, int in_dtype, size_t n, const float* scale, float* amax, float* scale_inv,
+                      uint8_t* out, int fp8_type, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_to_fp8: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_to_fp8: in_dtype %d", in_dtype);
+    MSAMP_REQUIRE(scale != nullptr && ((x != nullptr && out != nullptr) || n == 0), MSAMP_ERR_NULL,
+                  "msamp_cast_to_fp8: null pointer");
+    return dispatch_cast(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, 0, static_cast<hipStream_t>(stream));
+}
+
+int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
+                             uint8_t* out, int fp8_type, int margin, int flags, void* workspace,
+                             msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_to_fp8_intime: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_to_fp8_intime: in_dtype %d", in_dtype);
+    MSAMP_REQUIRE(scale && amax && scale_inv && ((x && out) || n == 0), MSAMP_ERR_NULL,
+                  "msamp_cast_to_fp8_intime: null pointer");
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_to_fp8_intime: workspace required");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc = dispatch_amax(x, in_dtype, n, workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st);
+    if (rc != MSAMP_OK) return rc;
+    return dispatch_cast(x, in_dtype, n, scale, nullptr, nullptr, out, fp8_type, 1, st);
+}
+
+int msamp_cast_from_fp8(const uint8_t* q, int fp8_type, size_t n, const float* scale_inv, void* out, int out_dtype,
+                        msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_from_fp8: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(out_dtype), MSAMP_ERR_DTYPE, "msamp_cast_from_fp8: out_dtype %d", out_dtype);
+    MSAMP_REQUIRE(scale_inv && ((q && out) || n == 0), MSAMP_ERR_NULL, "msamp_cast_from_fp8: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int ept = 16 / hp_size(out_dtype);
+    const int vec_ok = aligned(out, 16) && aligned(q, ept);
+    const int grid = grid_for(n, static_cast<size_t>(kCastThreads) * ept * 4);
+#define LAUNCH(FMT, OT) \
+    hipLaunchKernelGGL((cast_from_fp8_kernel<FMT, OT>), dim3(grid), dim3(kCastThreads), 0, st, q, static_cast<OT*>(out), n, scale_inv, vec_ok)
+    if (fp8_type == MSAMP_DT_E4M3) {
+        if (out_dtype == MSAMP_DT_F32) LAUNCH(MSAMP_DT_E4M3, float);
+        else if (out_dtype == MSAMP_DT_F16) LAUNCH(MSAMP_DT_E4M3, f16_t);
+        else LAUNCH(MSAMP_DT_E4M3, bf16_t);
+    } else {
+        if (out_dtype == MSAMP_DT_F32) LAUNCH(MSAMP_DT_E5M2, float);
+        else if (out_dtype == MSAMP_DT_F16) LAUNCH(MSAMP_DT_E5M2, f16_t);
+        else LAUNCH(MSAMP_DT_E5M2, bf16_t);
+    }
+#undef LAUNCH
+    MSAMP_CHECK_LAUNCH("cast_from_fp8_kernel");
+    return MSAMP_OK;
+}
+
+int msamp_cast_transpose(const void* x, int in_dtype, int rows, int cols, const float* scale, float* amax,
+                         float* scale_inv, uint8_t* out, uint8_t* out_t, int fp8_type, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_transpose: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_transpose: in_dtype %d", in_dtype);
+    MSAMP_REQUIRE(rows >= 0 && cols >= 0, MSAMP_ERR_SHAPE, "msamp_cast_transpose: shape %d x %d", rows, cols);
+    if (rows == 0 || cols == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(x && scale && out_t, MSAMP_ERR_NULL, "msamp_cast_transpose: null pointer");
+    return dispatch_ct(x, in_dtype, rows, cols, scale, amax, scale_inv, out, out_t, fp8_type, static_cast<hipStream_t>(stream));
+}
+
+int msamp_cast_transpose_intime(const void* x, int in_dtype, int rows, int cols, float* scale, float* amax,
+                                float* scale_inv, uint8_t* out, uint8_t* out_t, int fp8_type, int margin, int flags,
+                                void* workspace, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_transpose_intime: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_transpose_intime: in_dtype %d", in_dtype);
+    MSAMP_REQUIRE(rows >= 0 && cols >= 0, MSAMP_ERR_SHAPE, "msamp_cast_transpose_intime: shape %d x %d", rows, cols);
+    MSAMP_REQUIRE(scale && amax && scale_inv, MSAMP_ERR_NULL, "msamp_cast_transpose_intime: null meta pointer");
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_transpose_intime: workspace required");
+    MSAMP_REQUIRE((x && out_t) || rows == 0 || cols == 0, MSAMP_ERR_NULL, "msamp_cast_transpose_intime: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t n = static_cast<size_t>(rows) * cols;
+    int rc = dispatch_amax(x, in_dtype, n, workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st);
+    if (rc != MSAMP_OK || n == 0) return rc;
+    return dispatch_ct(x, in_dtype, rows, cols, scale, nullptr, nullptr, out, out_t, fp8_type, st);
+}
+
+int msamp_fp8_transpose(const uint8_t* q, int rows, int cols, uint8_t* out, msamp_stream_t stream) {
+    MSAMP_REQUIRE(rows >= 0 && cols >= 0, MSAMP_ERR_SHAPE, "msamp_fp8_transpose: shape %d x %d", rows, cols);
+    if (rows == 0 || cols == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(q && out, MSAMP_ERR_NULL, "msamp_fp8_transpose: null pointer");
+    return launch_ct<uint8_t, false>(q, rows, cols, nullptr, nullptr, nullptr, nullptr, out, MSAMP_DT_E4M3,
+                                     static_cast<hipStream_t>(stream));
+}
+
+int msamp_scale_cast(const void* x, int in_dtype, size_t n, const float* scale, void* out, int out_dtype,
+                     msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_hp(in_dtype) && is_hp(out_dtype), MSAMP_ERR_DTYPE, "msamp_scale_cast: dtypes %d -> %d", in_dtype, out_dtype);
+    MSAMP_REQUIRE(scale && ((x && out) || n == 0), MSAMP_ERR_NULL, "msamp_scale_cast: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (n == 0) return MSAMP_OK;
+    switch (in_dtype) {
+        case MSAMP_DT_F32:
+            return launch_scale_cast_out(static_cast<const float*>(x), n, scale, out, out_dtype, st);
+        case MSAMP_DT_F16:
+            return launch_scale_cast_out(static_cast<const f16_t*>(x), n, scale, out, out_dtype, st);
+        default:
+            return launch_scale_cast_out(static_cast<const bf16_t*>(x), n, scale, out, out_dtype, st);
+    }
+}
+
+int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int n, int window, float fp_max, int margin,
+                       msamp_stream_t stream) {
+    MSAMP_REQUIRE(n >= 0 && window >= 1, MSAMP_ERR_SHAPE, "msamp_scale_update: n=%d window=%d", n, window);
+    if (n == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(scales && amaxs, MSAMP_ERR_NULL, "msamp_scale_update: null pointer");
+    hipLaunchKernelGGL(scale_update_kernel, dim3((n + 63) / 64), dim3(64), 0, static_cast<hipStream_t>(stream), scales,
+                       amaxs, bad, n, window, fp_max, margin);
+    MSAMP_CHECK_LAUNCH("scale_update_kernel");
+    return MSAMP_OK;
+}
+
+}    // extern "C"

@@ -1,0 +1,211 @@
+// Shared device/host helpers for the gfx950 FP8 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <math.h>
+
+#include "../../include/msamp_hip.h"
+
+namespace msamp {
+
+constexpr int kWave = 64;
+
+// ---- error reporting -------------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what);
+
+#define MSAMP_REQUIRE(cond, code, ...)  \
+    do {                                \
+        if (!(cond)) {                  \
+            msamp::set_error(__VA_ARGS__); \
+            return (code);              \
+        }                               \
+    } while (0)
+
+#define MSAMP_CHECK_LAUNCH(what)                         \
+    do {                                                 \
+        hipError_t e__ = hipGetLastError();              \
+        if (e__ != hipSuccess) return msamp::hip_fail(e__, what); \
+    } while (0)
+
+inline bool is_fp8(int dt) { return dt == MSAMP_DT_E4M3 || dt == MSAMP_DT_E5M2; }
+inline bool is_hp(int dt) { return dt == MSAMP_DT_F32 || dt == MSAMP_DT_F16 || dt == MSAMP_DT_BF16; }
+inline float fp8_max(int dt) { return dt == MSAMP_DT_E4M3 ? 448.0f : 57344.0f; }
+inline int hp_size(int dt) { return dt == MSAMP_DT_F32 ? 4 : 2; }
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---- element types ---------------------------------------------------------------------------
+struct bf16_t {
+    uint16_t bits;
+};
+struct f16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ float f16_bits_to_float(uint32_t b) {
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(b)));
+}
+// round-to-nearest-even float -> bf16 bits, NaN kept quiet (same rule torch uses)
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ uint32_t float_to_f16_bits(float f) {
+    return static_cast<uint32_t>(__half_as_ushort(__float2half_rn(f)));
+}
+
+template <typename T>
+struct Elem;    // load/store of one element as float
+template <>
+struct Elem<float> {
+    static __device__ __forceinline__ float load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <>
+struct Elem<bf16_t> {
+    static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_bits_to_float(p->bits); }
+    static __device__ __forceinline__ void store(bf16_t* p, float v) {
+        p->bits = static_cast<uint16_t>(float_to_bf16_bits(v));
+    }
+};
+template <>
+struct Elem<f16_t> {
+    static __device__ __forceinline__ float load(const f16_t* p) { return f16_bits_to_float(p->bits); }
+    static __device__ __forceinline__ void store(f16_t* p, float v) {
+        p->bits = static_cast<uint16_t>(float_to_f16_bits(v));
+    }
+};
+
+// ---- FP8 conversion --------------------------------------------------------------------------
+// FMT: MSAMP_DT_E4M3 or MSAMP_DT_E5M2.  Saturating round-to-nearest-even through the gfx950
+// OCP converters; the clamp makes saturation independent of the wave's overflow mode and
+// NaN is patched to sign|0x7F afterwards (the clamp would otherwise turn it into -max).
+template <int FMT>
+__device__ __forceinline__ float sat(float v) {
+    constexpr float mx = (FMT == MSAMP_DT_E4M3) ? 448.0f : 57344.0f;
+    return __builtin_amdgcn_fmed3f(v, -mx, mx);
+}
+
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt_pk(float a, float b, uint32_t old, bool hi) {
+    if constexpr (FMT == MSAMP_DT_E4M3) {
+        return hi ? __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, false);
+    } else {
+        return hi ? __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, true) : __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, false);
+    }
+}
+
+__device__ __forceinline__ uint32_t nan_byte(float v) { return 0x7fu | ((__float_as_uint(v) >> 24) & 0x80u); }
+
+// four floats (already multiplied by the scale) -> four packed FP8 bytes, byte i = element i
+template <int FMT>
+__device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
+    uint32_t w = 0;
+    w = cvt_pk<FMT>(sat<FMT>(a), sat<FMT>(b), w, false);
+    w = cvt_pk<FMT>(sat<FMT>(c), sat<FMT>(d), w, true);
+    if (__builtin_expect((a != a) | (b != b) | (c != c) | (d != d), 0)) {
+        if (a != a) w = (w & 0xffffff00u) | nan_byte(a);
+        if (b != b) w = (w & 0xffff00ffu) | (nan_byte(b) << 8);
+        if (c != c) w = (w & 0xff00ffffu) | (nan_byte(c) << 16);
+        if (d != d) w = (w & 0x00ffffffu) | (nan_byte(d) << 24);
+    }
+    return w;
+}
+
+template <int FMT>
+__device__ __forceinline__ uint32_t quant1(float a) {
+    uint32_t w = cvt_pk<FMT>(sat<FMT>(a), 0.0f, 0u, false) & 0xffu;
+    if (a != a) w = nan_byte(a);
+    return w;
+}
+
+// packed FP8 word -> floats (exact)
+template <int FMT>
+__device__ __forceinline__ void dequant4(uint32_t w, float& a, float& b, float& c, float& d) {
+    typedef float v2f __attribute__((ext_vector_type(2)));
+    v2f lo, hi;
+    if constexpr (FMT == MSAMP_DT_E4M3) {
+        lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+        hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+    } else {
+        lo = __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+        hi = __builtin_amdgcn_cvt_pk_f32_bf8(w, true);
+    }
+    a = lo.x;
+    b = lo.y;
+    c = hi.x;
+    d = hi.y;
+}
+
+template <int FMT>
+__device__ __forceinline__ float dequant1(uint32_t byte) {
+    float a, b, c, d;
+    dequant4<FMT>(byte & 0xffu, a, b, c, d);
+    return a;
+}
+
+// ---- reductions ------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        uint32_t o = static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), off, 64));
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+// max over the block of a non-negative-float bit pattern (or any u32); result valid in thread 0.
+// `smem` must hold blockDim.x/64 words.
+__device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
+    v = wave_max_u32(v);
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();
+    if (lane == 0) smem[wid] = v;
+    __syncthreads();
+    if (wid == 0) {
+        v = lane < nw ? smem[lane] : 0u;
+        v = wave_max_u32(v);
+    }
+    return v;
+}
+
+// The pow-2 scale rule, evaluated the way float32 torch evaluates it: the quotient is an IEEE
+// float division, log2 is the correctly rounded float log2 (double log2 narrowed once), 2^|e|
+// overflows to +Inf from |e| = 128.
+__device__ __forceinline__ float scale_rule(float amax, float fallback, float fp_max, int margin) {
+    float q = fp_max / amax;
+    float e = floorf(static_cast<float>(log2(static_cast<double>(q)))) - static_cast<float>(margin);
+    float ae = fabsf(e);
+    float sf;
+    if (ae != ae) {
+        sf = ae;    // NaN
+    } else if (ae >= 128.0f) {
+        sf = __uint_as_float(0x7f800000u);
+    } else {
+        sf = __uint_as_float(static_cast<uint32_t>(static_cast<int>(ae) + 127) << 23);
+    }
+    if (!(amax > 0.0f)) sf = fallback;
+    if (!(fabsf(amax) < __uint_as_float(0x7f800000u))) sf = fallback;    // not finite (NaN or Inf)
+    if (e < 0.0f) sf = 1.0f / sf;
+    return sf;
+}
+
+inline int cu_count() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t p;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&p, dev) == hipSuccess)
+            n = p.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
+}
+
+}    // namespace msamp

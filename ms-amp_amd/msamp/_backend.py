@@ -1,0 +1,292 @@
+"""ctypes binding of libmsamp_hip.so: the only door from the Python host layer to the HIP kernels.
+
+Plays the role the reference gives to TransformerEngineWrapper and the msamp_adamw extension
+(msamp/common/utils/transformer_engine_wrapper.py:63-176, msamp/optim/adamw.cu:157-162).
+There is no CPU or eager fallback: if the library cannot be loaded, or an operand is not on
+the GPU, the call raises.
+"""
+
+import ctypes
+import os
+
+import torch
+
+_LIB_NAME = 'libmsamp_hip.so'
+_LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), 'lib', _LIB_NAME)
+
+DT_F32, DT_F16, DT_BF16, DT_E4M3, DT_E5M2 = 2, 3, 4, 5, 6
+FLAG_NAN_TO_INF = 1
+WORKSPACE_BYTES = 256
+ADAMW_CHUNK = 16384
+
+_TORCH_TO_DT = {torch.float32: DT_F32, torch.float16: DT_F16, torch.bfloat16: DT_BF16}
+
+_lib = None
+_workspaces = {}
+
+_vp, _i, _f, _d, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_double, ctypes.c_size_t
+
+_SIGNATURES = {
+    'msamp_hip_version': ([], _i),
+    'msamp_last_error': ([], ctypes.c_char_p),
+    'msamp_amax': ([_vp, _i, _sz, _vp, _vp, _vp], _i),
+    'msamp_compute_scaling_factor': ([_vp, _vp, _i, _vp, _i, _f, _i, _vp], _i),
+    'msamp_cast_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp], _i),
+    'msamp_cast_to_fp8_intime': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
+    'msamp_cast_from_fp8': ([_vp, _i, _sz, _vp, _vp, _i, _vp], _i),
+    'msamp_cast_transpose': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp], _i),
+    'msamp_cast_transpose_intime': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
+    'msamp_fp8_transpose': ([_vp, _i, _i, _vp, _vp], _i),
+    'msamp_scale_cast': ([_vp, _i, _sz, _vp, _vp, _i, _vp], _i),
+    'msamp_scale_update': ([_vp, _vp, _vp, _i, _i, _f, _i, _vp], _i),
+    'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
+    'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
+    'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def library_path():
+    """Path the library is loaded from (env MSAMP_HIP_LIB overrides the in-tree build)."""
+    return os.environ.get('MSAMP_HIP_LIB', _LIB_PATH)
+
+
+def load():
+    """Load the shared library once and declare the argument types of every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f'{_LIB_NAME} not found at {path}: build it with `make -C ms-amp_amd/csrc` '
+            '(hipcc, --offload-arch=gfx950). There is no fallback implementation.'
+        )
+    lib = ctypes.CDLL(path)
+    for name, (argtypes, restype) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = restype
+    _lib = lib
+    return lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        msg = load().msamp_last_error().decode(errors='replace')
+        raise RuntimeError(f'{what} failed with code {rc}: {msg}')
+
+
+def _gpu(t, what):
+    if not t.is_cuda:
+        raise ValueError(f'{what} is not in GPU memory; the FP8 kernels only run on the HIP device.')
+    return t
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dt(t):
+    try:
+        return _TORCH_TO_DT[t.dtype]
+    except KeyError:
+        raise TypeError(f'unsupported tensor dtype {t.dtype}') from None
+
+
+def workspace(device):
+    """Per-device zero-initialised scratch words shared by the two-pass kernels (stream ordered)."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+# ---- scaling ------------------------------------------------------------------------------------
+def amax(x, amax_cell):
+    """amax_cell[0] = max|x| (NaN propagates)."""
+    lib = load()
+    _gpu(x, 'input')
+    _check(lib.msamp_amax(_ptr(x), _dt(x), x.numel(), _ptr(amax_cell), _ptr(workspace(x.device)), _stream()), 'msamp_amax')
+
+
+def compute_scaling_factor(amax_t, scale_t, fp_max, margin):
+    """Element-wise pow-2 scale rule on float32 GPU tensors; returns a new tensor shaped like amax."""
+    lib = load()
+    _gpu(amax_t, 'amax')
+    a = amax_t.to(torch.float32).contiguous()
+    s = scale_t.to(device=a.device, dtype=torch.float32).contiguous()
+    if s.numel() not in (1, a.numel()):
+        raise ValueError('scale must have one element or as many as amax')
+    out = torch.empty_like(a)
+    _check(
+        lib.msamp_compute_scaling_factor(_ptr(a), _ptr(s), s.numel(), _ptr(out), a.numel(), fp_max, margin, _stream()),
+        'msamp_compute_scaling_factor'
+    )
+    return out
+
+
+def scale_update(scales, amaxs, fp_max, margin):
+    """In-place window update of flattened metas; returns the uint8 mask of non-finite current amaxs."""
+    lib = load()
+    _gpu(scales, 'scales')
+    n, window = amaxs.shape
+    bad = torch.empty(n, dtype=torch.uint8, device=scales.device)
+    _check(lib.msamp_scale_update(_ptr(scales), _ptr(amaxs), _ptr(bad), n, window, fp_max, margin, _stream()), 'msamp_scale_update')
+    return bad
+
+
+# ---- casts --------------------------------------------------------------------------------------
+def cast_to_fp8(x, scale, amax_cell, scale_inv, fp8_dt):
+    lib = load()
+    _gpu(x, 'input')
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _check(
+        lib.msamp_cast_to_fp8(_ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, _stream()),
+        'msamp_cast_to_fp8'
+    )
+    return out
+
+
+def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_inf=False):
+    lib = load()
+    _gpu(x, 'input')
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _check(
+        lib.msamp_cast_to_fp8_intime(
+            _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
+            FLAG_NAN_TO_INF if nan_to_inf else 0, _ptr(workspace(x.device)), _stream()
+        ), 'msamp_cast_to_fp8_intime'
+    )
+    return out
+
+
+def cast_from_fp8(q, scale_inv, fp8_dt, out_dtype):
+    lib = load()
+    _gpu(q, 'input')
+    out = torch.empty(q.shape, dtype=out_dtype, device=q.device)
+    _check(
+        lib.msamp_cast_from_fp8(_ptr(q), fp8_dt, q.numel(), _ptr(scale_inv), _ptr(out), _TORCH_TO_DT[out_dtype], _stream()),
+        'msamp_cast_from_fp8'
+    )
+    return out
+
+
+def cast_transpose(x, scale, amax_cell, scale_inv, fp8_dt, in_time=False, margin=0, nan_to_inf=False):
+    lib = load()
+    _gpu(x, 'input')
+    rows, cols = x.shape
+    out = torch.empty((rows, cols), dtype=torch.uint8, device=x.device)
+    out_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device)
+    if in_time:
+        rc = lib.msamp_cast_transpose_intime(
+            _ptr(x), _dt(x), rows, cols, _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), _ptr(out_t), fp8_dt,
+            margin, FLAG_NAN_TO_INF if nan_to_inf else 0, _ptr(workspace(x.device)), _stream()
+        )
+    else:
+        rc = lib.msamp_cast_transpose(
+            _ptr(x), _dt(x), rows, cols, _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), _ptr(out_t), fp8_dt,
+            _stream()
+        )
+    _check(rc, 'msamp_cast_transpose')
+    return out, out_t
+
+
+def fp8_transpose(q):
+    lib = load()
+    _gpu(q, 'input')
+    rows, cols = q.shape
+    out = torch.empty((cols, rows), dtype=torch.uint8, device=q.device)
+    _check(lib.msamp_fp8_transpose(_ptr(q), rows, cols, _ptr(out), _stream()), 'msamp_fp8_transpose')
+    return out
+
+
+def scale_cast(x, scale, out_dtype):
+    """out = out_dtype(float(x) * scale) with IEEE overflow."""
+    lib = load()
+    _gpu(x, 'input')
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _check(
+        lib.msamp_scale_cast(_ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(out), _TORCH_TO_DT[out_dtype], _stream()),
+        'msamp_scale_cast'
+    )
+    return out
+
+
+# ---- GEMM ---------------------------------------------------------------------------------------
+def fp8_gemm(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, out, accumulate=False, bias=None):
+    """out[N,M] (+)= (b[N,K] . a[M,K]^T) * a_scale_inv * b_scale_inv (+ bias[M])."""
+    lib = load()
+    _gpu(a, 'mat_a')
+    _gpu(b, 'mat_b')
+    m, k = a.shape
+    n = b.shape[0]
+    if b.shape[1] != k or tuple(out.shape) != (n, m):
+        raise ValueError(f'shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}')
+    _check(
+        lib.msamp_fp8_gemm(
+            _ptr(a), a_dt, _ptr(a_scale_inv), _ptr(b), b_dt, _ptr(b_scale_inv), _ptr(out), _dt(out), m, n, k,
+            1 if accumulate else 0, _ptr(bias), _dt(bias) if bias is not None else DT_F32, _stream()
+        ), 'msamp_fp8_gemm'
+    )
+    return out
+
+
+# ---- AdamW --------------------------------------------------------------------------------------
+_STATE_DT = {torch.float32: DT_F32, torch.float16: DT_F16}
+
+
+def state_dt(tensor, qtype_value=None):
+    """Library code of an optimizer-state payload (uint8 payloads need the qtype to tell the format)."""
+    if tensor.dtype == torch.uint8:
+        return qtype_value if qtype_value is not None else DT_E4M3
+    return _STATE_DT[tensor.dtype]
+
+
+def adamw_stage1(param, grad, exp_avg, exp_avg_dt, exp_avg_factor, exp_avg_amax, beta1, exp_avg_sq, exp_avg_sq_dt,
+                 exp_avg_sq_factor, exp_avg_sq_amax, beta2, eps, step, lr, bias_correction):
+    lib = load()
+    _gpu(param, 'param')
+    _check(
+        lib.msamp_adamw_fp8_stage1(
+            _ptr(param), _ptr(grad), param.numel(), _ptr(exp_avg), exp_avg_dt, exp_avg_factor, _ptr(exp_avg_amax), beta1,
+            _ptr(exp_avg_sq), exp_avg_sq_dt, exp_avg_sq_factor, _ptr(exp_avg_sq_amax), beta2, eps, step, lr,
+            1 if bias_correction else 0, _stream()
+        ), 'msamp_adamw_fp8_stage1'
+    )
+
+
+def adamw_stage2(grad, exp_avg, exp_avg_dt, old_factor, new_factor, beta1, exp_avg_sq, exp_avg_sq_dt, old_sq_factor,
+                 new_sq_factor, beta2):
+    lib = load()
+    _gpu(grad, 'grad')
+    _check(
+        lib.msamp_adamw_fp8_stage2(
+            _ptr(grad), grad.numel(), _ptr(exp_avg), exp_avg_dt, old_factor, new_factor, beta1, _ptr(exp_avg_sq),
+            exp_avg_sq_dt, old_sq_factor, new_sq_factor, beta2, _stream()
+        ), 'msamp_adamw_fp8_stage2'
+    )
+
+
+ADAMW_DESC_WORDS = 19    # int64 words per msamp_adamw_tensor (152 bytes)
+
+
+def adamw_fused(desc, n_tensors, block_map, n_blocks, weight_dt, grad_dt, lr, beta1, beta2, eps, weight_decay, step,
+                bias_correction, adam_mode, maximize, tensor_scale):
+    lib = load()
+    _gpu(desc, 'descriptor table')
+    _check(
+        lib.msamp_adamw_fp8_fused(
+            _ptr(desc), n_tensors, _ptr(block_map), n_blocks, weight_dt, grad_dt, lr, beta1, beta2, eps, weight_decay,
+            step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0, 1 if tensor_scale else 0,
+            _stream()
+        ), 'msamp_adamw_fp8_fused'
+    )

@@ -1,0 +1,107 @@
+"""F.linear with ScalingTensor weights: FP8 forward, dgrad and wgrad (msamp/nn/functional.py:16-194)."""
+
+import torch
+import torch.nn.functional as F
+
+from msamp.common.dtype import Dtypes
+from msamp.common.tensor import ScalingTensor
+from msamp.operators.gemm import Gemm
+from msamp.nn.state import model_state
+
+
+class _FP8GemmFunction(torch.autograd.Function):
+    """y = x W^T with x, W in E4M3; dx = dy W and dW = dy^T x with dy in E5M2; fp32 accumulation."""
+    @staticmethod
+    def forward(ctx, input, weight, metas, dtype_holder):
+        ctx.metas = metas
+        model_state.check_metas_in_flat(metas)
+        input_fp8 = input.cast(Dtypes.kfloat8_e4m3, meta=metas['input'])
+        weight_fp8 = weight.cast(Dtypes.kfloat8_e4m3)
+
+        ctx.input_fp8 = input_fp8
+        ctx.input_fp8.requires_grad = input.requires_grad
+        ctx.weight_fp8 = weight_fp8
+        ctx.weight = weight
+        ctx.output_dtype = dtype_holder.dtype
+        ctx.output_qtype = Dtypes.dtype_to_qtype[dtype_holder.dtype]
+        return Gemm.fp8_gemm(weight_fp8, input_fp8, ctx.output_qtype, use_split_accumulator=False)
+
+    @staticmethod
+    def backward(ctx, output_grad):
+        output_grad = output_grad.contiguous()
+        metas = ctx.metas
+        ograd_fp8, ograd_fp8_t = output_grad.fused_cast_transpose(Dtypes.kfloat8_e5m2, meta=metas['ograd'])
+
+        input_grad = None
+        if ctx.input_fp8.requires_grad:
+            weight_fp8_t = ctx.weight_fp8.fp8_transpose()
+            input_grad = Gemm.fp8_gemm(weight_fp8_t, ograd_fp8, ctx.output_qtype, use_split_accumulator=True)
+
+        if ctx.weight.requires_grad:
+            input_fp8_t = ctx.input_fp8.fp8_transpose()
+            if ctx.weight.grad is None:
+                wgrad = Gemm.fp8_gemm(input_fp8_t, ograd_fp8_t, ctx.output_qtype, use_split_accumulator=True)
+            else:
+                # gradient accumulation: add into the dequantized previous gradient
+                old_wgrad = ctx.weight.grad.to(ctx.output_dtype)
+                wgrad = Gemm.fp8_gemm(
+                    input_fp8_t, ograd_fp8_t, ctx.output_qtype, accumulate=True, out=old_wgrad, use_split_accumulator=True
+                )
+                del old_wgrad
+            if model_state.use_fp8_ddp:
+                wgrad.meta = metas['wgrad']
+            else:
+                wgrad = wgrad.cast(Dtypes.kfloat8_e4m3, meta=metas['wgrad'], sync=True)
+            ctx.weight.backward_grad_update(wgrad)
+
+        return input_grad, None, None, None
+
+
+class FunctionalOverider:
+    """Replaces torch.nn.functional.linear with a version that routes ScalingTensor weights to FP8."""
+    EMPTY_GRAD_TENSOR = torch.nn.Parameter(torch.tensor([]))
+    _installed = False
+
+    @classmethod
+    def override(cls):
+        if cls._installed:
+            return
+        cls._installed = True
+        F.linear = cls._get_wrapper_for_linear(F.linear)
+
+    @classmethod
+    def _get_wrapper_for_linear(cls, old_fn):
+        def new_fn(input, weight, bias=None):
+            """linear(input, weight, bias=None): y = x A^T + b; `weight` may be a ScalingTensor carrying
+            `_scaling_metas`, in which case the three GEMMs run in FP8 and the bias is added afterwards
+            in the output dtype (the autocast dtype if autocast is on, else the input's)."""
+            if not isinstance(input, torch.Tensor):
+                raise TypeError(f'input should be a torch.Tensor. current type: {type(input)}')
+            if not isinstance(weight, (torch.Tensor, ScalingTensor)):
+                raise TypeError(f'weight should be a torch.Tensor or ScalingTensor. current type: {type(weight)}')
+            if bias is not None and not isinstance(bias, torch.Tensor):
+                raise TypeError(f'bias should be a torch.Tensor. current type: {type(bias)}')
+            if isinstance(weight, torch.Tensor):
+                return old_fn(input, weight, bias=bias)
+            if not hasattr(weight, '_scaling_metas'):
+                raise ValueError('weight (ScalingTensor) should have _scaling_metas attribute.')
+
+            model_state.ready_to_scale_tensor = True
+            shape = input.shape
+            if len(shape) != 2:
+                input = input.reshape(-1, shape[-1])
+            if torch.is_autocast_enabled():
+                output_dtype = torch.get_autocast_gpu_dtype()
+            else:
+                output_dtype = input.dtype
+            out = _FP8GemmFunction.apply(input, weight, weight._scaling_metas, cls.EMPTY_GRAD_TENSOR.type(output_dtype))
+            if bias is not None:
+                out = out + bias.type(output_dtype).view(1, -1)
+            if len(shape) != 2:
+                out = out.view(shape[:-1] + (-1, ))
+            return out
+
+        return new_fn
+
+
+FunctionalOverider.override()

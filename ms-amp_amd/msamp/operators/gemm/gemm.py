@@ -1,0 +1,52 @@
+"""Gemm.fp8_gemm (msamp/operators/gemm/gemm.py:58-179) on the gfx950 FP8 MFMA kernel."""
+
+import torch
+import torch.nn.functional as F
+
+from msamp import _backend
+from msamp.common.dtype import Dtypes
+from msamp.common.tensor import ScalingTensor
+
+
+class Gemm:
+    """FP8 GEMM entry point."""
+    _te_base = 16
+
+    @staticmethod
+    def _round2times(value, base):
+        """Smallest multiple of base that is >= value."""
+        return (value + base - 1) // base * base
+
+    @classmethod
+    @torch.no_grad()
+    def fp8_gemm(cls, mat_a, mat_b, out_qtype, bias=None, accumulate=False, out=None, use_split_accumulator=False):
+        """out[N, M] = (mat_b[N, K] @ mat_a[M, K].T) * a.scale_inv * b.scale_inv.
+
+        mat_a, mat_b: contiguous FP8 ScalingTensors on the GPU.  The kernel accumulates in fp32
+        over the full K (use_split_accumulator has nothing to switch) and writes out_qtype; with
+        `accumulate` it adds into `out`.  Only K needs padding (to a multiple of 16 bytes, with
+        FP8 zeros); ragged M and N are handled inside the kernel.
+        """
+        assert isinstance(mat_a, ScalingTensor)
+        assert isinstance(mat_b, ScalingTensor)
+        assert mat_a.is_cuda and mat_a.is_contiguous()
+        assert mat_b.is_cuda and mat_b.is_contiguous()
+        assert Dtypes.is_fp8_qtype(mat_a.qtype) and Dtypes.is_fp8_qtype(mat_b.qtype)
+
+        M, K = mat_a.shape
+        N = len(mat_b)
+        a, b = mat_a.value, mat_b.value
+        pK = cls._round2times(K, cls._te_base) - K
+        if pK > 0:
+            a = F.pad(a, (0, pK))
+            b = F.pad(b, (0, pK))
+        out_dtype = Dtypes.get_dtype_from_qtype(out_qtype)
+        if out is None:
+            assert not accumulate, 'accumulate needs an output tensor'
+            out = torch.empty(N, M, dtype=out_dtype, device=a.device)
+        else:
+            assert out.is_cuda and out.is_contiguous() and out.dtype == out_dtype
+        _backend.fp8_gemm(
+            a, int(mat_a.qtype), mat_a.meta.scale_inv, b, int(mat_b.qtype), mat_b.meta.scale_inv, out, accumulate, bias
+        )
+        return out

@@ -1,0 +1,103 @@
+"""FP8 AdamW step (E4M3/E5M2 weights and grads, E4M3 first moment, scaled-fp16 second moment).
+
+Test infrastructure only.  Follows msamp/optim/adamw.py:148-199 and the kernels at
+msamp/optim/adamw.cu:39-50,66-72, evaluated left to right in float32 without fused
+multiply-add.
+"""
+
+import math
+
+import numpy as np
+import torch
+
+from . import fp8
+from .scaling import compute_scaling_factor
+
+
+def host_constants(lr, beta1, beta2, step, bias_correction=True):
+    """float32 step_size and sqrt(bias_correction2) as msamp/optim/adamw.cu:104-107 forms them
+    (float arguments, double pow, results narrowed to float)."""
+    b1 = float(np.float32(beta1))
+    b2 = float(np.float32(beta2))
+    bc1 = np.float32(1.0 - b1**step) if bias_correction else np.float32(1.0)
+    bc2 = np.float32(1.0 - b2**step) if bias_correction else np.float32(1.0)
+    step_size = np.float32(np.float32(lr) / bc1)
+    sbc2 = np.float32(math.sqrt(float(bc2)))
+    return float(step_size), float(sbc2)
+
+
+def moments(g, m_q, inv_m, v_q, inv_v, beta1, beta2, m_fmt=fp8.E4M3):
+    """m' and v' (float32) from the stored quantized moments; adamw.cu:40-42."""
+    b1 = torch.tensor(beta1, dtype=torch.float32)
+    b2 = torch.tensor(beta2, dtype=torch.float32)
+    one = torch.tensor(1.0, dtype=torch.float32)
+    mf = fp8.decode(m_q, m_fmt) if m_q.dtype == torch.uint8 else m_q.to(torch.float32)
+    vf = v_q.to(torch.float32)
+    m_new = b1 * mf * inv_m + (one - b1) * g
+    v_new = b2 * vf * inv_v + (one - b2) * (g * g)
+    return m_new, v_new
+
+
+def step_tensor(w_q, w_meta, w_fmt, g_q, g_scale_inv, g_fmt, m_q, m_meta, v_q, v_meta, *, lr, beta1, beta2, eps,
+                weight_decay, step, bias_correction=True, adam_mode=False, maximize=False):
+    """One fused step on one tensor.  Metas are dicts {'scale','scale_inv','amax'} of 0-d/1-d f32 tensors.
+
+    Returns new (w_q, w_meta, m_q, m_meta, v_q, v_meta) and the fp32 intermediates (p, m', v').
+    """
+    f32 = torch.float32
+    step_size, sbc2 = host_constants(lr, beta1, beta2, step, bias_correction)
+    step_size = torch.tensor(step_size, dtype=f32)
+    sbc2 = torch.tensor(sbc2, dtype=f32)
+    epsf = torch.tensor(eps, dtype=f32)
+
+    p = fp8.decode(w_q, w_fmt) * w_meta['scale_inv'].to(f32)
+    g = fp8.decode(g_q, g_fmt) * g_scale_inv.to(f32)
+    if maximize:
+        g = -g
+    if weight_decay != 0:
+        if adam_mode:
+            g = g + torch.tensor(weight_decay, dtype=f32) * p
+        else:
+            p = p * torch.tensor(1 - lr * weight_decay, dtype=f32)
+    inv_m = (1.0 / m_meta['scale']).to(f32)
+    inv_v = (1.0 / v_meta['scale']).to(f32)
+    m_new, v_new = moments(g, m_q, inv_m, v_q, inv_v, beta1, beta2)
+    denom = torch.sqrt(v_new) / sbc2 + epsf
+    p = p - step_size * (m_new / denom)
+
+    # weight: in-time requantization with fresh amax (adamw.py:173-174)
+    w_amax = p.abs().max()
+    w_scale = compute_scaling_factor(w_amax, w_meta['scale'], fp8.FP_MAX[w_fmt], 0)
+    w_new = fp8.encode(p * w_scale, w_fmt)
+    w_meta_new = {'scale': w_scale, 'scale_inv': torch.reciprocal(w_scale), 'amax': w_amax.reshape(1)}
+
+    # moments: fresh amax, fallback scale 1.0 (adamw.py:176-184)
+    one = torch.ones(())
+    m_amax = m_new.abs().max()
+    v_amax = v_new.abs().max()
+    m_scale = compute_scaling_factor(m_amax, one, fp8.FP_MAX[fp8.E4M3], 0)
+    v_scale = compute_scaling_factor(v_amax, one, 65504.0, 0)
+    m_out = fp8.encode(m_new * m_scale, fp8.E4M3)
+    v_out = (v_new * v_scale).to(torch.float16)
+    m_meta_new = {'scale': m_scale, 'scale_inv': torch.reciprocal(m_scale), 'amax': m_amax.reshape(1)}
+    v_meta_new = {'scale': v_scale, 'scale_inv': torch.reciprocal(v_scale), 'amax': v_amax.reshape(1)}
+    return (w_new, w_meta_new, m_out, m_meta_new, v_out, v_meta_new), (p, m_new, v_new)
+
+
+def stage1(p, g, m_q, inv_m, v_q, inv_v, *, lr, beta1, beta2, eps, step, bias_correction=True):
+    """adamw_fp8_stage1_kernel (adamw.cu:30-59) on fp32 param/grad: returns p', amax_m, amax_v."""
+    f32 = torch.float32
+    step_size, sbc2 = host_constants(lr, beta1, beta2, step, bias_correction)
+    m_new, v_new = moments(g, m_q, torch.tensor(inv_m, dtype=f32), v_q, torch.tensor(inv_v, dtype=f32), beta1, beta2)
+    denom = torch.sqrt(v_new) / torch.tensor(sbc2, dtype=f32) + torch.tensor(eps, dtype=f32)
+    p_new = p - torch.tensor(step_size, dtype=f32) * (m_new / denom)
+    return p_new, m_new.abs().max(), v_new.abs().max()
+
+
+def stage2(g, m_q, inv_m, new_m_scale, v_q, inv_v, new_v_scale, *, beta1, beta2):
+    """adamw_fp8_stage2_kernel (adamw.cu:61-74): requantized moments."""
+    f32 = torch.float32
+    m_new, v_new = moments(g, m_q, torch.tensor(inv_m, dtype=f32), v_q, torch.tensor(inv_v, dtype=f32), beta1, beta2)
+    m_out = fp8.encode(m_new * torch.tensor(new_m_scale, dtype=f32), fp8.E4M3)
+    v_out = (v_new * torch.tensor(new_v_scale, dtype=f32)).to(v_q.dtype)
+    return m_out, v_out

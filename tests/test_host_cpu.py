@@ -1,0 +1,215 @@
+"""Host-side logic that needs no GPU: dtype tables, meta state machine, hooks, model-state flattening,
+error behaviour, and that the C-ABI library loads and exports every declared symbol."""
+
+import ctypes
+import json
+import os
+import re
+
+import pytest
+import torch
+
+import msamp
+from msamp import _backend
+from msamp.common.dtype import Dtypes, Floating
+from msamp.common.tensor import HookManager, ScalingMeta, ScalingTensor, TypeCast
+from msamp.nn import FP8Linear, LinearReplacer, ScalingParameter, model_state
+from msamp.nn.state import ModelState
+from msamp.operators.gemm import Gemm
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = json.load(open(os.path.join(ROOT, 'tests', 'golden', 'reference_kats.json')))
+
+
+def test_fp_max_table():
+    k = GOLDEN['fp_max']
+    assert Floating.qfp_max[Dtypes.kfloat8_e4m3] == k['e4m3']
+    assert Floating.qfp_max[Dtypes.kfloat8_e5m2] == k['e5m2']
+    assert Floating.qfp_max[Dtypes.kfloat16] == k['fp16']
+    assert Floating.fp_maxs[torch.uint8] == k['e4m3'] and Floating.fp_maxs[torch.int8] == k['e5m2']
+    assert Floating.qfp_max[Dtypes.kfloat32] == torch.finfo(torch.float32).max
+    assert Floating.qfp_max[Dtypes.kbfloat16] == torch.finfo(torch.bfloat16).max
+
+
+def test_dtypes():
+    assert Dtypes.is_fp8_qtype(Dtypes.kfloat8_e4m3) and Dtypes.is_fp8_qtype(Dtypes.kfloat8_e5m2)
+    assert not Dtypes.is_fp8_qtype(Dtypes.kfloat16)
+    assert Dtypes.get_dtype_from_qtype(Dtypes.kfloat8_e4m3) == torch.uint8
+    assert Dtypes.get_dtype_from_qtype(Dtypes.kfloat8_e5m2) == torch.uint8
+    assert Dtypes.get_dtype_from_qtype(Dtypes.kbfloat16) == torch.bfloat16
+    assert Dtypes.dtype_to_qtype[torch.int8] == Dtypes.kfloat8_e5m2
+    assert [int(q) for q in (Dtypes.kfloat32, Dtypes.kfloat16, Dtypes.kbfloat16, Dtypes.kfloat8_e4m3, Dtypes.kfloat8_e5m2)] \
+        == [_backend.DT_F32, _backend.DT_F16, _backend.DT_BF16, _backend.DT_E4M3, _backend.DT_E5M2]
+    assert torch.randn(2).qtype == Dtypes.kfloat32
+
+
+def test_warmup_truth_table():
+    for c in GOLDEN['warmup_truth_table']['cases']:
+        meta = ScalingMeta(Dtypes.kfloat8_e4m3, window_size=c['window'], device='cpu')
+        for _ in range(c['counter']):
+            meta.amax_counter += 1
+        assert bool(meta.is_warmup()) == c['warmup']
+        assert meta.is_in_time_scaling() == c['in_time']
+
+
+def test_in_time_scaling_flag_and_context():
+    meta = ScalingMeta(Dtypes.kfloat8_e4m3, device='cpu')
+    assert meta.is_in_time_scaling()
+    with ScalingMeta.in_time_scaling_context(False):
+        assert not meta.is_in_time_scaling()
+        with ScalingMeta.in_time_scaling_context(True):
+            assert meta.is_in_time_scaling()
+        assert not meta.is_in_time_scaling()
+    assert meta.is_in_time_scaling() and ScalingMeta.in_time_scaling
+
+
+def test_meta_copy_clone():
+    a = ScalingMeta(Dtypes.kfloat8_e4m3, window_size=4, device='cpu')
+    a.scale.fill_(8)
+    a.amax[1] = 3
+    a.amax_counter += 2
+    b = a.clone()
+    assert b is not a and b.scale.item() == 8 and b.amax[1].item() == 3 and b.amax_counter.item() == 2
+    b.scale.fill_(2)
+    assert a.scale.item() == 8
+    c = ScalingMeta(Dtypes.kfloat8_e5m2, window_size=4, device='cpu')
+    c.copy_(a)
+    assert c.qtype == Dtypes.kfloat8_e4m3 and c.scale.item() == 8 and c.amax_counter.item() == 2
+
+
+def test_hook_manager():
+    seen = []
+    hm = HookManager()
+    h1 = hm.register_hook(lambda _, inp, out: seen.append((inp[0], out)))
+    h2 = hm.register_hook(lambda _, inp, out: seen.append((inp[0], out)))
+    x = torch.randn(2, 3)
+    hm(x)
+    assert len(seen) == 2 and all(i is x and o is x for i, o in seen)
+    h1.remove()
+    h2.remove()
+    seen.clear()
+    hm(x)
+    assert not seen
+
+
+def test_round2times():
+    for value, base, expected in GOLDEN['round2times']['cases']:
+        assert Gemm._round2times(value, base) == expected
+
+
+def test_scaling_tensor_type_checks_and_scale_only_ops():
+    meta = ScalingMeta(Dtypes.kfloat8_e4m3, device='cpu')
+    with pytest.raises(TypeError):
+        ScalingTensor(torch.zeros(4, dtype=torch.float16), meta)
+    st = ScalingTensor(torch.zeros(4, dtype=torch.uint8), meta)
+    st.mul_(2.0)
+    assert meta.scale_inv.item() == 2.0
+    st.div_(torch.tensor([4.0]))
+    assert meta.scale_inv.item() == 0.5
+    with pytest.raises(ValueError):
+        st.mul_(torch.ones(2))
+    assert not st.is_floating_point() and not torch.is_floating_point(st)
+    assert torch.zeros_like(st).dtype == torch.uint8
+    assert st.shape == (4, ) and st.numel() == 4 and len(st) == 4 and st.is_leaf and st.grad_fn is None
+    assert st.isnan().sum() == 0
+    st.value[1] = 127
+    assert st.isnan().tolist() == [False, True, False, False]
+    assert (ScalingTensor(torch.tensor([0x85], dtype=torch.uint8), meta).abs().value == 5).all()
+    with pytest.raises(TypeError):
+        st.copy_(torch.zeros(4))
+    with pytest.raises(TypeError):
+        st.to(torch.int32)
+    with pytest.raises(TypeError):
+        st.to(torch.float32, torch.float16)
+
+
+def test_has_inf_or_nan_and_amp_unscale_on_cpu():
+    meta = ScalingMeta(Dtypes.kfloat8_e4m3, device='cpu')
+    st = ScalingTensor(torch.zeros(4, dtype=torch.uint8), meta)
+    assert not st.has_inf_or_nan()
+    found = torch.zeros(1)
+    plain = torch.ones(3)
+    torch._amp_foreach_non_finite_check_and_unscale_([plain], found, torch.tensor(0.5))
+    assert plain.tolist() == [0.5] * 3 and found.item() == 0
+    meta.amax[0] = float('inf')
+    assert st.has_inf_or_nan()
+
+
+def test_compute_paths_refuse_cpu_tensors():
+    meta = ScalingMeta(Dtypes.kfloat8_e4m3, device='cpu')
+    with pytest.raises(ValueError):
+        TypeCast.cast_to_fp8(torch.randn(4), meta)
+    with pytest.raises(ValueError):
+        TypeCast.cast_from_fp8(torch.zeros(4, dtype=torch.uint8), meta, Dtypes.kfloat32)
+    with pytest.raises(ValueError):
+        _backend.fp8_transpose(torch.zeros(4, 4, dtype=torch.uint8))
+
+
+def test_model_state_flatten_and_check_on_cpu():
+    state = ModelState()
+    model = torch.nn.Sequential(FP8Linear(4, 8), torch.nn.ReLU(), FP8Linear(8, 2))
+    for m in model:
+        if isinstance(m, FP8Linear):    # keep this test on the CPU whatever the box
+            for meta in m.scaling_metas.values():
+                meta.cpu()
+    state.register_scaling_metas(model)
+    flat = state.flattened_scaling_metas
+    assert set(flat) == {'input', 'wgrad', 'ograd'}
+    assert flat['input']['amaxs'].shape == (2, 16) and flat['wgrad']['amaxs'].shape == (2, 1)
+    assert flat['ograd']['qtype'] == Dtypes.kfloat8_e5m2
+    first = model[0].scaling_metas['input']
+    assert first.locked
+    first.amax[0] = 5.0
+    first.scale.fill_(3.0)
+    first.amax_counter += 1
+    assert flat['input']['amaxs'][0, 0].item() == 5.0 and flat['input']['scales'][0].item() == 3.0
+    assert flat['input']['amax_counters'].tolist() == [1, 0]
+    state.check_metas_in_flat(model[0].scaling_metas)
+    first.scale = torch.ones(())
+    with pytest.raises(RuntimeError):
+        state.check_metas_in_flat(model[0].scaling_metas)
+    st = ScalingTensor(torch.zeros(2, dtype=torch.uint8), model[2].scaling_metas['input'])
+    with pytest.raises(ValueError):
+        st.data = ScalingTensor(torch.zeros(2, dtype=torch.uint8), ScalingMeta(Dtypes.kfloat8_e4m3, device='cpu'))
+
+
+def test_fp8linear_structure_and_replacer_attr_compare():
+    lin = FP8Linear(4, 8, use_bias=False)
+    assert isinstance(lin.weight, ScalingParameter) and lin.bias is None
+    assert [n for n, _ in lin.named_parameters()] == ['weight']
+    assert lin.weight.dtype == torch.float16 and lin.weight._scaling_metas is lin.scaling_metas
+    assert lin.scaling_metas['input'].window_size == 16 and lin.scaling_metas['wgrad'].window_size == 1
+    assert lin.half() is lin and lin.weight.dtype == torch.float16
+    a, b = LinearReplacer._compare_attrs(type(torch.nn.Linear(1, 1)), lin)
+    assert 'scaling_metas' in b
+
+
+def test_initialize_argument_checks():
+    with pytest.raises(ValueError):
+        msamp.initialize(object())
+    with pytest.raises(ValueError):
+        msamp.initialize(torch.nn.Linear(2, 2), opt_level='O3')
+    model = torch.nn.Linear(2, 2)
+    with pytest.raises(ValueError):
+        msamp.initialize(model, torch.optim.SGD(model.parameters(), lr=0.1))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, 'include', 'msamp_hip.h')).read()
+    declared = set(re.findall(r'\b(msamp_[a-z0-9_]+)\s*\(', header))
+    assert declared == set(_backend.EXPORTED_SYMBOLS), declared ^ set(_backend.EXPORTED_SYMBOLS)
+    lib = ctypes.CDLL(_backend.library_path())
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _backend.load().msamp_hip_version() >= 100
+    assert _backend.load().msamp_last_error() is not None
+
+
+def test_adamw_descriptor_layout_matches_header():
+    header = open(os.path.join(ROOT, 'include', 'msamp_hip.h')).read()
+    body = header[header.index('typedef struct msamp_adamw_tensor {'):header.index('} msamp_adamw_tensor;')]
+    n_ptr = len(re.findall(r'\*\s*\w+;', body))
+    assert n_ptr == 14
+    assert 8 * n_ptr + 8 + 12 + 12 + 8 == 8 * _backend.ADAMW_DESC_WORDS
+    assert int(re.search(r'#define MSAMP_ADAMW_CHUNK (\d+)', header).group(1)) == _backend.ADAMW_CHUNK
+    assert int(re.search(r'#define MSAMP_WORKSPACE_BYTES (\d+)', header).group(1)) == _backend.WORKSPACE_BYTES
