@@ -175,12 +175,20 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
     return v;
 }
 
-// The pow-2 scale rule, evaluated the way float32 torch evaluates it: the quotient is an IEEE
-// float division, log2 is the correctly rounded float log2 (double log2 narrowed once), 2^|e|
-// overflows to +Inf from |e| = 128.
+// The pow-2 scale rule, evaluated the way float32 torch evaluates it: `fp_max / amax` with a Python
+// float on the left is reciprocal(amax) * fp_max (two roundings, in eager mode and under TorchScript
+// alike), log2 is the correctly rounded float log2 (double log2 narrowed once), 2^|e| overflows to
+// +Inf from |e| = 128.
 __device__ __forceinline__ float scale_rule(float amax, float fallback, float fp_max, int margin) {
-    float q = fp_max / amax;
-    float e = floorf(static_cast<float>(log2(static_cast<double>(q)))) - static_cast<float>(margin);
+    const float recip = 1.0f / amax;
+    float q = recip * fp_max;
+    // floor(float(log2(q))) with the float rounding done by hand: keeping the double result live in
+    // double arithmetic stops the compiler from shrinking the call to the (not correctly rounded)
+    // float log2.  If narrowing d to float reaches the next integer, the floor is that integer.
+    const double d = log2(static_cast<double>(q));
+    double fl = floor(d);
+    if (static_cast<float>(d) >= static_cast<float>(fl + 1.0)) fl += 1.0;
+    float e = static_cast<float>(fl) - static_cast<float>(margin);
     float ae = fabsf(e);
     float sf;
     if (ae != ae) {

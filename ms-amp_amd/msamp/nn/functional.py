@@ -91,7 +91,7 @@ class FunctionalOverider:
             if len(shape) != 2:
                 input = input.reshape(-1, shape[-1])
             if torch.is_autocast_enabled():
-                output_dtype = torch.get_autocast_gpu_dtype()
+                output_dtype = torch.get_autocast_dtype('cuda')
             else:
                 output_dtype = input.dtype
             out = _FP8GemmFunction.apply(input, weight, weight._scaling_metas, cls.EMPTY_GRAD_TENSOR.type(output_dtype))

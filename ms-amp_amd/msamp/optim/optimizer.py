@@ -52,13 +52,21 @@ class LBOptimizer(Optimizer):
             if not ScalingMeta.in_time_scaling:
                 names.append('wgrad')
         margin = 0
+        masks = []
         for name in names:
             meta = metas[name]
             fp_max = Floating.qfp_max[meta['qtype']]
-            bad = _backend.scale_update(meta['scales'], meta['amaxs'], fp_max, margin)
-            counters = meta['amax_counters']
+            masks.append(_backend.scale_update(meta['scales'], meta['amaxs'], fp_max, margin))
+        # the counters live on the host (they steer which cast kernel is enqueued next), so the
+        # non-finite masks come back in one device-to-host copy per step
+        bad = torch.cat(masks).cpu().bool()
+        offset = 0
+        for name in names:
+            counters = metas[name]['amax_counters']
+            n = counters.numel()
             counters += 1
-            counters[bad.cpu().bool()] = 0
+            counters[bad[offset:offset + n]] = 0
+            offset += n
 
     # ---- state (de)serialisation with order indices instead of tensors ---------------------------
     def state_dict(self):

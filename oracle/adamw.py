@@ -14,6 +14,13 @@ from . import fp8
 from .scaling import compute_scaling_factor
 
 
+def _sqrt(x):
+    """IEEE correctly rounded float32 square root.  torch's CPU sqrt goes through a vector math
+    library that is not correctly rounded on large tensors (about 0.6 % of results are one ulp
+    off); numpy's is, and so are CUDA's sqrtf (the reference kernel) and the HIP kernel's."""
+    return torch.from_numpy(np.sqrt(x.detach().numpy()))
+
+
 def host_constants(lr, beta1, beta2, step, bias_correction=True):
     """float32 step_size and sqrt(bias_correction2) as msamp/optim/adamw.cu:104-107 forms them
     (float arguments, double pow, results narrowed to float)."""
@@ -39,7 +46,8 @@ def moments(g, m_q, inv_m, v_q, inv_v, beta1, beta2, m_fmt=fp8.E4M3):
 
 
 def step_tensor(w_q, w_meta, w_fmt, g_q, g_scale_inv, g_fmt, m_q, m_meta, v_q, v_meta, *, lr, beta1, beta2, eps,
-                weight_decay, step, bias_correction=True, adam_mode=False, maximize=False):
+                weight_decay, step, bias_correction=True, adam_mode=False, maximize=False, tensor_scale=True,
+                w_fp_max=None):
     """One fused step on one tensor.  Metas are dicts {'scale','scale_inv','amax'} of 0-d/1-d f32 tensors.
 
     Returns new (w_q, w_meta, m_q, m_meta, v_q, v_meta) and the fp32 intermediates (p, m', v').
@@ -50,7 +58,10 @@ def step_tensor(w_q, w_meta, w_fmt, g_q, g_scale_inv, g_fmt, m_q, m_meta, v_q, v
     sbc2 = torch.tensor(sbc2, dtype=f32)
     epsf = torch.tensor(eps, dtype=f32)
 
-    p = fp8.decode(w_q, w_fmt) * w_meta['scale_inv'].to(f32)
+    if w_fmt == 'f16':
+        p = w_q.to(f32) * w_meta['scale_inv'].to(f32)
+    else:
+        p = fp8.decode(w_q, w_fmt) * w_meta['scale_inv'].to(f32)
     g = fp8.decode(g_q, g_fmt) * g_scale_inv.to(f32)
     if maximize:
         g = -g
@@ -62,23 +73,32 @@ def step_tensor(w_q, w_meta, w_fmt, g_q, g_scale_inv, g_fmt, m_q, m_meta, v_q, v
     inv_m = (1.0 / m_meta['scale']).to(f32)
     inv_v = (1.0 / v_meta['scale']).to(f32)
     m_new, v_new = moments(g, m_q, inv_m, v_q, inv_v, beta1, beta2)
-    denom = torch.sqrt(v_new) / sbc2 + epsf
+    denom = _sqrt(v_new) / sbc2 + epsf
     p = p - step_size * (m_new / denom)
 
     # weight: in-time requantization with fresh amax (adamw.py:173-174)
     w_amax = p.abs().max()
-    w_scale = compute_scaling_factor(w_amax, w_meta['scale'], fp8.FP_MAX[w_fmt], 0)
-    w_new = fp8.encode(p * w_scale, w_fmt)
+    if w_fmt == 'f16':    # scaled fp16 weight (cast.py:68-95)
+        w_scale = compute_scaling_factor(w_amax, w_meta['scale'], 65504.0, 0)
+        w_new = (p * w_scale).to(torch.float16)
+    else:
+        w_scale = compute_scaling_factor(w_amax, w_meta['scale'], fp8.FP_MAX[w_fmt], 0)
+        w_new = fp8.encode(p * w_scale, w_fmt)
     w_meta_new = {'scale': w_scale, 'scale_inv': torch.reciprocal(w_scale), 'amax': w_amax.reshape(1)}
 
     # moments: fresh amax, fallback scale 1.0 (adamw.py:176-184)
     one = torch.ones(())
     m_amax = m_new.abs().max()
     v_amax = v_new.abs().max()
-    m_scale = compute_scaling_factor(m_amax, one, fp8.FP_MAX[fp8.E4M3], 0)
-    v_scale = compute_scaling_factor(v_amax, one, 65504.0, 0)
-    m_out = fp8.encode(m_new * m_scale, fp8.E4M3)
-    v_out = (v_new * v_scale).to(torch.float16)
+    m_scale = compute_scaling_factor(m_amax, one, fp8.FP_MAX[fp8.E4M3], 0) if tensor_scale else one
+    v_scale = compute_scaling_factor(v_amax, one, 65504.0, 0) if tensor_scale else one
+    m_store, v_store = m_new, v_new
+    if adam_mode and weight_decay != 0:
+        # the second stage recomputes the moments from the gradient WITHOUT the L2 term (adamw.py:186-199)
+        g_raw = fp8.decode(g_q, g_fmt) * g_scale_inv.to(f32)
+        m_store, v_store = moments(-g_raw if maximize else g_raw, m_q, inv_m, v_q, inv_v, beta1, beta2)
+    m_out = fp8.encode(m_store * m_scale, fp8.E4M3)
+    v_out = (v_store * v_scale).to(torch.float16)
     m_meta_new = {'scale': m_scale, 'scale_inv': torch.reciprocal(m_scale), 'amax': m_amax.reshape(1)}
     v_meta_new = {'scale': v_scale, 'scale_inv': torch.reciprocal(v_scale), 'amax': v_amax.reshape(1)}
     return (w_new, w_meta_new, m_out, m_meta_new, v_out, v_meta_new), (p, m_new, v_new)
@@ -89,7 +109,7 @@ def stage1(p, g, m_q, inv_m, v_q, inv_v, *, lr, beta1, beta2, eps, step, bias_co
     f32 = torch.float32
     step_size, sbc2 = host_constants(lr, beta1, beta2, step, bias_correction)
     m_new, v_new = moments(g, m_q, torch.tensor(inv_m, dtype=f32), v_q, torch.tensor(inv_v, dtype=f32), beta1, beta2)
-    denom = torch.sqrt(v_new) / torch.tensor(sbc2, dtype=f32) + torch.tensor(eps, dtype=f32)
+    denom = _sqrt(v_new) / torch.tensor(sbc2, dtype=f32) + torch.tensor(eps, dtype=f32)
     p_new = p - torch.tensor(step_size, dtype=f32) * (m_new / denom)
     return p_new, m_new.abs().max(), v_new.abs().max()
 

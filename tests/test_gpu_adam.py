@@ -1,0 +1,146 @@
+"""GPU parity of the FP8 AdamW kernels against the CPU oracle: quantized weights and moments within
+one code (1 FP8 ulp) after a step -- in practice bit-equal -- and metas bit-exact."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import adamw as oadam, cast as ocast, fp8
+from tests.gpu_util import same_float
+
+pytestmark = pytest.mark.gpu
+
+HYPER = dict(lr=3e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+
+
+@pytest.fixture(scope='module')
+def be():
+    from msamp import _backend
+    _backend.load()
+    return _backend
+
+
+def _quant(x, fmt):
+    meta = ocast.new_meta()
+    return ocast.cast_to_fp8(x, meta, fmt, in_time=True), meta
+
+
+def _inputs(n, seed, w_fmt, g_fmt, zero_state=False):
+    g = torch.Generator().manual_seed(seed)
+    wf = 0.02 * torch.randn(n, generator=g)
+    if w_fmt == 'f16':
+        wm = ocast.new_meta()
+        w = ocast.cast_to_fp16(wf, wm, in_time=True)
+    else:
+        w, wm = _quant(wf, w_fmt)
+    gq, gm = _quant(1e-3 * torch.randn(n, generator=g), g_fmt)
+    mf = torch.zeros(n) if zero_state else (1e-4 * torch.randn(n, generator=g)).abs()
+    vf = torch.zeros(n) if zero_state else (1e-4 * torch.randn(n, generator=g)).abs()
+    m, mm = _quant(mf, fp8.E4M3)
+    vm = ocast.new_meta()
+    v = ocast.cast_to_fp16(vf, vm, in_time=True)
+    return dict(w=w, wm=wm, g=gq, gm=gm, m=m, mm=mm, v=v, vm=vm)
+
+
+def _dev_meta(meta):
+    return [meta['scale'].clone().cuda().reshape(()), meta['scale_inv'].clone().cuda().reshape(()), meta['amax'].clone().cuda()]
+
+
+def _code_distance(a, b):
+    """Distance in code steps between two FP8 payloads (sign-magnitude order)."""
+    def key(t):
+        t = t.to(torch.int32)
+        return torch.where(t >= 128, -(t - 128), t)
+    return (key(a.cpu()) - key(b.cpu())).abs()
+
+
+def _fused(be, tensors, w_dt, g_dt, step, **kw):
+    """Run msamp_adamw_fp8_fused on a list of tensor dicts; returns device copies of everything."""
+    dev = []
+    rows = []
+    for t in tensors:
+        d = dict(w=t['w'].cuda(), g=t['g'].cuda(), m=t['m'].cuda(), v=t['v'].cuda(), wm=_dev_meta(t['wm']),
+                 gsi=t['gm']['scale_inv'].clone().cuda().reshape(()), mm=_dev_meta(t['mm']), vm=_dev_meta(t['vm']))
+        dev.append(d)
+        rows.append((d['w'].data_ptr(), d['g'].data_ptr(), d['m'].data_ptr(), d['v'].data_ptr(),
+                     d['wm'][0].data_ptr(), d['wm'][1].data_ptr(), d['wm'][2].data_ptr(), d['gsi'].data_ptr(),
+                     d['mm'][0].data_ptr(), d['mm'][1].data_ptr(), d['mm'][2].data_ptr(),
+                     d['vm'][0].data_ptr(), d['vm'][1].data_ptr(), d['vm'][2].data_ptr(), d['w'].numel(), 0, 0, 0, 0))
+    desc = torch.from_numpy(np.asarray(rows, dtype=np.int64)).cuda()
+    chunks = [(t['w'].numel() + be.ADAMW_CHUNK - 1) // be.ADAMW_CHUNK for t in tensors]
+    bm = np.stack([np.repeat(np.arange(len(tensors), dtype=np.int32), chunks),
+                   np.concatenate([np.arange(c, dtype=np.int32) for c in chunks])], axis=1).copy()
+    block_map = torch.from_numpy(bm).cuda()
+    hyper = dict(HYPER)
+    hyper.update(kw)
+    be.adamw_fused(desc, len(tensors), block_map, block_map.shape[0], w_dt, g_dt, hyper['lr'], hyper['beta1'], hyper['beta2'],
+                   hyper['eps'], hyper['weight_decay'], step, hyper.get('bias_correction', True), hyper.get('adam_mode', False),
+                   hyper.get('maximize', False), hyper.get('tensor_scale', True))
+    torch.cuda.synchronize()
+    # the scratch words of the descriptors are left zeroed
+    assert (desc[:, 15].cpu() == 0).all()
+    return dev
+
+
+def _check(dev, t, w_fmt, g_fmt, step, **kw):
+    hyper = dict(HYPER)
+    hyper.update(kw)
+    (w2, wm2, m2, mm2, v2, vm2), _ = oadam.step_tensor(
+        t['w'], t['wm'], w_fmt, t['g'], t['gm']['scale_inv'], g_fmt, t['m'], t['mm'], t['v'], t['vm'], step=step, **hyper
+    )
+    for got, want, name in ((dev['wm'], wm2, 'w'), (dev['mm'], mm2, 'm'), (dev['vm'], vm2, 'v')):
+        assert same_float(got[0], want['scale']), name
+        assert same_float(got[1], want['scale_inv']), name
+        assert same_float(got[2][0], want['amax'][0]), name
+    if w_fmt == 'f16':
+        dw = (dev['w'].cpu().view(torch.int16).int() - w2.view(torch.int16).int()).abs()
+    else:
+        dw = _code_distance(dev['w'], w2)
+    dm = _code_distance(dev['m'], m2)
+    dv = (dev['v'].cpu().view(torch.int16).int() - v2.view(torch.int16).int()).abs()
+    assert dw.max().item() <= 1 and dm.max().item() <= 1 and dv.max().item() <= 1
+    # and almost all of them are bit-equal
+    for d in (dw, dm, dv):
+        assert (d != 0).float().mean().item() < 1e-3
+
+
+@pytest.mark.parametrize('w_fmt,w_dt,g_fmt,g_dt', [(fp8.E4M3, 5, fp8.E5M2, 6), ('f16', 3, fp8.E4M3, 5), (fp8.E5M2, 6, fp8.E4M3, 5)])
+@pytest.mark.parametrize('step,zero_state', [(1, True), (2, False)])
+def test_fused_step_multi_tensor(be, w_fmt, w_dt, g_fmt, g_dt, step, zero_state):
+    sizes = [16384 * 4, 16384 * 2 + 777, 5, 4096 * 1024]
+    tensors = [_inputs(n, 100 + i, w_fmt, g_fmt, zero_state) for i, n in enumerate(sizes)]
+    dev = _fused(be, tensors, w_dt, g_dt, step)
+    for d, t in zip(dev, tensors):
+        _check(d, t, w_fmt, g_fmt, step)
+
+
+@pytest.mark.parametrize('kw', [dict(adam_mode=True), dict(maximize=True), dict(bias_correction=False), dict(weight_decay=0.0),
+                                dict(tensor_scale=False)])
+def test_fused_step_variants(be, kw):
+    t = _inputs(16384 * 3 + 100, 7, fp8.E4M3, fp8.E5M2)
+    dev = _fused(be, [t], 5, 6, 3, **kw)
+    _check(dev[0], t, fp8.E4M3, fp8.E5M2, 3, **kw)
+
+
+def test_fused_step_is_deterministic(be):
+    t = _inputs(16384 * 9, 21, fp8.E4M3, fp8.E5M2)
+    a = _fused(be, [t], 5, 6, 2)[0]
+    b = _fused(be, [t], 5, 6, 2)[0]
+    assert torch.equal(a['w'], b['w']) and torch.equal(a['m'], b['m']) and torch.equal(a['v'], b['v'])
+
+
+def test_stage1_stage2_entry_points(be):
+    n = 100003
+    t = _inputs(n, 33, fp8.E4M3, fp8.E5M2)
+    p0 = fp8.decode(t['w'], fp8.E4M3) * t['wm']['scale_inv']
+    g0 = fp8.decode(t['g'], fp8.E5M2) * t['gm']['scale_inv']
+    inv_m, inv_v = (1.0 / t['mm']['scale']).item(), (1.0 / t['vm']['scale']).item()
+    hyper = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+    p_want, am_want, av_want = oadam.stage1(p0, g0, t['m'], inv_m, t['v'], inv_v, step=4, **hyper)
+    p, g, m, v = p0.cuda(), g0.cuda(), t['m'].cuda(), t['v'].cuda()
+    am, av = torch.zeros(1, device='cuda'), torch.zeros(1, device='cuda')
+    be.adamw_stage1(p, g, m, 5, inv_m, am, 0.9, v, 3, inv_v, av, 0.999, 1e-8, 4, 1e-3, True)
+    assert torch.equal(p.cpu(), p_want) and am.item() == am_want.item() and av.item() == av_want.item()
+    m_want, v_want = oadam.stage2(g0, t['m'], inv_m, 4096.0, t['v'], inv_v, 2.0**20, beta1=0.9, beta2=0.999)
+    be.adamw_stage2(g, m, 5, inv_m, 4096.0, 0.9, v, 3, inv_v, 2.0**20, 0.999)
+    assert torch.equal(m.cpu(), m_want) and torch.equal(v.cpu(), v_want)

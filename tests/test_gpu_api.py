@@ -1,0 +1,269 @@
+"""GPU tests of the msamp API surface on the HIP kernels: the reference's own test ideas
+(tests/common/tensor, tests/nn, tests/optim, tests/test_initialize.py) on this implementation."""
+
+import copy
+import itertools
+from functools import partial
+
+import pytest
+import torch
+
+import msamp
+from msamp.common.dtype import Dtypes
+from msamp.common.tensor import ScalingMeta, ScalingTensor, TypeCast
+from msamp.nn import FP8Linear, LinearReplacer, ScalingParameter, model_state
+from msamp.optim import DSAdam, LBAdam, LBAdamW, LBAdamWBase
+from oracle import cast as ocast, fp8, gemm as ogemm
+from tests.gpu_util import rel_fro, same_float
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _fresh_state():
+    model_state.clear()
+    ScalingMeta.in_time_scaling = True
+    yield
+    model_state.clear()
+
+
+def test_cast_fp8_and_fp16_round_trip():
+    torch.manual_seed(100)
+    x16 = torch.rand((4, 4), dtype=torch.float16, device='cuda')
+    meta = ScalingMeta(Dtypes.kfloat8_e4m3)
+    q = TypeCast.cast_to_fp8(x16, meta)
+    assert q.dtype == torch.uint8 and q.shape == x16.shape
+    assert torch.allclose(x16, TypeCast.cast_from_fp8(q, meta, Dtypes.kfloat16), 0, 0.1)
+    x32 = torch.rand((4, 4), device='cuda')
+    meta = ScalingMeta(Dtypes.kfloat16)
+    h = TypeCast.cast_to_fp16(x32, meta)
+    assert h.dtype == torch.float16
+    assert torch.allclose(x32, TypeCast.cast_from_fp16(h, meta, Dtypes.kfloat32), 0, 1e-3)
+    with pytest.raises(ValueError):
+        TypeCast.cast_from_fp8(x16, meta, Dtypes.kfloat32)
+
+
+def test_scaling_tensor_casts_and_scale_ops():
+    torch.manual_seed(0)
+    x = torch.randn(64, 48, device='cuda') * 1e-3
+    st = x.cast(Dtypes.kfloat16)
+    assert st.dtype == torch.float16 and st.qtype == Dtypes.kfloat16
+    assert torch.allclose(st.float(), x, rtol=2e-3, atol=0)
+    # scaled fp16 -> E4M3 reuses the stored amax: compare with the oracle's recipe bit for bit
+    q = st.cast(Dtypes.kfloat8_e4m3)
+    old = {'scale': st.meta.scale.cpu(), 'scale_inv': st.meta.scale_inv.cpu(), 'amax': st.meta.amax.cpu()}
+    want_q, want_meta = ocast.scaled_fp16_to_fp8(st.value.cpu(), old, fp8.E4M3)
+    assert torch.equal(q.value.cpu(), want_q)
+    assert same_float(q.meta.scale, want_meta['scale']) and same_float(q.meta.scale_inv, want_meta['scale_inv'])
+    assert same_float(q.meta.amax, want_meta['amax'])
+    assert torch.allclose(q.float(), x, rtol=0.07, atol=1e-6)
+    # a tiny value survives fp16 -> E4M3 through the scale
+    tiny = torch.tensor([2.0**-17], device='cuda').cast(Dtypes.kfloat16).cast(Dtypes.kfloat8_e4m3)
+    assert tiny.float().item() == 2.0**-17
+    # mul_/div_ act on scale_inv only
+    before = q.value.clone()
+    q.mul_(2.0)
+    assert torch.equal(q.value, before) and torch.allclose(q.float(), 2 * x, rtol=0.07, atol=1e-6)
+    q.div_(torch.tensor(2.0, device='cuda'))
+    assert torch.allclose(q.float(), x, rtol=0.07, atol=1e-6)
+    # fused cast+transpose equals cast then transpose
+    a, at = x.fused_cast_transpose(Dtypes.kfloat8_e4m3)
+    b = x.cast(Dtypes.kfloat8_e4m3)
+    assert torch.equal(a.value, b.value) and torch.equal(at.value, b.fp8_transpose().value)
+    assert torch.equal(at.value, b.value.t().contiguous())
+    # non-finite input shows in amax
+    bad = torch.tensor([1.0, float('nan')], device='cuda').cast(Dtypes.kfloat8_e4m3)
+    assert bad.has_inf_or_nan() and not b.has_inf_or_nan()
+    assert b.half().dtype == torch.float16 and b.bfloat16().dtype == torch.bfloat16 and b.to(torch.float32).dtype == torch.float32
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+def test_fp8linear_against_nn_linear(dtype):
+    torch.manual_seed(1000)
+    lin = torch.nn.Linear(32, 16).cuda().to(dtype)
+    ref = copy.deepcopy(lin)
+    model = LinearReplacer.replace(lin, Dtypes.kfloat16)
+    assert isinstance(model, FP8Linear) and isinstance(model.weight, ScalingParameter)
+    x = torch.randn(8, 4, 32, device='cuda', dtype=dtype, requires_grad=True)
+    x2 = x.detach().clone().requires_grad_(True)
+    y, y2 = model(x), ref(x2)
+    assert y.dtype == dtype and y.shape == y2.shape
+    assert torch.allclose(y.float(), y2.float(), 0, 0.1)
+    y.sum().backward()
+    y2.sum().backward()
+    assert torch.allclose(x.grad.float(), x2.grad.float(), 0, 0.1)
+    assert torch.equal(model.bias.grad, ref.bias.grad)
+    assert isinstance(model.weight.grad, ScalingTensor) and model.weight.grad.qtype == Dtypes.kfloat8_e4m3
+    assert torch.allclose(model.weight.grad.float(), ref.weight.grad.float(), 0.07, 0.5)    # FP8 inputs, E4M3 storage
+
+
+def test_fp8linear_autocast_and_grad_accumulation():
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(16, 16).cuda()
+    model = LinearReplacer.replace(copy.deepcopy(lin), Dtypes.kfloat16)
+    x = torch.randn(8, 16, device='cuda')
+    with torch.autocast('cuda', dtype=torch.bfloat16):
+        assert model(x).dtype == torch.bfloat16
+    full = LinearReplacer.replace(copy.deepcopy(lin), Dtypes.kfloat16)
+    full(x).sum().backward()
+    for part in x.chunk(2):
+        model(part).sum().backward()
+    assert torch.allclose(model.weight.grad.float(), full.weight.grad.float(), 0.14, 0.5)
+
+
+def test_flattened_metas_are_checked():
+    model = LinearReplacer.replace(torch.nn.Linear(8, 8).cuda(), Dtypes.kfloat16)
+    x = torch.randn(4, 8, device='cuda')
+    model(x)
+    model.scaling_metas['input'].scale = torch.ones((), device='cuda')
+    with pytest.raises(RuntimeError):
+        model(x)
+
+
+def test_fp8linear_step_against_oracle_pipeline():
+    """x, W, dy -> casts (in-time warm-up), three GEMMs: y and dx against the oracle's casts + fp32-class GEMM."""
+    torch.manual_seed(5)
+    tokens, d_in, d_out = 256, 128, 192
+    lin = torch.nn.Linear(d_in, d_out, bias=False).cuda().bfloat16()
+    w_ref = lin.weight.detach().cpu()
+    model = LinearReplacer.replace(lin, Dtypes.kbfloat16)
+    x = torch.randn(tokens, d_in, device='cuda', dtype=torch.bfloat16, requires_grad=True)
+    dy = (torch.randn(tokens, d_out, device='cuda') * 1e-3).bfloat16()
+    y = model(x)
+    y.backward(dy)
+    xm, wm, gm = ocast.new_meta(), ocast.new_meta(), ocast.new_meta()
+    xq = ocast.cast_to_fp8(x.detach().cpu(), xm, fp8.E4M3, in_time=True)
+    wq = ocast.cast_to_fp8(w_ref, wm, fp8.E4M3, in_time=True)
+    gq = ocast.cast_to_fp8(dy.cpu(), gm, fp8.E5M2, in_time=True)
+    y_want = ogemm.fp8_gemm(wq, wm['scale_inv'], fp8.E4M3, xq, xm['scale_inv'], fp8.E4M3)
+    dx_want = ogemm.fp8_gemm(wq.t().contiguous(), wm['scale_inv'], fp8.E4M3, gq, gm['scale_inv'], fp8.E5M2)
+    dw_want = ogemm.fp8_gemm(xq.t().contiguous(), xm['scale_inv'], fp8.E4M3, gq.t().contiguous(), gm['scale_inv'], fp8.E5M2)
+    assert rel_fro(y.float(), y_want) < 1e-2 and rel_fro(x.grad.float(), dx_want) < 1e-2
+    assert rel_fro(model.weight.grad.float(), dw_want) < 0.05    # E4M3 storage of the weight gradient
+    metas = model.scaling_metas
+    assert same_float(metas['input'].amax[0], xm['amax'][0]) and same_float(metas['input'].scale, xm['scale'])
+    assert same_float(metas['ograd'].amax[0], gm['amax'][0]) and same_float(metas['ograd'].scale, gm['scale'])
+
+
+def _check_optimizer_step(torch_cls, lb_cls, diff=3e-4):
+    x = torch.randn(4, 4, device='cuda')
+    linear = torch.nn.Linear(4, 4).cuda()
+    wd, steps = 1e-3, 4
+    m1 = copy.deepcopy(linear)
+    o1 = torch_cls(m1.parameters(), weight_decay=wd)
+    for _ in range(steps):
+        m1(x).sum().backward()
+        o1.step()
+        o1.zero_grad()
+    model_state.clear()
+    m2 = LinearReplacer.replace(copy.deepcopy(linear), Dtypes.kfloat16)
+    o2 = lb_cls(m2.parameters(), weight_decay=wd)
+    for _ in range(steps):
+        m2(x).sum().backward()
+        o2.all_reduce_grads(m2)
+        o2.step()
+        o2.zero_grad()
+    assert torch.allclose(m1.weight, m2.weight.float(), 0, diff)
+    assert torch.allclose(m1.bias, m2.bias.float(), 0, diff)
+
+
+def test_optimizers_track_torch_adamw():
+    torch.manual_seed(100)
+    dtypes = [torch.uint8, torch.float16]
+    pairs = list(itertools.product(dtypes, dtypes)) + [(torch.float32, torch.float32)]
+    for m_dt, v_dt in pairs:
+        kw = dict(exp_avg_dtype=m_dt, exp_avg_sq_dtype=v_dt)
+        _check_optimizer_step(torch.optim.AdamW, partial(LBAdamWBase, **kw))
+        _check_optimizer_step(torch.optim.AdamW, partial(LBAdamW, **kw))
+        _check_optimizer_step(torch.optim.AdamW, partial(DSAdam, **kw))
+        _check_optimizer_step(torch.optim.Adam, partial(LBAdam, **kw))
+
+
+def test_historical_window_quantization():
+    model = LinearReplacer.replace(torch.nn.Linear(4, 8).cuda(), Dtypes.kfloat16)
+    opt = LBAdamW(model.parameters())
+    window = []
+    for i in list(range(17)) * 6:
+        x = torch.full((1, 4), float(i), device='cuda')
+        window = (window + [i])[-16:]
+        y = model(x)
+        assert model.scaling_metas['input'].amax.max().item() == max(window)
+        y.sum().backward()
+        opt.all_reduce_grads(model)
+        opt.step()
+    assert model.scaling_metas['input'].amax_counter.item() == 17 * 6
+    assert not model.scaling_metas['input'].is_in_time_scaling()
+
+
+def test_optimizer_state_dict_round_trip():
+    torch.manual_seed(7)
+    x = torch.randn(4, 4, device='cuda')
+    linear = torch.nn.Linear(4, 4).cuda()
+    m1 = LinearReplacer.replace(copy.deepcopy(linear), Dtypes.kfloat16)
+    o1 = LBAdamW(m1.parameters())
+    for _ in range(2):
+        m1(x).sum().backward()
+        o1.step()
+        o1.zero_grad()
+    sd = o1.state_dict()
+    assert set(sd) == {'state', 'param_groups'} and set(sd['state']) == {0, 1}
+    st = sd['state'][0]
+    assert st['step'] == 2 and isinstance(st['exp_avg'], ScalingTensor) and st['exp_avg'].dtype == torch.uint8
+    assert isinstance(st['exp_avg_sq'], ScalingTensor) and st['exp_avg_sq'].dtype == torch.float16
+    m2 = LinearReplacer.replace(copy.deepcopy(linear), Dtypes.kfloat16)    # re-flattens m1's metas too
+    m2.weight.copy_(m1.weight)
+    m2.bias.data.copy_(m1.bias.data)
+    o2 = LBAdamW(m2.parameters())
+    o2.load_state_dict(copy.deepcopy(sd))
+    # metas of the two models must see the same history for the runs to stay equal
+    for k in ('input', 'wgrad', 'ograd'):
+        m2.scaling_metas[k].copy_(m1.scaling_metas[k])
+    for m, o in ((m1, o1), (m2, o2)):
+        m(x).sum().backward()
+        o.step()
+    assert torch.equal(m1.weight.value, m2.weight.value)
+    assert torch.equal(o1.state[m1.weight]['exp_avg'].value, o2.state[m2.weight]['exp_avg'].value)
+
+
+@pytest.mark.parametrize('opt_level', ['O1', 'O2'])
+def test_initialize_and_train(opt_level):
+    torch.manual_seed(11)
+    model = torch.nn.Sequential(torch.nn.Linear(32, 64), torch.nn.ReLU(), torch.nn.Linear(64, 16)).cuda()
+    model[2].use_fp32_linear = False
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-2, weight_decay=0.01)
+    model, opt = msamp.initialize(model, opt, opt_level=opt_level)
+    assert isinstance(opt, LBAdamW) and all(isinstance(m, FP8Linear) for m in (model[0], model[2]))
+    assert opt.exp_avg_dtype == (torch.uint8 if opt_level == 'O2' else torch.float32)
+    assert [type(p) for p in opt.param_groups[0]['params']] == [ScalingParameter, torch.nn.Parameter] * 2
+    x = torch.randn(64, 32, device='cuda')
+    target = torch.randn(64, 16, device='cuda')
+    losses = []
+    for _ in range(30):
+        loss = torch.nn.functional.mse_loss(model(x), target)
+        loss.backward()
+        msamp.clip_grad_norm_(model.parameters(), 10.0)
+        opt.step()
+        opt.zero_grad()
+        losses.append(loss.item())
+    assert losses[-1] < 0.7 * losses[0]
+    st = opt.state[model[0].weight]
+    if opt_level == 'O2':
+        assert st['exp_avg'].dtype == torch.uint8 and st['exp_avg_sq'].dtype == torch.float16
+    model_state.clear()
+    lin = torch.nn.Linear(4, 4).cuda()
+    _, adam_opt = msamp.initialize(lin, torch.optim.Adam(lin.parameters()), opt_level=opt_level)
+    assert isinstance(adam_opt, LBAdam) and adam_opt.use_adam
+
+
+def test_grad_scaler_unscale_with_scaling_tensor_grads():
+    model = LinearReplacer.replace(torch.nn.Linear(8, 8).cuda(), Dtypes.kfloat16)
+    x = torch.randn(4, 8, device='cuda')
+    (model(x).sum() * 128.0).backward()
+    g = model.weight.grad
+    before = g.float().clone()
+    found = torch.zeros(1, device='cuda')
+    torch._amp_foreach_non_finite_check_and_unscale_([g, model.bias.grad], found, torch.tensor(1 / 128.0, device='cuda'))
+    assert found.item() == 0 and torch.allclose(g.float(), before / 128.0)
+    g.meta.amax[0] = float('inf')
+    torch._amp_foreach_non_finite_check_and_unscale_([g], found, torch.tensor(1.0, device='cuda'))
+    assert found.item() == 1

@@ -1,0 +1,228 @@
+"""GPU parity of the cast group against the CPU oracle: bytes, amax, scale and scale_inv bit-exact.
+All calls go through the C ABI (msamp._backend)."""
+
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import cast as ocast, fp8, scaling
+from tests.gpu_util import FMT, c1_input, make_meta, oracle_meta, same_float
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), 'golden', 'reference_kats.json')))
+
+
+@pytest.fixture(scope='module')
+def be():
+    from msamp import _backend
+    _backend.load()
+    return _backend
+
+
+@pytest.mark.parametrize('fp8_dt', [5, 6])
+@pytest.mark.parametrize('src', [torch.float16, torch.bfloat16])
+def test_quantize_every_16bit_pattern(be, fp8_dt, src):
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(src)
+    for scale in (1.0, 2.0**-7, 2.0**9, 3.0):
+        s, si, am = make_meta(scale=scale)
+        got = be.cast_to_fp8(x.cuda(), s, None, si, fp8_dt).cpu()
+        want = fp8.encode(x.float() * torch.tensor(scale), FMT[fp8_dt])
+        assert torch.equal(got, want), (fp8_dt, src, scale, (got != want).sum().item())
+        assert si.item() == (torch.tensor(1.0) / torch.tensor(scale)).item()
+
+
+@pytest.mark.parametrize('fp8_dt', [5, 6])
+def test_quantize_fp32_fine_grid_and_specials(be, fp8_dt):
+    # every float32 whose low 12 mantissa bits are a fixed pattern, across all exponents the format resolves
+    hi = torch.arange(0, 1 << 20, dtype=torch.int64)
+    bits = ((hi << 12) | 0x7ff).to(torch.int32)    # wraps into negative values too
+    x = bits.view(torch.float32)
+    s, si, am = make_meta(scale=1.0)
+    got = be.cast_to_fp8(x.cuda(), s, None, None, fp8_dt).cpu()
+    want = fp8.encode(x, FMT[fp8_dt])
+    assert torch.equal(got, want)
+    fmax = fp8.FP_MAX[FMT[fp8_dt]]
+    sp = torch.tensor([float('nan'), -float('nan'), float('inf'), -float('inf'), fmax, fmax * 1.03, fmax * 1.07, -fmax * 4, 0.0, -0.0, 1e-30])
+    got = be.cast_to_fp8(sp.cuda(), s, None, None, fp8_dt).cpu()
+    assert torch.equal(got, fp8.encode(sp, FMT[fp8_dt]))
+
+
+@pytest.mark.parametrize('fp8_dt', [5, 6])
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.float16, torch.bfloat16])
+def test_dequantize_all_codes(be, fp8_dt, out_dtype):
+    codes = torch.arange(256, dtype=torch.uint8).repeat(67)    # vector body + scalar tail
+    for si_val in (1.0, 1 / 32, 3.0):
+        si = torch.full((), si_val, device='cuda')
+        got = be.cast_from_fp8(codes.cuda(), si, fp8_dt, out_dtype).cpu()
+        want = ocast.cast_from_fp8(codes, torch.tensor(si_val), FMT[fp8_dt], out_dtype)
+        assert same_float(got, want)
+
+
+def test_scale_rule_known_answers_and_adversarial(be):
+    k = GOLDEN['scaling_factor']
+    for c in k['cases']:
+        out = be.compute_scaling_factor(torch.tensor([c['amax']], device='cuda'), torch.tensor([c['scale']], device='cuda'), k['fp_max'], k['margin'])
+        assert out.item() == c['expected']
+    vals = [0.0, -0.0, -1.0, float('inf'), float('nan'), 1e-45, 1e-42, 1e-38, 3.4e38, 448.0, 449.0, 224.0, 57344.0, 65504.0]
+    for fp_max in (448.0, 57344.0, 65504.0):
+        for kexp in range(-40, 41):
+            base = torch.tensor(fp_max * 2.0**kexp, dtype=torch.float32)
+            for _ in range(6):    # amax just around every power-of-two boundary of fp_max/amax
+                vals.append(base.item())
+                base = torch.nextafter(base, torch.tensor(float('inf')))
+            base = torch.tensor(fp_max * 2.0**kexp, dtype=torch.float32)
+            for _ in range(6):
+                base = torch.nextafter(base, torch.tensor(0.0))
+                vals.append(base.item())
+    g = torch.Generator().manual_seed(1)
+    amax = torch.cat([torch.tensor(vals, dtype=torch.float32), torch.exp(torch.rand(50000, generator=g) * 80 - 40)])
+    scale = torch.full_like(amax, 3.0)
+    for fp_max in (448.0, 57344.0, 65504.0):
+        for margin in (0, 2):
+            got = be.compute_scaling_factor(amax.cuda(), scale.cuda(), fp_max, margin).cpu()
+            want = scaling.compute_scaling_factor(amax, scale, fp_max, margin)
+            assert same_float(got, want), (fp_max, margin, amax[(got != want) & ~(got.isnan() & want.isnan())][:8])
+    # one-element fallback scale broadcasts
+    got = be.compute_scaling_factor(amax.cuda(), torch.tensor([3.0], device='cuda'), 448.0, 0).cpu()
+    assert same_float(got, scaling.compute_scaling_factor(amax, torch.tensor(3.0), 448.0, 0))
+
+
+@pytest.mark.parametrize('fp8_dt', [5, 6])
+def test_config1_in_time_cast_full_size(be, fp8_dt):
+    x = c1_input(seed=0)
+    s, si, am = make_meta()
+    q = be.cast_to_fp8_intime(x.cuda(), s, am[0:1], si, fp8_dt)
+    om = oracle_meta()
+    want = ocast.cast_to_fp8(x, om, FMT[fp8_dt], in_time=True)
+    assert torch.equal(q.cpu(), want)
+    assert same_float(am[0], om['amax'][0]) and same_float(s, om['scale']) and same_float(si, om['scale_inv'])
+    back = be.cast_from_fp8(q, si, fp8_dt, torch.float32).cpu()
+    assert torch.equal(back, ocast.cast_from_fp8(want, om['scale_inv'], FMT[fp8_dt]))
+    # run to run determinism
+    s2, si2, am2 = make_meta()
+    q2 = be.cast_to_fp8_intime(x.cuda(), s2, am2[0:1], si2, fp8_dt)
+    assert torch.equal(q, q2) and am2[0].item() == am[0].item()
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('n', [1, 3, 1000, 4097, 16384 * 3 + 5, 1 << 20])
+def test_in_time_cast_ragged_sizes(be, dtype, n):
+    g = torch.Generator().manual_seed(n)
+    x = (torch.randn(n + 1, generator=g) * 3).to(dtype)
+    xg = x.cuda()
+    for off, fp8_dt in ((0, 5), (1, 6)):    # offset 1 makes the device view misaligned for vector loads
+        view = x[off:off + n]
+        s, si, am = make_meta()
+        q = be.cast_to_fp8_intime(xg[off:off + n], s, am[0:1], si, fp8_dt)
+        om = oracle_meta()
+        want = ocast.cast_to_fp8(view, om, FMT[fp8_dt], in_time=True)
+        assert torch.equal(q.cpu(), want)
+        assert same_float(am[0], om['amax'][0]) and same_float(s, om['scale']) and same_float(si, om['scale_inv'])
+
+
+def test_delayed_cast_accumulates_amax_and_skips_nan(be):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(100000, generator=g).to(torch.bfloat16)
+    x[17] = float('nan')
+    s, si, am = make_meta(window=4, scale=16.0)
+    om = oracle_meta(window=4, scale=16.0)
+    for mult in (1.0, 4.0, 0.5):
+        xm = x * mult    # formed once on the host so both sides see identical bits (NaN included)
+        q = be.cast_to_fp8(xm.cuda(), s, am[0:1], si, 5)
+        want = ocast.cast_to_fp8(xm, om, fp8.E4M3, in_time=False)
+        assert torch.equal(q.cpu(), want)
+        assert same_float(am, om['amax']) and s.item() == 16.0 and si.item() == 1 / 16
+    assert q.cpu()[17].item() & 0x7F == 0x7F
+
+
+def test_in_time_nan_inf_and_sync_semantics(be):
+    x = torch.tensor([1.0, float('nan'), -2.0, 0.5] * 300)
+    s, si, am = make_meta(scale=8.0)
+    q = be.cast_to_fp8_intime(x.cuda(), s, am[0:1], si, 5)
+    om = oracle_meta(scale=8.0)
+    want = ocast.cast_to_fp8(x, om, fp8.E4M3, in_time=True)
+    assert torch.isnan(am[0]).item() and s.item() == 8.0 and si.item() == 0.125 and torch.equal(q.cpu(), want)
+    s, si, am = make_meta(scale=8.0)
+    q = be.cast_to_fp8_intime(x.cuda(), s, am[0:1], si, 5, nan_to_inf=True)
+    om = oracle_meta(scale=8.0)
+    want = ocast.cast_to_fp8(x, om, fp8.E4M3, in_time=True, sync=True)
+    assert am[0].item() == float('inf') and s.item() == 0.125 and si.item() == 8.0 and torch.equal(q.cpu(), want)
+    xi = torch.tensor([1.0, float('inf'), -float('inf')] * 100)
+    s, si, am = make_meta(scale=8.0)
+    q = be.cast_to_fp8_intime(xi.cuda(), s, am[0:1], si, 6)
+    om = oracle_meta(scale=8.0)
+    want = ocast.cast_to_fp8(xi, om, fp8.E5M2, in_time=True)
+    assert am[0].item() == float('inf') and same_float(s, om['scale']) and torch.equal(q.cpu(), want)
+    z = torch.zeros(5000)
+    s, si, am = make_meta(scale=4.0)
+    q = be.cast_to_fp8_intime(z.cuda(), s, am[0:1], si, 5)
+    assert am[0].item() == 0.0 and s.item() == 4.0 and si.item() == 0.25 and q.sum().item() == 0
+
+
+@pytest.mark.parametrize('shape', [(64, 64), (100, 36), (17, 5), (1, 130), (257, 1), (512, 1024), (96, 4100)])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+def test_cast_transpose(be, shape, dtype):
+    g = torch.Generator().manual_seed(shape[0] * 7 + shape[1])
+    x = (torch.randn(*shape, generator=g) * 2).to(dtype)
+    # in time, E5M2 (the output-gradient case)
+    s, si, am = make_meta()
+    q, qt = be.cast_transpose(x.cuda(), s, am[0:1], si, 6, in_time=True)
+    om = oracle_meta()
+    want, want_t = ocast.cast_transpose(x, om, fp8.E5M2, in_time=True)
+    assert torch.equal(q.cpu(), want) and torch.equal(qt.cpu(), want_t)
+    assert same_float(am[0], om['amax'][0]) and same_float(s, om['scale']) and same_float(si, om['scale_inv'])
+    # delayed, E4M3
+    s, si, am = make_meta(window=2, scale=4.0)
+    q, qt = be.cast_transpose(x.cuda(), s, am[0:1], si, 5)
+    om = oracle_meta(window=2, scale=4.0)
+    want, want_t = ocast.cast_transpose(x, om, fp8.E4M3, in_time=False)
+    assert torch.equal(q.cpu(), want) and torch.equal(qt.cpu(), want_t)
+    assert same_float(am, om['amax']) and si.item() == 0.25
+    # separate transpose of the payload equals the fused one
+    assert torch.equal(be.fp8_transpose(q), qt)
+
+
+def test_fp8_transpose_is_involution_at_full_size(be):
+    g = torch.Generator().manual_seed(2)
+    q = torch.randint(0, 256, (8192, 4096), dtype=torch.uint8, generator=g).cuda()
+    t = be.fp8_transpose(q)
+    assert t.shape == (4096, 8192) and torch.equal(t, q.t().contiguous())
+    assert torch.equal(be.fp8_transpose(t), q)
+
+
+def test_scaled_16bit_payloads(be):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(70001, generator=g) * 1e-3
+    for out_dtype in (torch.float16, torch.bfloat16, torch.float32):
+        sc = torch.tensor(2.0**14)
+        got = be.scale_cast(x.cuda(), sc.cuda(), out_dtype).cpu()
+        assert same_float(got.float(), (x * sc.view(1)).to(out_dtype).float())
+    big = torch.tensor([70000.0, -70000.0, 1.0]).cuda()
+    assert be.scale_cast(big, torch.ones((), device='cuda'), torch.float16).cpu().tolist() == [float('inf'), -float('inf'), 1.0]
+    am = torch.zeros(1, device='cuda')
+    be.amax(x.cuda().half(), am)
+    assert am.item() == x.half().abs().max().item()
+    be.amax(x.cuda(), am)
+    assert am.item() == x.abs().max().item()
+
+
+def test_window_update_sequence(be):
+    k = GOLDEN['window']
+    w = k['window_size']
+    scales = torch.ones(3, device='cuda')
+    amaxs = torch.zeros(3, w, device='cuda')
+    o_scales, o_amaxs, o_cnt = torch.ones(3), torch.zeros(3, w), torch.zeros(3, dtype=torch.int32)
+    recent = []
+    for step, i in enumerate(list(range(k['inputs_cycle'])) * k['repeats']):
+        cur = torch.tensor([float(i), float(i) * 0.37, float('inf') if step % 11 == 5 else 2.0 * i])
+        amaxs[:, 0] = cur.cuda()
+        o_amaxs[:, 0] = cur
+        recent = (recent + [i])[-w:]
+        assert amaxs[0].max().item() == max(recent)
+        bad = be.scale_update(scales, amaxs, 448.0, 0).cpu().bool()
+        o_bad = scaling.update_scaling_factors(o_scales, o_amaxs, o_cnt, 448.0)
+        assert torch.equal(bad, o_bad) and same_float(scales, o_scales) and same_float(amaxs, o_amaxs)

@@ -1,0 +1,146 @@
+"""GPU parity of the FP8 GEMM: within 1e-2 relative Frobenius error of an fp32-class matmul on the
+dequantized operands (the bar for this path); fp32 output is held to 1e-3
+(the FP8 MFMA aligns the 64 products of a K block to a common exponent with a finite number of bits,
+so heavily cancelling sums are not exact to float32)."""
+
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import fp8, gemm as ogemm
+from tests.gpu_util import FMT, rel_fro
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = json.load(open(os.path.join(os.path.dirname(__file__), 'golden', 'reference_kats.json')))
+TOL_F32, TOL_16 = 1e-3, 1e-2
+
+
+@pytest.fixture(scope='module')
+def be():
+    from msamp import _backend
+    _backend.load()
+    return _backend
+
+
+def _rand_fp8(shape, fp8_dt, seed, spread=1.0):
+    """Random FP8 payload (finite codes) built by quantizing N(0, spread) on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(*shape, generator=g) * spread
+    return fp8.encode(x, FMT[fp8_dt])
+
+
+def _run(be, a, a_dt, a_si, b, b_dt, b_si, out_dtype=torch.float32, accumulate=False, bias=None, out=None):
+    n, m = b.shape[0], a.shape[0]
+    if out is None:
+        out = torch.empty(n, m, dtype=out_dtype, device='cuda')
+    be.fp8_gemm(a.cuda(), a_dt, torch.tensor(a_si, device='cuda'), b.cuda(), b_dt, torch.tensor(b_si, device='cuda'), out,
+                accumulate, None if bias is None else bias.cuda())
+    return out
+
+
+def test_reference_ones_case_through_api():
+    import msamp    # noqa: F401
+    from msamp.common.dtype import Dtypes
+    from msamp.operators.gemm import Gemm
+    k = GOLDEN['gemm_ones']
+    ta = torch.ones(k['a_shape'], device='cuda')
+    tb = torch.ones(k['b_shape'], device='cuda')
+    sa, sb = ta.cast(Dtypes.kfloat8_e4m3), tb.cast(Dtypes.kfloat8_e4m3)
+    out = Gemm.fp8_gemm(sa, sb, Dtypes.kfloat32)
+    assert list(out.shape) == k['out_shape'] and out.equal(torch.matmul(tb, ta.t())) and (out == k['value']).all()
+    out = torch.ones(k['out_shape'], device='cuda')
+    out = Gemm.fp8_gemm(sa, sb, Dtypes.kfloat32, out=out)
+    assert (out == k['value']).all()
+
+
+@pytest.mark.parametrize('a_dt,b_dt', [(5, 5), (5, 6), (6, 5), (6, 6)])
+@pytest.mark.parametrize('m,n,k', [(32, 32, 64), (128, 128, 128), (256, 256, 256), (300, 200, 384), (1, 1, 16), (33, 65, 48),
+                                   (512, 384, 1040), (129, 257, 144)])
+def test_random_against_oracle(be, a_dt, b_dt, m, n, k):
+    a = _rand_fp8((m, k), a_dt, 1000 + m + k)
+    b = _rand_fp8((n, k), b_dt, 2000 + n + k)
+    a_si, b_si = 0.125, 2.0
+    want = ogemm.fp8_gemm(a, torch.tensor(a_si), FMT[a_dt], b, torch.tensor(b_si), FMT[b_dt])
+    got = _run(be, a, a_dt, a_si, b, b_dt, b_si)
+    assert rel_fro(got, want) < TOL_F32
+    got16 = _run(be, a, a_dt, a_si, b, b_dt, b_si, out_dtype=torch.bfloat16)
+    assert rel_fro(got16.float(), want) < TOL_16
+
+
+def test_orientation_probe(be):
+    """One-hot rows: out[n, m] must pair row n of b with row m of a."""
+    m, n, k = 70, 40, 64
+    a = torch.zeros(m, k)
+    b = torch.zeros(n, k)
+    for i in range(m):
+        a[i, i % k] = 1.0 + (i % 7)
+    for j in range(n):
+        b[j, (3 * j) % k] = 1.0 + (j % 5)
+    aq, bq = fp8.encode(a, fp8.E4M3), fp8.encode(b, fp8.E4M3)
+    got = _run(be, aq, 5, 1.0, bq, 5, 1.0).cpu()
+    assert torch.equal(got, b @ a.t())
+
+
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.float16, torch.bfloat16])
+def test_accumulate_and_bias(be, out_dtype):
+    m, n, k = 192, 136, 256
+    a, b = _rand_fp8((m, k), 5, 1), _rand_fp8((n, k), 6, 2, spread=0.01)
+    g = torch.Generator().manual_seed(3)
+    prev = torch.randn(n, m, generator=g).to(out_dtype)
+    bias = torch.randn(m, generator=g).to(out_dtype)
+    want = ogemm.fp8_gemm(a, torch.tensor(0.5), fp8.E4M3, b, torch.tensor(4.0), fp8.E5M2, out=prev.float(), bias=bias.float())
+    got = _run(be, a, 5, 0.5, b, 6, 4.0, accumulate=True, bias=bias, out=prev.cuda().clone())
+    assert rel_fro(got.float(), want) < (TOL_F32 if out_dtype == torch.float32 else TOL_16)
+
+
+def test_k_not_multiple_of_16_is_padded_by_the_operator():
+    import msamp    # noqa: F401
+    from msamp.common.dtype import Dtypes
+    from msamp.operators.gemm import Gemm
+    g = torch.Generator().manual_seed(4)
+    ta, tb = torch.randn(5, 7, generator=g).cuda(), torch.randn(3, 7, generator=g).cuda()
+    sa, sb = ta.cast(Dtypes.kfloat8_e4m3), tb.cast(Dtypes.kfloat8_e5m2)
+    out = Gemm.fp8_gemm(sa, sb, Dtypes.kfloat32)
+    want = sb.float() @ sa.float().t()
+    assert out.shape == (3, 5) and rel_fro(out, want) < TOL_F32
+
+
+def test_bad_arguments_raise(be):
+    a = torch.zeros(16, 24, dtype=torch.uint8, device='cuda')
+    si = torch.ones((), device='cuda')
+    with pytest.raises(RuntimeError):
+        be.fp8_gemm(a, 5, si, a, 5, si, torch.empty(16, 16, device='cuda'))    # K % 16 != 0
+    with pytest.raises(ValueError):
+        be.fp8_gemm(a, 5, si, a, 5, si, torch.empty(8, 16, device='cuda'))    # wrong output shape
+
+
+def test_config2_fp8linear_shapes_sampled(be):
+    """The three GEMMs of one FP8Linear step at x[8192,4096], W[4096,4096]: forward, dgrad, wgrad.
+    Checked on a sample of output rows/columns against the oracle, plus linearity in the scale."""
+    tokens, d_in, d_out = 8192, 4096, 4096
+    x = _rand_fp8((tokens, d_in), 5, 11)
+    w = _rand_fp8((d_out, d_in), 5, 12, spread=0.02 * 64)
+    dy = _rand_fp8((tokens, d_out), 6, 13)
+    xs, ws, dys = 1 / 64., 1 / 4096., 2.0**-16
+    rows = torch.tensor([0, 1, 255, 256, 4095, 4096, 8191])
+    cols = torch.tensor([0, 31, 32, 1000, 4095])
+    # forward: y[tokens, d_out] = x W^T  -> a = W, b = x
+    y = _run(be, w, 5, ws, x, 5, xs, out_dtype=torch.bfloat16)
+    want = ogemm.fp8_gemm(w[cols], torch.tensor(ws), fp8.E4M3, x[rows], torch.tensor(xs), fp8.E4M3)
+    assert rel_fro(y[rows.cuda()][:, cols.cuda()].float(), want) < TOL_16
+    # dgrad: dx[tokens, d_in] = dy W -> a = W^T[d_in, d_out], b = dy
+    wt = w.t().contiguous()
+    dx = _run(be, wt, 5, ws, dy, 6, dys, out_dtype=torch.bfloat16)
+    want = ogemm.fp8_gemm(wt[cols], torch.tensor(ws), fp8.E4M3, dy[rows], torch.tensor(dys), fp8.E5M2)
+    assert rel_fro(dx[rows.cuda()][:, cols.cuda()].float(), want) < TOL_16
+    # wgrad: dW[d_out, d_in] = dy^T x -> a = x^T[d_in, tokens], b = dy^T[d_out, tokens]
+    xt, dyt = x.t().contiguous(), dy.t().contiguous()
+    dw = _run(be, xt, 5, xs, dyt, 6, dys, out_dtype=torch.float32)
+    r2 = torch.tensor([0, 1, 2047, 4095])
+    want = ogemm.fp8_gemm(xt[cols], torch.tensor(xs), fp8.E4M3, dyt[r2], torch.tensor(dys), fp8.E5M2)
+    assert rel_fro(dw[r2.cuda()][:, cols.cuda()], want) < TOL_F32
+    dw2 = _run(be, xt, 5, 2 * xs, dyt, 6, dys, out_dtype=torch.float32)
+    assert torch.equal(dw2, 2 * dw)
