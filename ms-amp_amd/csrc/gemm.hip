@@ -10,6 +10,8 @@
 // workgroups of one XCD (one L2) work on neighbouring tiles.
 #include "common.cuh"
 
+#include <type_traits>
+
 namespace msamp {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -130,8 +132,16 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
     TileLoader<BR, KGUARD> lx;
     TileLoader<BC, KGUARD> ly;
     const int nk = (K + kBK - 1) / kBK;
-    lx.gload(X, row0, NR, K, 0);
-    ly.gload(Y, col0, NC, K, 0);
+    // Every row of a tile is K bytes apart, so with a power-of-two K all rows of one K slice sit in
+    // the same memory channel; workgroups therefore walk the K slices in rotated order, each
+    // starting at a different slice, instead of all hammering one channel at a time.
+    const int k_rot = (tr * 7 + tc * 3 + (blockIdx.x >> 3)) % nk;
+    auto slice = [&](int kt) {
+        int s = kt + k_rot;
+        return (s >= nk ? s - nk : s) * kBK;
+    };
+    lx.gload(X, row0, NR, K, slice(0));
+    ly.gload(Y, col0, NC, K, slice(0));
     lx.lstore(smem);
     ly.lstore(smem + BR * kBK);
     __syncthreads();
@@ -140,8 +150,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
         const uint8_t* sx = smem + (kt & 1) * kStage;
         const uint8_t* sy = sx + BR * kBK;
         if (kt + 1 < nk) {
-            lx.gload(X, row0, NR, K, (kt + 1) * kBK);
-            ly.gload(Y, col0, NC, K, (kt + 1) * kBK);
+            lx.gload(X, row0, NR, K, slice(kt + 1));
+            ly.gload(Y, col0, NC, K, slice(kt + 1));
         }
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -182,6 +192,230 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
     }
 }
 
+
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+// one 16-byte chunk of an output row, element by element: ragged right edge, bias, accumulate
+template <typename OT>
+__device__ __noinline__ void store_chunk_slow(OT* out, uint4 val, int gcol, int NC, int accumulate, const void* bias,
+                                              int bias_dt) {
+    constexpr int kEsz = static_cast<int>(sizeof(OT));
+    constexpr int kElems = 16 / kEsz;
+    for (int e = 0; e < kElems; ++e) {
+        if (gcol + e >= NC) break;
+        const int wi = e * kEsz / 4;
+        const uint32_t word = wi == 0 ? val.x : (wi == 1 ? val.y : (wi == 2 ? val.z : val.w));
+        float v;
+        if constexpr (kEsz == 4) {
+            v = __uint_as_float(word);
+        } else if constexpr (__is_same(OT, bf16_t)) {
+            v = bf16_bits_to_float((word >> ((e & 1) * 16)) & 0xffffu);
+        } else {
+            v = f16_bits_to_float((word >> ((e & 1) * 16)) & 0xffffu);
+        }
+        if (bias != nullptr) v += load_bias(bias, bias_dt, gcol + e);
+        store_out<OT>(out + e, v, accumulate != 0);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Main kernel: 256 x 256 x 128 tile, four wavefronts each owning a 128 x 128 quadrant (256 fp32
+// accumulators per lane in the accumulation registers).  Tiles travel global -> LDS with the
+// direct-to-LDS load (no staging registers, no LDS store instructions); two LDS stages; fragments are
+// double-buffered in registers so that the LDS reads of the next 64-byte K sub-step are in flight
+// while the 16 MFMAs of the current one execute.  One workgroup barrier per 128-byte K slice, placed
+// between the two sub-steps; the loads for slice kt+2 are issued right after it.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+constexpr int kDmaTile = 256;
+constexpr int kDmaStage = 2 * kDmaTile * kBK;    // X + Y slice: 64 KiB
+
+__device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }    // vmcnt(0), others unbounded
+
+template <int XF, int YF, typename OT>
+__global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
+                                                                     const uint8_t* __restrict__ Y, OT* __restrict__ D,
+                                                                     int NR, int NC, int K,
+                                                                     const float* __restrict__ x_scale_inv,
+                                                                     const float* __restrict__ y_scale_inv, int accumulate,
+                                                                     const void* __restrict__ bias, int bias_dt) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    int tr, tc;
+    tile_of_block((NR + kDmaTile - 1) / kDmaTile, (NC + kDmaTile - 1) / kDmaTile, tr, tc);
+    const int row0 = tr * kDmaTile, col0 = tc * kDmaTile;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wr = wave >> 1, wc = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    // ---- global -> LDS: one wave instruction fills 8 rows x 128 bytes (1 KiB, lane-contiguous).
+    // Lane l lands in row l/8, 16-byte slot l%8 and therefore fetches the logical chunk
+    // slot ^ swizzle(row); rows past the end of the matrix are clamped to its last row.
+    const int chunk = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
+    uint32_t xoff[8], yoff[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = (i * 4 + wave) * 8 + (lane >> 3);
+        int gx = row0 + r, gy = col0 + r;
+        gx = gx < NR ? gx : NR - 1;
+        gy = gy < NC ? gy : NC - 1;
+        xoff[i] = static_cast<uint32_t>(gx) * static_cast<uint32_t>(K) + chunk * 16;
+        yoff[i] = static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
+    }
+    auto issue = [&](int kt, int stage) {
+        const uint8_t* xk = X + static_cast<size_t>(kt) * kBK;
+        const uint8_t* yk = Y + static_cast<size_t>(kt) * kBK;
+        uint8_t* sx = smem + stage * kDmaStage + wave * 1024;
+        uint8_t* sy = sx + kDmaTile * kBK;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(xk + xoff[i]), (lds_ptr_t)(sx + i * 4096), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(yk + yoff[i]), (lds_ptr_t)(sy + i * 4096), 16, 0, 0);
+        }
+    };
+
+    // ---- LDS -> fragments.  Row of this lane inside a 32-row block and its swizzled chunk offsets.
+    const int fsw = (lane & 7) ^ ((lane >> 3) & 1);
+    const int off_a = ((2 * lh) ^ fsw) << 4;    // sub-step 0, first 16 bytes; second is ^16; sub-step 1 is ^64
+    const int xrow = (wr * 128 + l32) * kBK;
+    const int yrow = kDmaTile * kBK + (wc * 128 + l32) * kBK;
+    auto load_frags = [&](int stage, int ks, v8i* fx, v8i* fy) {
+        const uint8_t* base = smem + stage * kDmaStage;
+        const int o0 = off_a ^ (ks * 64), o1 = o0 ^ 16;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const v4i lo = *reinterpret_cast<const v4i*>(base + xrow + i * 32 * kBK + o0);
+            const v4i hi = *reinterpret_cast<const v4i*>(base + xrow + i * 32 * kBK + o1);
+            fx[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const v4i lo = *reinterpret_cast<const v4i*>(base + yrow + j * 32 * kBK + o0);
+            const v4i hi = *reinterpret_cast<const v4i*>(base + yrow + j * 32 * kBK + o1);
+            fy[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    };
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row l%32,
+    // four consecutive D columns per register quad -- the layout the epilogue wants.
+    auto mfma_block = [&](const v8i* fx, const v8i* fy) {
+        constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
+        constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fy[j], fx[i], acc[i][j], cb, bl, 0, 0, 0, 0);
+    };
+
+    const int nk = K / kBK;
+    v8i fx0[4], fy0[4], fx1[4], fy1[4];
+    issue(0, 0);
+    if (nk > 1) {
+        issue(1, 1);
+        __builtin_amdgcn_s_waitcnt(0x4F70);    // vmcnt(16): the 16 loads of slice 0 have landed
+    } else {
+        wait_vmcnt0();
+    }
+    __syncthreads();
+    load_frags(0, 0, fx0, fy0);
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        load_frags(cur, 1, fx1, fy1);
+        mfma_block(fx0, fy0);
+        wait_vmcnt0();    // slice kt+1 (issued one barrier ago) has landed
+        __syncthreads();  // ... for every wave, and every wave holds slice kt in registers
+        if (kt + 2 < nk) issue(kt + 2, cur);
+        if (kt + 1 < nk) load_frags(cur ^ 1, 0, fx0, fy0);
+        mfma_block(fx1, fy1);
+    }
+    __syncthreads();    // LDS is reused below
+
+    // ---- epilogue: per 32-row block, accumulators -> this wave's LDS patch -> 16-byte row stores
+    constexpr int kEsz = static_cast<int>(sizeof(OT));
+    constexpr int kPitch = 128 * kEsz + 16;    // bytes per patch row (padding staggers the banks)
+    uint8_t* patch = smem + wave * (32 * kPitch);
+    const float alpha = (*x_scale_inv) * (*y_scale_inv);
+    const bool vec_ok = (NC % (16 / kEsz) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
+    const bool plain = vec_ok && !accumulate && bias == nullptr;
+    constexpr int kChunksPerRow = 128 * kEsz / 16;      // 16 (2-byte) or 32 (float)
+    constexpr int kRowsPerPass = 64 / kChunksPerRow;    // 4 or 2
+    constexpr int kElemsPerChunk = 16 / kEsz;           // 8 or 4
+    static_for<4>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        static_for<4>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int c = j * 32 + q * 8 + lh * 4;
+                uint8_t* dst = patch + l32 * kPitch + c * kEsz;
+                const float v0 = acc[i][j][4 * q] * alpha, v1 = acc[i][j][4 * q + 1] * alpha;
+                const float v2 = acc[i][j][4 * q + 2] * alpha, v3 = acc[i][j][4 * q + 3] * alpha;
+                if constexpr (kEsz == 4) {
+                    *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
+                } else if constexpr (__is_same(OT, bf16_t)) {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(float_to_bf16_bits(v0) | (float_to_bf16_bits(v1) << 16),
+                                                                float_to_bf16_bits(v2) | (float_to_bf16_bits(v3) << 16));
+                } else {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(float_to_f16_bits(v0) | (float_to_f16_bits(v1) << 16),
+                                                                float_to_f16_bits(v2) | (float_to_f16_bits(v3) << 16));
+                }
+            }
+        });
+        __builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): the patch is written (same wave reads it back)
+        for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
+            const int pr = pass * kRowsPerPass + lane / kChunksPerRow;
+            const int pc = lane % kChunksPerRow;
+            const int grow = row0 + wr * 128 + i * 32 + pr;
+            const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
+            const uint4 val = *reinterpret_cast<const uint4*>(patch + pr * kPitch + pc * 16);
+            if (grow >= NR || gcol >= NC) continue;
+            OT* out = D + static_cast<size_t>(grow) * NC + gcol;
+            if (plain && gcol + kElemsPerChunk <= NC) {
+                *reinterpret_cast<uint4*>(out) = val;
+            } else {
+                store_chunk_slow<OT>(out, val, gcol, NC, accumulate, bias, bias_dt);
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);    // patch reads done before the next block overwrites it
+    });
+}
+
+template <int XF, int YF, typename OT>
+static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                           const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    constexpr int smem = 2 * kDmaStage;
+    static bool configured = false;
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT>;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel)");
+        configured = true;
+    }
+    const int tiles = ((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys,
+                       accumulate, bias, bias_dt);
+    MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel");
+    return MSAMP_OK;
+}
+
 template <int BR, int BC, int XF, int YF, typename OT, bool KGUARD>
 static int launch_gemm_k(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                        const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
@@ -210,9 +444,13 @@ static int launch_gemm(const uint8_t* X, const uint8_t* Y, void* D, int NR, int 
 template <int XF, int YF, typename OT>
 static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                      const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
-    // large tiles once they fill the chip at least once; otherwise smaller ones for more workgroups
+    // the direct-to-LDS kernel needs whole 128-byte K slices and 32-bit row offsets; it pays off once
+    // its 256 x 256 tiles give most of the chip something to do.  Everything else takes the generic
+    // register-staged kernel with 128 x 128 tiles.
     const long big = static_cast<long>((NR + 255) / 256) * ((NC + 255) / 256);
-    if (big >= cu_count()) return launch_gemm<256, 256, XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    const bool fits32 = static_cast<unsigned long long>(NR) * K < (1ull << 32) && static_cast<unsigned long long>(NC) * K < (1ull << 32);
+    if (K % kBK == 0 && fits32 && big * 2 >= cu_count())
+        return launch_gemm_dma<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
     return launch_gemm<128, 128, XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
 }
 

@@ -96,6 +96,28 @@ def test_accumulate_and_bias(be, out_dtype):
     assert rel_fro(got.float(), want) < (TOL_F32 if out_dtype == torch.float32 else TOL_16)
 
 
+@pytest.mark.parametrize('m,n,k', [(4096, 2048, 256), (4100, 2056, 384), (3001, 2999, 128)])
+@pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32, torch.float16])
+def test_large_tiles_ragged_edges_accumulate_bias(be, m, n, k, out_dtype):
+    """Shapes big enough for the 256x256 direct-to-LDS kernel, with ragged right/bottom edges,
+    odd row lengths (no 16-byte row stores), bias and accumulation."""
+    a, b = _rand_fp8((m, k), 5, 5), _rand_fp8((n, k), 6, 6, spread=0.05)
+    tol = TOL_F32 if out_dtype == torch.float32 else TOL_16
+    want = ogemm.fp8_gemm(a, torch.tensor(0.25), fp8.E4M3, b, torch.tensor(8.0), fp8.E5M2)
+    got = _run(be, a, 5, 0.25, b, 6, 8.0, out_dtype=out_dtype)
+    assert rel_fro(got.float(), want) < tol
+    g = torch.Generator().manual_seed(9)
+    prev = torch.randn(n, m, generator=g).to(out_dtype)
+    bias = torch.randn(m, generator=g).to(out_dtype)
+    want2 = want + prev.float() + bias.float().view(1, -1)
+    got2 = _run(be, a, 5, 0.25, b, 6, 8.0, accumulate=True, bias=bias, out=prev.cuda().clone())
+    assert rel_fro(got2.float(), want2) < tol
+    # untouched memory around the output: write into the middle of a larger buffer
+    buf = torch.full((n + 2, m), 7.0, dtype=out_dtype, device='cuda')
+    _run(be, a, 5, 0.25, b, 6, 8.0, out=buf[1:n + 1])
+    assert (buf[0] == 7).all() and (buf[n + 1] == 7).all() and torch.equal(buf[1:n + 1], got)
+
+
 def test_k_not_multiple_of_16_is_padded_by_the_operator():
     import msamp    # noqa: F401
     from msamp.common.dtype import Dtypes
