@@ -51,10 +51,10 @@ enum {
     MSAMP_FLAG_NAN_TO_INF = 1 /* amax: NaN/+Inf -> +Inf before the scale rule (cast.py:37-40, sync=True) */
 };
 
-/* bytes of zero-initialised device workspace the *_intime and fused-AdamW entry points need;
- * the library leaves it zeroed again when each call's kernels finish.  Calls that share one
- * workspace must be ordered on one stream. */
-#define MSAMP_WORKSPACE_BYTES 256
+/* bytes of device workspace the two-pass entry points (msamp_amax, *_intime) need: the first pass
+ * leaves per-workgroup partial maxima there for the second.  No initialisation is required; calls
+ * that share one workspace must be ordered on one stream. */
+#define MSAMP_WORKSPACE_BYTES 8192
 
 int msamp_hip_version(void);
 const char* msamp_last_error(void);

@@ -51,15 +51,61 @@ __device__ __forceinline__ void amax_publish(float* amax, float v) {
 // ---------------------------------------------------------------------------------------------
 // Quantize with a given scale.  WITH_AMAX: also fold max|x| (NaN skipped) into *amax.
 // reverse != 0 walks the tiles back to front (second pass of the in-time cast).
-template <typename IT, int FMT, bool WITH_AMAX>
+// Workspace of the two-pass (in-time) casts, in 32-bit words: [0] scale in force before the call,
+// [1] number of partial maxima, [kWsPartials...] per-workgroup partial maxima of the first pass
+// (float bit patterns of |x|, NaN patterns included).
+constexpr int kWsPartials = 16;
+constexpr int kMaxPartials = 1024;
+
+struct InTimeArgs {
+    const uint32_t* ws;    // nullptr: the scale comes from *scale_p
+    float* scale_out;
+    float* amax_out;
+    float fp_max;
+    int margin;
+    int flags;
+};
+
+// every workgroup of the second pass derives the same amax and scale from the partial maxima
+__device__ __forceinline__ float resolve_in_time_scale(const InTimeArgs& a, uint32_t* red, float* scale_inv) {
+    __shared__ float s_scale;
+    const int np = static_cast<int>(a.ws[1]);
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < np; i += blockDim.x) {
+        const uint32_t v = a.ws[kWsPartials + i];
+        m = v > m ? v : m;
+    }
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0) {
+        float am = __uint_as_float(m);
+        if ((a.flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
+        const float s = scale_rule(am, __uint_as_float(a.ws[0]), a.fp_max, a.margin);
+        s_scale = s;
+        if (blockIdx.x == 0 && blockIdx.y == 0) {
+            *a.amax_out = am;
+            *a.scale_out = s;
+            *scale_inv = 1.0f / s;
+        }
+    }
+    __syncthreads();
+    return s_scale;
+}
+
+template <typename IT, int FMT, bool WITH_AMAX, bool INTIME>
 __global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __restrict__ x,
                                                                     uint8_t* __restrict__ out, size_t n,
                                                                     const float* __restrict__ scale_p, float* amax,
-                                                                    float* scale_inv, int vec_ok, int reverse) {
+                                                                    float* scale_inv, int vec_ok, int reverse,
+                                                                    InTimeArgs it) {
     constexpr int EPT = In16<IT>::EPT;
     constexpr size_t TILE = static_cast<size_t>(kCastThreads) * EPT * kCastUnroll;
     __shared__ uint32_t red[kCastThreads / kWave];
-    const float s = *scale_p;
+    float s;
+    if constexpr (INTIME) {
+        s = resolve_in_time_scale(it, red, scale_inv);
+    } else {
+        s = *scale_p;
+    }
     const int tid = threadIdx.x;
     float mx = 0.0f;
     const size_t ntiles = (n + TILE - 1) / TILE;
@@ -100,19 +146,19 @@ __global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __r
         uint32_t m = block_max_u32(__float_as_uint(mx), red);
         if (tid == 0) amax_publish(amax, __uint_as_float(m));
     }
-    if (scale_inv != nullptr && blockIdx.x == 0 && tid == 0) *scale_inv = 1.0f / s;
+    if constexpr (!INTIME) {
+        if (scale_inv != nullptr && blockIdx.x == 0 && tid == 0) *scale_inv = 1.0f / s;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
-// NaN-propagating max|x| with the scale rule folded into the last block to finish.
-// ws[0]: arrival counter, ws[1]: running max of |x| bit patterns; both zero on entry and exit.
+// First pass of the in-time casts: NaN-propagating max|x| per workgroup, written to the workspace
+// (no atomics, no fences: the kernel boundary orders it before the second pass).
 __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 
 template <typename IT>
-__global__ __launch_bounds__(kCastThreads) void amax_kernel(const IT* __restrict__ x, size_t n, uint32_t* ws,
-                                                             float* amax, float* scale, float* scale_inv,
-                                                             float fp_max, int margin, int flags, int update_scale,
-                                                             int vec_ok) {
+__global__ __launch_bounds__(kCastThreads) void amax_partial_kernel(const IT* __restrict__ x, size_t n, uint32_t* ws,
+                                                                     const float* scale, int vec_ok) {
     constexpr int EPT = 16 / sizeof(IT);
     constexpr int UNROLL = 8;
     constexpr size_t TILE = static_cast<size_t>(kCastThreads) * EPT * UNROLL;
@@ -157,21 +203,34 @@ __global__ __launch_bounds__(kCastThreads) void amax_kernel(const IT* __restrict
         if constexpr (sizeof(IT) == 2 && !__is_same(IT, bf16_t)) {
             m = __float_as_uint(f16_bits_to_float(m >> 16));
         }
-        if (m != 0u) atomicMax(&ws[1], m);
-        __threadfence();
-        const uint32_t ticket = atomicAdd(&ws[0], 1u);
-        if (ticket == gridDim.x - 1) {
-            __threadfence();
-            const uint32_t bits = atomicExch(&ws[1], 0u);
-            atomicExch(&ws[0], 0u);
-            float a = __uint_as_float(bits);
-            if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(a < __uint_as_float(0x7f800000u))) a = __uint_as_float(0x7f800000u);
-            *amax = a;
-            if (update_scale) {
-                const float s = scale_rule(a, *scale, fp_max, margin);
-                *scale = s;
-                *scale_inv = 1.0f / s;
-            }
+        ws[kWsPartials + blockIdx.x] = m;
+        if (blockIdx.x == 0) {
+            ws[0] = scale != nullptr ? __float_as_uint(*scale) : __float_as_uint(1.0f);
+            ws[1] = gridDim.x;
+        }
+    }
+}
+
+// reduce the partial maxima into amax[0] (and, if asked, run the scale rule) in one workgroup
+__global__ __launch_bounds__(kCastThreads) void amax_finalize_kernel(const uint32_t* ws, float* amax, float* scale,
+                                                                      float* scale_inv, float fp_max, int margin, int flags,
+                                                                      int update_scale) {
+    __shared__ uint32_t red[kCastThreads / kWave];
+    const int np = static_cast<int>(ws[1]);
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < np; i += blockDim.x) {
+        const uint32_t v = ws[kWsPartials + i];
+        m = v > m ? v : m;
+    }
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0) {
+        float a = __uint_as_float(m);
+        if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(a < __uint_as_float(0x7f800000u))) a = __uint_as_float(0x7f800000u);
+        *amax = a;
+        if (update_scale) {
+            const float s = scale_rule(a, __uint_as_float(ws[0]), fp_max, margin);
+            *scale = s;
+            *scale_inv = 1.0f / s;
         }
     }
 }
@@ -393,16 +452,23 @@ static int grid_for(size_t n, size_t tile) {
 
 template <typename IT>
 static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, float* scale_inv, uint8_t* out,
-                       int fp8_type, int reverse, hipStream_t st) {
+                       int fp8_type, const InTimeArgs* it, hipStream_t st) {
     constexpr int EPT = In16<IT>::EPT;
     const int vec_ok = aligned(x, 16) && aligned(out, EPT);
-    const int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * kCastUnroll);
-#define LAUNCH(FMT, AM) \
-    hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, AM>), dim3(grid), dim3(kCastThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, reverse)
-    if (fp8_type == MSAMP_DT_E4M3) {
-        if (amax) LAUNCH(MSAMP_DT_E4M3, true); else LAUNCH(MSAMP_DT_E4M3, false);
+    int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * kCastUnroll);
+    const InTimeArgs none = {nullptr, nullptr, nullptr, 0.0f, 0, 0};
+#define LAUNCH(FMT, AM, INT) \
+    hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, AM, INT>), dim3(grid), dim3(kCastThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, INT ? 1 : 0, INT ? *it : none)
+    if (it != nullptr) {
+        // second pass of an in-time cast: fewer, longer-lived workgroups (each one re-derives the scale),
+        // walking the tensor back to front to meet what the first pass left in the caches
+        const int cap = cu_count() * 4;
+        grid = grid < cap ? grid : cap;
+        if (fp8_type == MSAMP_DT_E4M3) LAUNCH(MSAMP_DT_E4M3, false, true); else LAUNCH(MSAMP_DT_E5M2, false, true);
+    } else if (fp8_type == MSAMP_DT_E4M3) {
+        if (amax) LAUNCH(MSAMP_DT_E4M3, true, false); else LAUNCH(MSAMP_DT_E4M3, false, false);
     } else {
-        if (amax) LAUNCH(MSAMP_DT_E5M2, true); else LAUNCH(MSAMP_DT_E5M2, false);
+        if (amax) LAUNCH(MSAMP_DT_E5M2, true, false); else LAUNCH(MSAMP_DT_E5M2, false, false);
     }
 #undef LAUNCH
     MSAMP_CHECK_LAUNCH("cast_to_fp8_kernel");
@@ -410,41 +476,49 @@ static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, f
 }
 
 template <typename IT>
-static int launch_amax(const IT* x, size_t n, uint32_t* ws, float* amax, float* scale, float* scale_inv, float fp_max,
-                       int margin, int flags, int update_scale, hipStream_t st) {
+static int launch_amax(const IT* x, size_t n, uint32_t* ws, const float* scale, hipStream_t st) {
     constexpr int EPT = 16 / sizeof(IT);
     const int vec_ok = aligned(x, 16);
-    const int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * 8);
-    hipLaunchKernelGGL((amax_kernel<IT>), dim3(grid), dim3(kCastThreads), 0, st, x, n, ws, amax, scale, scale_inv, fp_max,
-                       margin, flags, update_scale, vec_ok);
-    MSAMP_CHECK_LAUNCH("amax_kernel");
+    int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * 8);
+    const int cap = cu_count() * 4 < kMaxPartials ? cu_count() * 4 : kMaxPartials;
+    grid = grid < cap ? grid : cap;
+    hipLaunchKernelGGL((amax_partial_kernel<IT>), dim3(grid), dim3(kCastThreads), 0, st, x, n, ws, scale, vec_ok);
+    MSAMP_CHECK_LAUNCH("amax_partial_kernel");
     return MSAMP_OK;
 }
 
-static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, float* amax, float* scale, float* scale_inv,
-                         float fp_max, int margin, int flags, int update_scale, hipStream_t st) {
+// first pass: partial maxima of |x| into the workspace (plus the scale in force, for the rule's fallback)
+static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const float* scale, hipStream_t st) {
     uint32_t* w = static_cast<uint32_t*>(ws);
     switch (dtype) {
         case MSAMP_DT_F32:
-            return launch_amax(static_cast<const float*>(x), n, w, amax, scale, scale_inv, fp_max, margin, flags, update_scale, st);
+            return launch_amax(static_cast<const float*>(x), n, w, scale, st);
         case MSAMP_DT_F16:
-            return launch_amax(static_cast<const f16_t*>(x), n, w, amax, scale, scale_inv, fp_max, margin, flags, update_scale, st);
+            return launch_amax(static_cast<const f16_t*>(x), n, w, scale, st);
         case MSAMP_DT_BF16:
-            return launch_amax(static_cast<const bf16_t*>(x), n, w, amax, scale, scale_inv, fp_max, margin, flags, update_scale, st);
+            return launch_amax(static_cast<const bf16_t*>(x), n, w, scale, st);
     }
     set_error("unsupported input dtype %d", dtype);
     return MSAMP_ERR_DTYPE;
 }
 
+static int finalize_amax(void* ws, float* amax, float* scale, float* scale_inv, float fp_max, int margin, int flags,
+                         int update_scale, hipStream_t st) {
+    hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(kCastThreads), 0, st, static_cast<const uint32_t*>(ws), amax, scale,
+                       scale_inv, fp_max, margin, flags, update_scale);
+    MSAMP_CHECK_LAUNCH("amax_finalize_kernel");
+    return MSAMP_OK;
+}
+
 static int dispatch_cast(const void* x, int dtype, size_t n, const float* scale, float* amax, float* scale_inv,
-                         uint8_t* out, int fp8_type, int reverse, hipStream_t st) {
+                         uint8_t* out, int fp8_type, const InTimeArgs* it, hipStream_t st) {
     switch (dtype) {
         case MSAMP_DT_F32:
-            return launch_cast(static_cast<const float*>(x), n, scale, amax, scale_inv, out, fp8_type, reverse, st);
+            return launch_cast(static_cast<const float*>(x), n, scale, amax, scale_inv, out, fp8_type, it, st);
         case MSAMP_DT_F16:
-            return launch_cast(static_cast<const f16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, reverse, st);
+            return launch_cast(static_cast<const f16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, it, st);
         case MSAMP_DT_BF16:
-            return launch_cast(static_cast<const bf16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, reverse, st);
+            return launch_cast(static_cast<const bf16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, it, st);
     }
     set_error("unsupported input dtype %d", dtype);
     return MSAMP_ERR_DTYPE;
@@ -516,7 +590,10 @@ int msamp_amax(const void* x, int dtype, size_t n, float* amax, void* workspace,
     MSAMP_REQUIRE(amax != nullptr && (x != nullptr || n == 0), MSAMP_ERR_NULL, "msamp_amax: null pointer");
     MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_amax: workspace required");
     MSAMP_REQUIRE(is_hp(dtype), MSAMP_ERR_DTYPE, "msamp_amax: unsupported dtype %d", dtype);
-    return dispatch_amax(x, dtype, n, workspace, amax, nullptr, nullptr, 0.0f, 0, 0, 0, static_cast<hipStream_t>(stream));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int rc = dispatch_amax(x, dtype, n, workspace, nullptr, st);
+    if (rc != MSAMP_OK) return rc;
+    return finalize_amax(workspace, amax, nullptr, nullptr, 0.0f, 0, 0, 0, st);
 }
 
 int msamp_compute_scaling_factor(const float* amax, const float* scale_in, int scale_in_n, float* scale_out, int n,
@@ -537,7 +614,7 @@ int msamp_cast_to_fp8(const void* x, int in_dtype, size_t n, const float* scale,
     MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_to_fp8: in_dtype %d", in_dtype);
     MSAMP_REQUIRE(scale != nullptr && ((x != nullptr && out != nullptr) || n == 0), MSAMP_ERR_NULL,
                   "msamp_cast_to_fp8: null pointer");
-    return dispatch_cast(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, 0, static_cast<hipStream_t>(stream));
+    return dispatch_cast(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, nullptr, static_cast<hipStream_t>(stream));
 }
 
 int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
@@ -549,9 +626,10 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
                   "msamp_cast_to_fp8_intime: null pointer");
     MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_to_fp8_intime: workspace required");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int rc = dispatch_amax(x, in_dtype, n, workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st);
+    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
     if (rc != MSAMP_OK) return rc;
-    return dispatch_cast(x, in_dtype, n, scale, nullptr, nullptr, out, fp8_type, 1, st);
+    const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags};
+    return dispatch_cast(x, in_dtype, n, scale, nullptr, scale_inv, out, fp8_type, &it, st);
 }
 
 int msamp_cast_from_fp8(const uint8_t* q, int fp8_type, size_t n, const float* scale_inv, void* out, int out_dtype,
@@ -600,7 +678,9 @@ int msamp_cast_transpose_intime(const void* x, int in_dtype, int rows, int cols,
     MSAMP_REQUIRE((x && out_t) || rows == 0 || cols == 0, MSAMP_ERR_NULL, "msamp_cast_transpose_intime: null pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const size_t n = static_cast<size_t>(rows) * cols;
-    int rc = dispatch_amax(x, in_dtype, n, workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st);
+    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
+    if (rc != MSAMP_OK) return rc;
+    rc = finalize_amax(workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st);
     if (rc != MSAMP_OK || n == 0) return rc;
     return dispatch_ct(x, in_dtype, rows, cols, scale, nullptr, nullptr, out, out_t, fp8_type, st);
 }

@@ -181,14 +181,24 @@ __device__ __forceinline__ uint32_t block_max_u32(uint32_t v, uint32_t* smem) {
 // +Inf from |e| = 128.
 __device__ __forceinline__ float scale_rule(float amax, float fallback, float fp_max, int margin) {
     const float recip = 1.0f / amax;
-    float q = recip * fp_max;
-    // floor(float(log2(q))) with the float rounding done by hand: keeping the double result live in
-    // double arithmetic stops the compiler from shrinking the call to the (not correctly rounded)
-    // float log2.  If narrowing d to float reaches the next integer, the floor is that integer.
-    const double d = log2(static_cast<double>(q));
-    double fl = floor(d);
-    if (static_cast<float>(d) >= static_cast<float>(fl + 1.0)) fl += 1.0;
-    float e = static_cast<float>(fl) - static_cast<float>(margin);
+    const float q = recip * fp_max;
+    // e = floor(float(log2(q))).  For a positive normal q whose mantissa is not within 2^-17 of the
+    // next power of two, the float rounding of log2(q) cannot reach the next integer (half an ulp of
+    // any float of magnitude <= 128 is below 2^-17 / ln 2), so e is the exponent field.  Otherwise
+    // take the long road: double log2, narrowed by hand -- keeping the double result live in double
+    // arithmetic stops the compiler from shrinking the call to the (not correctly rounded) float
+    // log2; if narrowing d to float reaches the next integer, the floor is that integer.
+    const uint32_t qb = __float_as_uint(q);
+    const uint32_t qe = (qb >> 23) & 0xffu;
+    float e;
+    if ((qb >> 31) == 0u && qe != 0u && qe != 255u && (qb & 0x7fffffu) < 0x7fff80u) {
+        e = static_cast<float>(static_cast<int>(qe) - 127 - margin);
+    } else {
+        const double d = log2(static_cast<double>(q));
+        double fl = floor(d);
+        if (static_cast<float>(d) >= static_cast<float>(fl + 1.0)) fl += 1.0;
+        e = static_cast<float>(fl) - static_cast<float>(margin);
+    }
     float ae = fabsf(e);
     float sf;
     if (ae != ae) {

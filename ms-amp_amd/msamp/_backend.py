@@ -16,7 +16,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 
 DT_F32, DT_F16, DT_BF16, DT_E4M3, DT_E5M2 = 2, 3, 4, 5, 6
 FLAG_NAN_TO_INF = 1
-WORKSPACE_BYTES = 256
+WORKSPACE_BYTES = 8192
 ADAMW_CHUNK = 16384
 
 _TORCH_TO_DT = {torch.float32: DT_F32, torch.float16: DT_F16, torch.bfloat16: DT_BF16}
@@ -101,7 +101,7 @@ def _dt(t):
 
 
 def workspace(device):
-    """Per-device zero-initialised scratch words shared by the two-pass kernels (stream ordered)."""
+    """Per-device scratch words shared by the two-pass kernels (calls are stream ordered)."""
     key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
     ws = _workspaces.get(key)
     if ws is None:
