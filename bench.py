@@ -196,7 +196,7 @@ def bench_adam(iters=5, total_params=1_000_000_000):
     def step():
         state['t'] += 1
         _backend.adamw_fused(desc, len(sizes), block_map, block_map.shape[0], _backend.DT_E4M3, _backend.DT_E5M2, 3e-4, 0.9,
-                             0.95, 1e-8, 0.1, state['t'], True, False, False, True)
+                             0.95, 1e-8, 0.1, state['t'], True, False, False, True, blocks_per_tensor=chunks)
 
     ms = _time_gpu(step, iters, warm=2)
     return {'ms': ms, 'Gparams_per_s': total_params / ms / 1e6, 'GBps_algorithmic': total_params * 9 / ms / 1e6,

@@ -162,15 +162,19 @@ typedef struct msamp_adamw_tensor {
  * tensor_scale == 0) and meta rewrite; (3) recompute and requantize w (weight_dtype), m (E4M3),
  * v (scaled fp16), walking the blocks back to front so the re-read meets the cache.
  * `tensors`: DEVICE array of descriptors; `block_map`: DEVICE array of n_blocks
- * {tensor index, chunk index} int32 pairs (chunks of MSAMP_ADAMW_CHUNK elements) built by the
- * caller once per parameter set.  weight_dtype: E4M3/E5M2/F16; grad_dtype: E4M3/E5M2.
+ * {tensor index, chunk index} int32 pairs (chunks of MSAMP_ADAMW_CHUNK elements, tensors in order)
+ * built by the caller once per parameter set.  `blocks_per_tensor` (HOST array of n_tensors counts,
+ * nullable) with `group_blocks` > 0 makes the library process whole tensors in groups of at most
+ * group_blocks chunks, so that a group's second pass re-reads from the Infinity Cache instead of HBM.
+ * weight_dtype: E4M3/E5M2/F16; grad_dtype: E4M3/E5M2.
  * Hyper-parameters arrive as doubles and are narrowed the way the reference narrows them
  * (adamw.cu:99-107, adamw.py:160-164). */
 #define MSAMP_ADAMW_CHUNK 16384
 int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int32_t* block_map, int n_blocks,
                           int weight_dtype, int grad_dtype, double lr, double beta1, double beta2, double eps,
                           double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
-                          int tensor_scale, msamp_stream_t stream);
+                          int tensor_scale, const int32_t* blocks_per_tensor, int group_blocks,
+                          msamp_stream_t stream);
 
 #ifdef __cplusplus
 }

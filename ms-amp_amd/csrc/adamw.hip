@@ -9,7 +9,7 @@ namespace msamp {
 constexpr int kAdamThreads = 256;
 
 struct AdamConsts {
-    float beta1, beta2, omb1, omb2, eps, step_size, sbc2, decay, wd;
+    float beta1, beta2, omb1, omb2, eps, step_size, sbc2, inv_sbc2, decay, wd;
     int adam_mode, maximize, use_decay;
 };
 
@@ -152,34 +152,40 @@ __device__ __forceinline__ float load_w1(const void* base, size_t i) {
     }
 }
 
-// the element-wise update shared by both passes.  RAW_MOMENTS (write pass): the moments that get
-// stored are recomputed from the gradient without the Adam-mode L2 term, as the reference's second
-// stage does (msamp/optim/adamw.py:186-199), while p' keeps the term.
-template <int NE, bool RAW_MOMENTS>
-__device__ __forceinline__ void update(float* p, const float* g_in, float* m, float* v, float w_si, float g_si,
-                                       float inv_m, float inv_v, const AdamConsts& k) {
+// ---- element-wise pieces shared by both passes ------------------------------------------------
+// Exact part: dequantized weight (decayed), gradient (negated / with the Adam-mode L2 term) and the
+// new moments, all as the reference evaluates them.
+__device__ __forceinline__ void prepare(float w_raw, float g_raw, float m_old, float v_old, float w_si, float g_si,
+                                        float inv_m, float inv_v, const AdamConsts& k, float& pj, float& g_plain,
+                                        float& m_new, float& v_new) {
 #pragma clang fp contract(off)
-#pragma unroll
-    for (int j = 0; j < NE; ++j) {
-        float pj = p[j] * w_si;
-        float gj = g_in[j] * g_si;
-        if (k.maximize) gj = -gj;
-        const float g_raw = gj;
-        if (k.use_decay) {
-            if (k.adam_mode) {
-                const float t = k.wd * pj;
-                gj = gj + t;
-            } else {
-                pj = pj * k.decay;
-            }
+    pj = w_raw * w_si;
+    float gj = g_raw * g_si;
+    if (k.maximize) gj = -gj;
+    g_plain = gj;
+    if (k.use_decay) {
+        if (k.adam_mode) {
+            const float t = k.wd * pj;
+            gj = gj + t;
+        } else {
+            pj = pj * k.decay;
         }
-        float m_new, v_new;
-        moments(m[j], v[j], gj, inv_m, inv_v, k, m_new, v_new);
-        p[j] = param_update(pj, m_new, v_new, k);
-        if (RAW_MOMENTS && k.use_decay && k.adam_mode) moments(m[j], v[j], g_raw, inv_m, inv_v, k, m_new, v_new);
-        m[j] = m_new;
-        v[j] = v_new;
     }
+    moments(m_old, v_old, gj, inv_m, inv_v, k, m_new, v_new);
+}
+
+// Cheap estimate of p' = p - step * m' / (sqrt(v') / sbc2 + eps) with the hardware's 1-ulp sqrt and
+// reciprocal, and a bound on its distance from the exactly rounded chain of param_update():
+// the update term is off by at most 13 unit roundoffs, the subtraction adds one rounding on each side.
+// Non-finite inputs make the bound NaN, which every caller treats as "take the exact path".
+__device__ __forceinline__ void estimate(float pj, float m_new, float v_new, const AdamConsts& k, float& p_est,
+                                         float& err) {
+    const float root = __builtin_amdgcn_sqrtf(v_new);
+    const float den = fmaf(root, k.inv_sbc2, k.eps);
+    const float r = m_new * __builtin_amdgcn_rcpf(den);
+    const float d = k.step_size * r;
+    p_est = pj - d;
+    err = fmaf(1.0e-6f, fabsf(d), 2.0e-7f * fabsf(p_est));
 }
 
 template <int WDT, int GDT>
@@ -191,6 +197,10 @@ __device__ __forceinline__ void load16(const msamp_adamw_tensor& d, size_t i, fl
     load_w16<MSAMP_DT_F16>(d.exp_avg_sq, i, v);
 }
 
+// First pass: exact max |m'| and |v'| (they are cheap), and the exact max |p'| found by bounding:
+// every element gets the cheap estimate; only elements whose upper bound reaches the best lower bound
+// seen so far (by this wavefront, or already published for the tensor) are evaluated exactly.  The
+// element that attains the true maximum always passes that test, so the result is the exact maximum.
 template <int WDT, int GDT>
 __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_tensor* __restrict__ tensors,
                                                                    const int32_t* __restrict__ block_map,
@@ -202,32 +212,47 @@ __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_te
     const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
     const float w_si = *d.w_scale_inv, g_si = *d.g_scale_inv;
     const float inv_m = 1.0f / *d.m_scale, inv_v = 1.0f / *d.v_scale;
-    uint32_t mxp = 0;
+    uint32_t mxp = 0;    // exact |p'| bit patterns of the candidates (NaN patterns compare highest)
     float mxm = 0.0f, mxv = 0.0f;
+    // lower bound on the tensor's max |p'|: what other workgroups have published so far
+    float floor_p = __uint_as_float(__hip_atomic_load(&d.acc[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    if (!(floor_p >= 0.0f)) floor_p = 0.0f;    // a NaN already published: everything is exact from here on
     if (base + MSAMP_ADAMW_CHUNK <= n) {
-#pragma unroll 2
+#pragma unroll 1
         for (int s = 0; s < kSteps; ++s) {
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
-            float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
+            float p[kEPT], g[kEPT], m[kEPT], v[kEPT], hi[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            update<kEPT, false>(p, g, m, v, w_si, g_si, inv_m, inv_v, k);
+            float lo_max = 0.0f;
 #pragma unroll
             for (int j = 0; j < kEPT; ++j) {
-                const uint32_t ab = __float_as_uint(p[j]) & 0x7fffffffu;
-                mxp = ab > mxp ? ab : mxp;
-                mxm = fmaxf(mxm, fabsf(m[j]));
-                mxv = fmaxf(mxv, fabsf(v[j]));
+                float pj, g_plain, m_new, v_new, p_est, err;
+                prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+                estimate(pj, m_new, v_new, k, p_est, err);
+                mxm = fmaxf(mxm, fabsf(m_new));
+                mxv = fmaxf(mxv, fabsf(v_new));
+                p[j] = pj, m[j] = m_new, v[j] = v_new;
+                hi[j] = fabsf(p_est) + err;
+                lo_max = fmaxf(lo_max, fabsf(p_est) - err);    // NaN estimates are skipped here, caught below
+            }
+            floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
+#pragma unroll
+            for (int j = 0; j < kEPT; ++j) {
+                if (!(hi[j] < floor_p)) {
+                    const uint32_t ab = __float_as_uint(param_update(p[j], m[j], v[j], k)) & 0x7fffffffu;
+                    mxp = ab > mxp ? ab : mxp;
+                }
             }
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
-            float p = load_w1<WDT>(d.weight, i), g = load_w1<GDT>(d.grad, i);
-            float m = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
-            update<1, false>(&p, &g, &m, &v, w_si, g_si, inv_m, inv_v, k);
-            const uint32_t ab = __float_as_uint(p) & 0x7fffffffu;
+            float pj, g_plain, m_new, v_new;
+            prepare(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), load_w1<MSAMP_DT_E4M3>(d.exp_avg, i),
+                    load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i), w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+            const uint32_t ab = __float_as_uint(param_update(pj, m_new, v_new, k)) & 0x7fffffffu;
             mxp = ab > mxp ? ab : mxp;
-            mxm = fmaxf(mxm, fabsf(m));
-            mxv = fmaxf(mxv, fabsf(v));
+            mxm = fmaxf(mxm, fabsf(m_new));
+            mxv = fmaxf(mxv, fabsf(v_new));
         }
     }
     const uint32_t a = block_max_u32(mxp, red);
@@ -241,7 +266,7 @@ __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_te
 }
 
 __global__ void fused_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, float w_fp_max, int tensor_scale) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;    // `tensors` is pre-offset to the group's first tensor
     if (t >= n_tensors) return;
     msamp_adamw_tensor& d = tensors[t];
     const float ap = __uint_as_float(d.acc[0]), am = __uint_as_float(d.acc[1]), av = __uint_as_float(d.acc[2]);
@@ -291,6 +316,20 @@ __device__ __forceinline__ void store_w1(void* base, size_t i, float f) {
     }
 }
 
+// weight payload of one element from the exact p' (slow path of the second pass)
+template <int WDT>
+__device__ __forceinline__ uint32_t quant_weight_exact(float pj, float m_new, float v_new, float ws, const AdamConsts& k) {
+    const float pe = param_update(pj, m_new, v_new, k) * ws;
+    if constexpr (WDT == MSAMP_DT_F16) {
+        return float_to_f16_bits(pe);
+    } else {
+        return quant1<WDT>(pe);
+    }
+}
+
+// Second pass: recompute m', v' exactly and requantize them; for the weight, quantize both ends of the
+// estimate's error interval -- when they give the same code (rounding is monotonic) that code is the
+// exact answer, otherwise (or for anything non-finite) the element takes the exact chain.
 template <int WDT, int GDT>
 __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_tensor* __restrict__ tensors,
                                                                     const int32_t* __restrict__ block_map,
@@ -302,31 +341,61 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
     const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
     const float w_si = d.saved[0], g_si = *d.g_scale_inv, inv_m = d.saved[1], inv_v = d.saved[2];
     const float ws = *d.w_scale, ms = *d.m_scale, vs = *d.v_scale;
+    const bool raw_moments = k.use_decay && k.adam_mode;    // stored moments ignore the L2 term (see prepare)
     if (base + MSAMP_ADAMW_CHUNK <= n) {
-#pragma unroll 2
+#pragma unroll 1
         for (int s = 0; s < kSteps; ++s) {
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            update<kEPT, true>(p, g, m, v, w_si, g_si, inv_m, inv_v, k);
+            uint32_t wq[kEPT];
 #pragma unroll
             for (int j = 0; j < kEPT; ++j) {
-                p[j] *= ws;
-                m[j] *= ms;
-                v[j] *= vs;
+                float pj, g_plain, m_new, v_new, p_est, err;
+                prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+                estimate(pj, m_new, v_new, k, p_est, err);
+                const float lo = (p_est - err) * ws, hi = (p_est + err) * ws;
+                bool same;
+                uint32_t code;
+                if constexpr (WDT == MSAMP_DT_F16) {
+                    code = float_to_f16_bits(lo);
+                    same = code == float_to_f16_bits(hi);
+                } else {
+                    const uint32_t two = cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(hi), 0u, false);
+                    code = two & 0xffu;
+                    same = code == ((two >> 8) & 0xffu);
+                }
+                if (!(same && err < __uint_as_float(0x7f800000u))) code = quant_weight_exact<WDT>(pj, m_new, v_new, ws, k);
+                wq[j] = code;
+                if (raw_moments) moments(m[j], v[j], g_plain, inv_m, inv_v, k, m_new, v_new);
+                m[j] = m_new * ms;
+                v[j] = v_new * vs;
             }
-            store_w16<WDT>(d.weight, i, p);
+            if constexpr (WDT == MSAMP_DT_F16) {
+                uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(d.weight) + i);
+                o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
+                o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
+            } else {
+                uint4 o;
+                o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
+                o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
+                o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
+                o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
+                *reinterpret_cast<uint4*>(static_cast<uint8_t*>(d.weight) + i) = o;
+            }
             store_w16<MSAMP_DT_E4M3>(d.exp_avg, i, m);
             store_w16<MSAMP_DT_F16>(d.exp_avg_sq, i, v);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
-            float p = load_w1<WDT>(d.weight, i), g = load_w1<GDT>(d.grad, i);
-            float m = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
-            update<1, true>(&p, &g, &m, &v, w_si, g_si, inv_m, inv_v, k);
-            store_w1<WDT>(d.weight, i, p * ws);
-            store_w1<MSAMP_DT_E4M3>(d.exp_avg, i, m * ms);
-            store_w1<MSAMP_DT_F16>(d.exp_avg_sq, i, v * vs);
+            const float m_old = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v_old = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
+            float pj, g_plain, m_new, v_new;
+            prepare(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
+                    g_plain, m_new, v_new);
+            store_w1<WDT>(d.weight, i, param_update(pj, m_new, v_new, k) * ws);
+            if (raw_moments) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
+            store_w1<MSAMP_DT_E4M3>(d.exp_avg, i, m_new * ms);
+            store_w1<MSAMP_DT_F16>(d.exp_avg_sq, i, v_new * vs);
         }
     }
 }
@@ -410,7 +479,7 @@ int msamp_adamw_fp8_stage2(const float* grad, size_t n, void* exp_avg, int exp_a
 int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int32_t* block_map, int n_blocks,
                           int weight_dtype, int grad_dtype, double lr, double beta1, double beta2, double eps,
                           double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
-                          int tensor_scale, msamp_stream_t stream) {
+                          int tensor_scale, const int32_t* blocks_per_tensor, int group_blocks, msamp_stream_t stream) {
     MSAMP_REQUIRE(n_tensors >= 0 && n_blocks >= 0, MSAMP_ERR_SHAPE, "msamp_adamw_fp8_fused: n_tensors=%d n_blocks=%d",
                   n_tensors, n_blocks);
     if (n_tensors == 0 || n_blocks == 0) return MSAMP_OK;
@@ -423,33 +492,56 @@ int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int3
     k.omb1 = 1.0f - k.beta1, k.omb2 = 1.0f - k.beta2;
     k.eps = static_cast<float>(eps);
     host_consts(static_cast<float>(lr), k.beta1, k.beta2, step, bias_correction, &k.step_size, &k.sbc2);
+    k.inv_sbc2 = 1.0f / k.sbc2;
     k.decay = static_cast<float>(1.0 - lr * weight_decay);
     k.wd = static_cast<float>(weight_decay);
     k.adam_mode = adam_mode, k.maximize = maximize, k.use_decay = weight_decay != 0.0;
     const float w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
     hipStream_t st = static_cast<hipStream_t>(stream);
-#define FUSED_LAUNCH(KERNEL)                                                                                          \
+#define FUSED_LAUNCH(KERNEL, NB, BM)                                                                                  \
     do {                                                                                                              \
         if (weight_dtype == MSAMP_DT_E4M3 && grad_dtype == MSAMP_DT_E4M3)                                             \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E4M3, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k); \
+            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E4M3, MSAMP_DT_E4M3>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
         else if (weight_dtype == MSAMP_DT_E4M3)                                                                       \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E4M3, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k); \
+            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E4M3, MSAMP_DT_E5M2>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
         else if (weight_dtype == MSAMP_DT_E5M2 && grad_dtype == MSAMP_DT_E4M3)                                        \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E5M2, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k); \
+            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E5M2, MSAMP_DT_E4M3>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
         else if (weight_dtype == MSAMP_DT_E5M2)                                                                       \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E5M2, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k); \
+            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E5M2, MSAMP_DT_E5M2>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
         else if (grad_dtype == MSAMP_DT_E4M3)                                                                         \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_F16, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k); \
+            hipLaunchKernelGGL((KERNEL<MSAMP_DT_F16, MSAMP_DT_E4M3>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
         else                                                                                                          \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_F16, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k); \
+            hipLaunchKernelGGL((KERNEL<MSAMP_DT_F16, MSAMP_DT_E5M2>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
     } while (0)
-    FUSED_LAUNCH(fused_amax_kernel);
-    MSAMP_CHECK_LAUNCH("fused_amax_kernel");
-    hipLaunchKernelGGL(fused_scales_kernel, dim3((n_tensors + 63) / 64), dim3(64), 0, st, tensors, n_tensors, w_fp_max,
-                       tensor_scale);
-    MSAMP_CHECK_LAUNCH("fused_scales_kernel");
-    FUSED_LAUNCH(fused_write_kernel);
-    MSAMP_CHECK_LAUNCH("fused_write_kernel");
+    // Groups of whole tensors, each small enough that what the first pass read (5 B/param) and what
+    // the second writes (4 B/param) stay in the 256 MB Infinity Cache: the second pass then re-reads
+    // from cache and HBM sees 9 B/param.  Without the per-tensor block counts everything is one group.
+    int t0 = 0, b0 = 0;
+    while (t0 < n_tensors) {
+        int t1 = t0, b1 = b0;
+        if (blocks_per_tensor == nullptr || group_blocks <= 0) {
+            t1 = n_tensors, b1 = n_blocks;
+        } else {
+            do {
+                b1 += blocks_per_tensor[t1];
+                ++t1;
+            } while (t1 < n_tensors && b1 - b0 + blocks_per_tensor[t1] <= group_blocks);
+        }
+        MSAMP_REQUIRE(b1 <= n_blocks, MSAMP_ERR_SHAPE, "msamp_adamw_fp8_fused: blocks_per_tensor exceeds n_blocks");
+        const int nb = b1 - b0, nt = t1 - t0;
+        if (nb > 0) {
+            FUSED_LAUNCH(fused_amax_kernel, nb, block_map + 2 * b0);
+            MSAMP_CHECK_LAUNCH("fused_amax_kernel");
+        }
+        hipLaunchKernelGGL(fused_scales_kernel, dim3((nt + 63) / 64), dim3(64), 0, st, tensors + t0, nt, w_fp_max,
+                           tensor_scale);
+        MSAMP_CHECK_LAUNCH("fused_scales_kernel");
+        if (nb > 0) {
+            FUSED_LAUNCH(fused_write_kernel, nb, block_map + 2 * b0);
+            MSAMP_CHECK_LAUNCH("fused_write_kernel");
+        }
+        t0 = t1, b0 = b1;
+    }
 #undef FUSED_LAUNCH
     return MSAMP_OK;
 }

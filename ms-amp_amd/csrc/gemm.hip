@@ -194,6 +194,19 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
 
 
 
+// two floats -> packed 16-bit pair with the hardware's round-to-nearest-even converters
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
     if constexpr (N > 0) {
@@ -226,19 +239,27 @@ __device__ __noinline__ void store_chunk_slow(OT* out, uint4 val, int gcol, int 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Main kernel: 256 x 256 x 128 tile, four wavefronts each owning a 128 x 128 quadrant (256 fp32
-// accumulators per lane in the accumulation registers).  Tiles travel global -> LDS with the
-// direct-to-LDS load (no staging registers, no LDS store instructions); two LDS stages; fragments are
-// double-buffered in registers so that the LDS reads of the next 64-byte K sub-step are in flight
-// while the 16 MFMAs of the current one execute.  One workgroup barrier per 128-byte K slice, placed
-// between the two sub-steps; the loads for slice kt+2 are issued right after it.
+// Main kernel: 256 x 256 output tile over 128-byte K slices, four wavefronts each owning a 128 x 128
+// quadrant (16 accumulators of the 32x32x64 FP8 MFMA = 256 accumulation registers per lane).
+//  * Tiles travel global -> LDS with the direct-to-LDS load: no staging registers, no LDS stores.  A
+//    lane group of 8 fetches one whole 128-byte line (full-line requests are what the L2 serves best).
+//  * Two 64 KiB LDS stages.  A slice is computed in two 64-byte sub-steps; the fragments of the next
+//    sub-step are read while the 16 MFMAs of the current one execute (two register buffers).
+//  * One workgroup barrier per slice, between the sub-steps: by then every wave holds the whole slice
+//    in registers, so the stage is refilled right away (X half now, Y half during the next sub-step 0).
+//  * LDS reads and tile loads are interleaved with the MFMAs one at a time, so that neither the LDS nor
+//    the vector-memory queue backs up and stalls the MFMA stream.
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 constexpr int kDmaTile = 256;
 constexpr int kDmaStage = 2 * kDmaTile * kBK;    // X + Y slice: 64 KiB
 
-__device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }    // vmcnt(0), others unbounded
+// s_waitcnt vmcnt(N), leaving the other counters unconstrained (gfx9 encoding: vmcnt = [3:0] and [15:14])
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
 
 template <int XF, int YF, typename OT>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
@@ -255,10 +276,13 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     const int wr = wave >> 1, wc = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    // ---- global -> LDS: one wave instruction fills 8 rows x 128 bytes (1 KiB, lane-contiguous).
-    // Lane l lands in row l/8, 16-byte slot l%8 and therefore fetches the logical chunk
-    // slot ^ swizzle(row); rows past the end of the matrix are clamped to its last row.
+    // ---- global -> LDS.  A stage holds 256 X rows then 256 Y rows, 128 bytes per row.  One wave
+    // instruction fills 8 rows (1 KiB, lane-contiguous): lane l lands in row l/8, 16-byte position l%8,
+    // and therefore fetches the logical chunk position ^ swizzle(row).  Rows past the end of the matrix
+    // are clamped to its last row (their results are never stored).
     const int chunk = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)smem)));
     uint32_t xoff[8], yoff[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -269,41 +293,28 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         xoff[i] = static_cast<uint32_t>(gx) * static_cast<uint32_t>(K) + chunk * 16;
         yoff[i] = static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
     }
-    auto issue = [&](int kt, int stage) {
-        const uint8_t* xk = X + static_cast<size_t>(kt) * kBK;
-        const uint8_t* yk = Y + static_cast<size_t>(kt) * kBK;
-        uint8_t* sx = smem + stage * kDmaStage + wave * 1024;
-        uint8_t* sy = sx + kDmaTile * kBK;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(xk + xoff[i]), (lds_ptr_t)(sx + i * 4096), 16, 0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(yk + yoff[i]), (lds_ptr_t)(sy + i * 4096), 16, 0, 0);
-        }
+    // one of the 16 loads of a slice (0..7: X rows, 8..15: Y rows), so they can be spread between MFMAs
+    auto dma = [&](int kt, int stage, int which) {
+        const uint8_t* src = (which < 8 ? X : Y) + static_cast<size_t>(kt) * kBK;
+        const uint32_t off = which < 8 ? xoff[which] : yoff[which - 8];
+        const uint32_t dst = lds_base + stage * kDmaStage + (which < 8 ? 0 : kDmaTile * kBK) + ((which & 7) * 4 + wave) * 1024;
+        // Written as assembly so that the compiler does not see an LDS write it cannot tell apart from
+        // the fragment reads: it would otherwise make every LDS read wait for all loads in flight.
+        // Completion is tracked by hand with wait_vmcnt<>() before the barriers below.  M0 holds the
+        // wave's LDS destination.
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + off) : "memory", "m0");
     };
 
-    // ---- LDS -> fragments.  Row of this lane inside a 32-row block and its swizzled chunk offsets.
+    // ---- LDS -> fragments: this lane's row inside a 32-row block and its swizzled 16-byte chunks
     const int fsw = (lane & 7) ^ ((lane >> 3) & 1);
-    const int off_a = ((2 * lh) ^ fsw) << 4;    // sub-step 0, first 16 bytes; second is ^16; sub-step 1 is ^64
+    const int off_a = ((2 * lh) ^ fsw) << 4;    // sub-step 0, low half; high half is ^16, sub-step 1 is ^64
     const int xrow = (wr * 128 + l32) * kBK;
     const int yrow = kDmaTile * kBK + (wc * 128 + l32) * kBK;
-    auto load_frags = [&](int stage, int ks, v8i* fx, v8i* fy) {
-        const uint8_t* base = smem + stage * kDmaStage;
-        const int o0 = off_a ^ (ks * 64), o1 = o0 ^ 16;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const v4i lo = *reinterpret_cast<const v4i*>(base + xrow + i * 32 * kBK + o0);
-            const v4i hi = *reinterpret_cast<const v4i*>(base + xrow + i * 32 * kBK + o1);
-            fx[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const v4i lo = *reinterpret_cast<const v4i*>(base + yrow + j * 32 * kBK + o0);
-            const v4i hi = *reinterpret_cast<const v4i*>(base + yrow + j * 32 * kBK + o1);
-            fy[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
+    // fragment half h (0..15): X blocks 0..3 then Y blocks 0..3, low then high 16 bytes
+    auto frag_half = [&](int stage, int ks, int h) -> v4i {
+        const int blk = (h >> 1) & 3;
+        const int base = (h < 8 ? xrow : yrow) + blk * 32 * kBK + ((off_a ^ (ks * 64)) ^ ((h & 1) * 16));
+        return *reinterpret_cast<const v4i*>(smem + stage * kDmaStage + base);
     };
 
     v16f acc[4][4];
@@ -313,39 +324,87 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-    // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row l%32,
-    // four consecutive D columns per register quad -- the layout the epilogue wants.
-    auto mfma_block = [&](const v8i* fx, const v8i* fy) {
+
+    const int nk = K / kBK;
+    v4i fa[16], fb[16];    // fragment halves [X0..X3, Y0..Y3] x {low, high}, two buffers
+
+    // One sub-step: 16 MFMAs on `cur`, 16 fragment-half reads into `nxt`, 8 tile loads.
+    // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row l%32, four
+    // consecutive D columns per register quad -- the layout the epilogue wants.
+    // EARLY: the loads go out two per MFMA during the first four MFMAs (they are needed soonest).
+    auto sub_step = [&](const v4i* cur, v4i* nxt, int rd_stage, int rd_ks, bool do_read, int ld_kt, int ld_stage,
+                        int ld_first, bool do_load, bool early) {
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fy[j], fx[i], acc[i][j], cb, bl, 0, 0, 0, 0);
+            for (int j = 0; j < 4; ++j) {
+                const int n = i * 4 + j;
+                const v8i fx = __builtin_shufflevector(cur[2 * i], cur[2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                const v8i fy = __builtin_shufflevector(cur[8 + 2 * j], cur[8 + 2 * j + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fy, fx, acc[i][j], cb, bl, 0, 0, 0, 0);
+                if (do_read) nxt[n] = frag_half(rd_stage, rd_ks, n);
+                if (do_load) {
+                    if (early) {
+                        if (n < 4) {
+                            dma(ld_kt, ld_stage, ld_first + 2 * n);
+                            dma(ld_kt, ld_stage, ld_first + 2 * n + 1);
+                        }
+                    } else if (n & 1) {
+                        dma(ld_kt, ld_stage, ld_first + (n >> 1));
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < 16; ++n) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // one LDS read
+        }
     };
 
-    const int nk = K / kBK;
-    v8i fx0[4], fy0[4], fx1[4], fy1[4];
-    issue(0, 0);
+    // prologue: slice 0 and the X half of slice 1; wait for slice 0; read its first fragments
+#pragma unroll
+    for (int w = 0; w < 16; ++w) dma(0, 0, w);
     if (nk > 1) {
-        issue(1, 1);
-        __builtin_amdgcn_s_waitcnt(0x4F70);    // vmcnt(16): the 16 loads of slice 0 have landed
+#pragma unroll
+        for (int w = 0; w < 8; ++w) dma(1, 1, w);
+        wait_vmcnt<8>();
     } else {
-        wait_vmcnt0();
+        wait_vmcnt<0>();
     }
     __syncthreads();
-    load_frags(0, 0, fx0, fy0);
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        load_frags(cur, 1, fx1, fy1);
-        mfma_block(fx0, fy0);
-        wait_vmcnt0();    // slice kt+1 (issued one barrier ago) has landed
-        __syncthreads();  // ... for every wave, and every wave holds slice kt in registers
-        if (kt + 2 < nk) issue(kt + 2, cur);
-        if (kt + 1 < nk) load_frags(cur ^ 1, 0, fx0, fy0);
-        mfma_block(fx1, fy1);
+#pragma unroll
+    for (int n = 0; n < 16; ++n) fa[n] = frag_half(0, 0, n);
+
+    // slice kt lives in stage kt & 1.  Sub-step 0: MFMAs on its first half, read its second half, send the
+    // Y half of slice kt+1 on its way (its X half went out during the previous sub-step 1).  Barrier: slice
+    // kt+1 has landed for every wave and nobody needs the LDS copy of slice kt any more.  Sub-step 1: MFMAs
+    // on the second half, read the first half of slice kt+1, start refilling this stage with slice kt+2.
+    int kt = 0;
+    for (; kt + 3 < nk; kt += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            sub_step(fa, fb, u, 1, true, kt + u + 1, u ^ 1, 8, true, true);
+            wait_vmcnt<0>();
+            __syncthreads();
+            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, 0, true, false);
+        }
     }
+    for (; kt < nk; kt += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k1 = kt + u;
+            if (k1 < nk) {
+                sub_step(fa, fb, u, 1, true, k1 + 1, u ^ 1, 8, k1 + 1 < nk, true);
+                wait_vmcnt<0>();
+                __syncthreads();
+                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, 0, k1 + 2 < nk, false);
+            }
+        }
+    }
+    wait_vmcnt<0>();
     __syncthreads();    // LDS is reused below
 
     // ---- epilogue: per 32-row block, accumulators -> this wave's LDS patch -> 16-byte row stores
@@ -371,11 +430,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 if constexpr (kEsz == 4) {
                     *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
                 } else if constexpr (__is_same(OT, bf16_t)) {
-                    *reinterpret_cast<uint2*>(dst) = make_uint2(float_to_bf16_bits(v0) | (float_to_bf16_bits(v1) << 16),
-                                                                float_to_bf16_bits(v2) | (float_to_bf16_bits(v3) << 16));
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(v0, v1), pack_bf16(v2, v3));
                 } else {
-                    *reinterpret_cast<uint2*>(dst) = make_uint2(float_to_f16_bits(v0) | (float_to_f16_bits(v1) << 16),
-                                                                float_to_f16_bits(v2) | (float_to_f16_bits(v3) << 16));
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_f16(v0, v1), pack_f16(v2, v3));
                 }
             }
         });

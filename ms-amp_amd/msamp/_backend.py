@@ -42,7 +42,7 @@ _SIGNATURES = {
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
-    'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
+    'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -279,14 +279,24 @@ def adamw_stage2(grad, exp_avg, exp_avg_dt, old_factor, new_factor, beta1, exp_a
 ADAMW_DESC_WORDS = 19    # int64 words per msamp_adamw_tensor (152 bytes)
 
 
+# chunks per cache-resident group of the fused AdamW step; 0 = one group (the kernels are compute-bound, so
+# splitting the launch only costs occupancy)
+ADAMW_GROUP_BLOCKS = int(os.environ.get('MSAMP_ADAMW_GROUP_BLOCKS', 0))
+
+
 def adamw_fused(desc, n_tensors, block_map, n_blocks, weight_dt, grad_dt, lr, beta1, beta2, eps, weight_decay, step,
-                bias_correction, adam_mode, maximize, tensor_scale):
+                bias_correction, adam_mode, maximize, tensor_scale, blocks_per_tensor=None, group_blocks=None):
+    """blocks_per_tensor: host-side sequence of chunk counts (one per tensor) enabling cache-sized groups."""
     lib = load()
     _gpu(desc, 'descriptor table')
+    bpt = None
+    if blocks_per_tensor is not None:
+        bpt = (ctypes.c_int32 * n_tensors)(*blocks_per_tensor)
+    gb = ADAMW_GROUP_BLOCKS if group_blocks is None else group_blocks
     _check(
         lib.msamp_adamw_fp8_fused(
             _ptr(desc), n_tensors, _ptr(block_map), n_blocks, weight_dt, grad_dt, lr, beta1, beta2, eps, weight_decay,
             step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0, 1 if tensor_scale else 0,
-            _stream()
+            ctypes.cast(bpt, ctypes.c_void_p) if bpt is not None else None, gb if bpt is not None else 0, _stream()
         ), 'msamp_adamw_fp8_fused'
     )

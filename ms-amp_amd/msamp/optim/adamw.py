@@ -59,15 +59,15 @@ class LBAdamW(LBAdamWBase):
         sig = tuple(rows)
         cached = self._fused_cache.get(key)
         if cached is not None and cached[0] == sig:
-            return cached[1], cached[2], cached[3]
+            return cached[1], cached[2], cached[3], cached[4]
         device = params[0].value.device
         desc = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), _backend.ADAMW_DESC_WORDS)).to(device)
         chunks = [(p.value.numel() + _backend.ADAMW_CHUNK - 1) // _backend.ADAMW_CHUNK for p in params]
         tensor_idx = np.repeat(np.arange(len(params), dtype=np.int32), chunks)
         chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in chunks]) if chunks else np.zeros(0, np.int32)
         block_map = torch.from_numpy(np.stack([tensor_idx, chunk_idx], axis=1).copy()).to(device)
-        self._fused_cache[key] = (sig, desc, block_map, int(block_map.shape[0]))
-        return desc, block_map, int(block_map.shape[0])
+        self._fused_cache[key] = (sig, desc, block_map, int(block_map.shape[0]), chunks)
+        return desc, block_map, int(block_map.shape[0]), chunks
 
     def _fused_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, step, *, beta1, beta2, lr, weight_decay, eps,
                     maximize):
@@ -75,10 +75,10 @@ class LBAdamW(LBAdamWBase):
         ms, vs = [exp_avgs[i] for i in idx], [exp_avg_sqs[i] for i in idx]
         wq, gq = ps[0].qtype, gs[0].qtype
         key = (int(wq), int(gq), id(ps[0]))
-        desc, block_map, n_blocks = self._fused_tables(key, ps, gs, ms, vs)
+        desc, block_map, n_blocks, chunks = self._fused_tables(key, ps, gs, ms, vs)
         _backend.adamw_fused(
             desc, len(ps), block_map, n_blocks, int(wq), int(gq), lr, beta1, beta2, eps, weight_decay, step,
-            self.bias_correction, self.use_adam, maximize, self.tensor_scale
+            self.bias_correction, self.use_adam, maximize, self.tensor_scale, blocks_per_tensor=chunks
         )
 
     # ---- per-tensor path (reference recipe) -----------------------------------------------

@@ -75,7 +75,8 @@ def _fused(be, tensors, w_dt, g_dt, step, **kw):
     hyper.update(kw)
     be.adamw_fused(desc, len(tensors), block_map, block_map.shape[0], w_dt, g_dt, hyper['lr'], hyper['beta1'], hyper['beta2'],
                    hyper['eps'], hyper['weight_decay'], step, hyper.get('bias_correction', True), hyper.get('adam_mode', False),
-                   hyper.get('maximize', False), hyper.get('tensor_scale', True))
+                   hyper.get('maximize', False), hyper.get('tensor_scale', True), blocks_per_tensor=chunks,
+                   group_blocks=hyper.get('group_blocks'))
     torch.cuda.synchronize()
     # the scratch words of the descriptors are left zeroed
     assert (desc[:, 15].cpu() == 0).all()
@@ -120,6 +121,17 @@ def test_fused_step_variants(be, kw):
     t = _inputs(16384 * 3 + 100, 7, fp8.E4M3, fp8.E5M2)
     dev = _fused(be, [t], 5, 6, 3, **kw)
     _check(dev[0], t, fp8.E4M3, fp8.E5M2, 3, **kw)
+
+
+def test_fused_step_grouping_does_not_change_results(be):
+    sizes = [16384 * 3, 16384 * 5 + 9, 100, 16384 * 2]
+    tensors = [_inputs(n, 300 + i, fp8.E4M3, fp8.E5M2) for i, n in enumerate(sizes)]
+    ref = _fused(be, tensors, 5, 6, 2, group_blocks=0)
+    for gb in (1, 4, 6, 1000):
+        got = _fused(be, tensors, 5, 6, 2, group_blocks=gb)
+        for a, b in zip(ref, got):
+            assert torch.equal(a['w'], b['w']) and torch.equal(a['m'], b['m']) and torch.equal(a['v'], b['v'])
+            assert all(torch.equal(x, y) for x, y in zip(a['wm'] + a['mm'] + a['vm'], b['wm'] + b['mm'] + b['vm']))
 
 
 def test_fused_step_is_deterministic(be):
