@@ -106,19 +106,19 @@ def bench_fp8linear(steps, warmup):
 
 
 def _time_gpu(fn, iters, warm=3):
+    """Average duration of one call, from HIP events around a batch of `iters` back-to-back calls on the
+    current stream (what a kernel sustains once the launch queue is primed)."""
     import torch
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
-    total = 0.0
+    s, e = _events()
+    s.record()
     for _ in range(iters):
-        s, e = _events()
-        s.record()
         fn()
-        e.record()
-        e.synchronize()
-        total += s.elapsed_time(e)
-    return total / iters
+    e.record()
+    e.synchronize()
+    return s.elapsed_time(e) / iters
 
 
 def bench_cast(iters=20):
