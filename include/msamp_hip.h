@@ -48,13 +48,15 @@ enum {
 
 /* flags of msamp_cast_to_fp8_intime / msamp_cast_transpose_intime */
 enum {
-    MSAMP_FLAG_NAN_TO_INF = 1 /* amax: NaN/+Inf -> +Inf before the scale rule (cast.py:37-40, sync=True) */
+    MSAMP_FLAG_NAN_TO_INF = 1, /* amax: NaN/+Inf -> +Inf before the scale rule (cast.py:37-40, sync=True) */
+    MSAMP_FLAG_TWO_PASS = 2    /* never take the one-pass (register-resident, grid-barrier) kernel */
 };
 
-/* bytes of device workspace the two-pass entry points (msamp_amax, *_intime) need: the first pass
- * leaves per-workgroup partial maxima there for the second.  No initialisation is required; calls
- * that share one workspace must be ordered on one stream. */
-#define MSAMP_WORKSPACE_BYTES 8192
+/* bytes of device workspace the amax and in-time entry points (msamp_amax, *_intime) need: partial
+ * maxima of a first pass, or the per-workgroup slots through which the one-pass kernel's
+ * workgroups meet.  Zero it once after allocating it (every call leaves it ready for the next);
+ * calls that share one workspace must be ordered on one stream. */
+#define MSAMP_WORKSPACE_BYTES 16384
 
 int msamp_hip_version(void);
 const char* msamp_last_error(void);

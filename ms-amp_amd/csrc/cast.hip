@@ -3,6 +3,9 @@
 // wavefront shuffle reductions, one atomic per block.
 #include "common.cuh"
 
+#include <atomic>
+#include <mutex>
+
 namespace msamp {
 
 constexpr int kCastThreads = 256;
@@ -13,16 +16,16 @@ struct In16;    // one 16-byte load = EPT elements as float
 template <>
 struct In16<float> {
     static constexpr int EPT = 4;
-    static __device__ __forceinline__ void load(const float* p, float* v) {
-        float4 t = *reinterpret_cast<const float4*>(p);
-        v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+    static __device__ __forceinline__ void decode(const uint4& t, float* v) {
+        v[0] = __uint_as_float(t.x), v[1] = __uint_as_float(t.y), v[2] = __uint_as_float(t.z), v[3] = __uint_as_float(t.w);
     }
+    static __device__ __forceinline__ void load(const float* p, float* v) { decode(*reinterpret_cast<const uint4*>(p), v); }
 };
 template <>
 struct In16<bf16_t> {
     static constexpr int EPT = 8;
-    static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
-        uint4 t = *reinterpret_cast<const uint4*>(p);
+    static __device__ __forceinline__ void load(const bf16_t* p, float* v) { decode(*reinterpret_cast<const uint4*>(p), v); }
+    static __device__ __forceinline__ void decode(const uint4& t, float* v) {
         v[0] = __uint_as_float(t.x << 16), v[1] = __uint_as_float(t.x & 0xffff0000u);
         v[2] = __uint_as_float(t.y << 16), v[3] = __uint_as_float(t.y & 0xffff0000u);
         v[4] = __uint_as_float(t.z << 16), v[5] = __uint_as_float(t.z & 0xffff0000u);
@@ -32,8 +35,8 @@ struct In16<bf16_t> {
 template <>
 struct In16<f16_t> {
     static constexpr int EPT = 8;
-    static __device__ __forceinline__ void load(const f16_t* p, float* v) {
-        uint4 t = *reinterpret_cast<const uint4*>(p);
+    static __device__ __forceinline__ void load(const f16_t* p, float* v) { decode(*reinterpret_cast<const uint4*>(p), v); }
+    static __device__ __forceinline__ void decode(const uint4& t, float* v) {
         v[0] = f16_bits_to_float(t.x & 0xffffu), v[1] = f16_bits_to_float(t.x >> 16);
         v[2] = f16_bits_to_float(t.y & 0xffffu), v[3] = f16_bits_to_float(t.y >> 16);
         v[4] = f16_bits_to_float(t.z & 0xffffu), v[5] = f16_bits_to_float(t.z >> 16);
@@ -236,6 +239,139 @@ __global__ __launch_bounds__(kCastThreads) void amax_finalize_kernel(const uint3
 }
 
 // ---------------------------------------------------------------------------------------------
+// One-pass in-time cast for tensors that fit the register file of the chip: each 512-lane workgroup
+// (two per CU) keeps a contiguous run of x in registers (up to kResVecs 16-byte vectors per lane),
+// publishes max|x| of its run, waits until every workgroup has published, and quantizes from
+// registers, so x is read once.
+// The grid-wide meeting uses no atomics and no fences: workgroup b stores {token, max} as one
+// 8-byte word into slot b of the workspace (slots start at byte kWsSlotBytes), then the first wave
+// of every workgroup polls all slots until each carries this call's token, reducing the maxima on
+// the way; every workgroup then derives the same scale by itself.  Tokens come from a host counter,
+// so slots never need clearing.  All workgroups must be resident together: the host launches at most
+// two per CU and keeps the kernel to one stream per device; the wait is bounded all the same, and a
+// wait that runs out reports NaN as the amax.
+constexpr int kResThreads = 512;
+constexpr int kResVecs = 16;
+constexpr int kResBlocksPerCu = 2;
+constexpr int kWsSlotBytes = 8192;
+constexpr int kMaxSlots = 512;
+static_assert(kWsSlotBytes + kMaxSlots * 8 <= MSAMP_WORKSPACE_BYTES, "slots exceed the workspace");
+
+template <typename IT>
+__device__ __forceinline__ uint32_t abs_bits_hi(uint32_t raw) {    // raw element bits -> ordered key
+    if constexpr (sizeof(IT) == 4) return raw & 0x7fffffffu;
+    else return (raw << 16) & 0x7fff0000u;
+}
+
+template <typename IT, int FMT>
+__global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void cast_intime_resident_kernel(const IT* __restrict__ x,
+                                                                           uint8_t* __restrict__ out, size_t n,
+                                                                           float* scale, float* amax, float* scale_inv,
+                                                                           uint64_t* slots, float fp_max, int margin,
+                                                                           int flags, int rounds, uint32_t token,
+                                                                           uint32_t spin_limit) {
+    constexpr int EPT = 16 / sizeof(IT);
+    using Raw = typename std::conditional<sizeof(IT) == 4, uint32_t, uint16_t>::type;
+    __shared__ uint32_t red[kResThreads / kWave];
+    __shared__ uint32_t s_scale;
+    const int tid = threadIdx.x;
+    // the host keeps the vector count within 32 bits (at most one register file of vectors)
+    const uint32_t nvec = static_cast<uint32_t>(n / EPT);
+    // each workgroup owns one contiguous run of rounds * kResThreads vectors
+    const uint32_t v0 = blockIdx.x * static_cast<uint32_t>(rounds) * kResThreads + tid;
+    const float old_scale = *scale;    // read before any workgroup can pass the meeting and replace it
+
+    uint4 v[kResVecs];
+#pragma unroll
+    for (int r = 0; r < kResVecs; ++r) {
+        // unconditional (clamped) loads, so that all of them are in flight together; a vector read
+        // twice changes no maximum, and the store phase skips the duplicates
+        const uint32_t idx = v0 + r * kResThreads;
+        v[r] = reinterpret_cast<const uint4*>(x)[idx < nvec ? idx : nvec - 1];
+    }
+    // the ragged end (fewer than EPT elements) rides with the first lanes of workgroup 0
+    const size_t tail0 = static_cast<size_t>(nvec) * EPT;
+    const bool has_tail = blockIdx.x == 0 && tail0 + tid < n;
+    Raw tail_raw = 0;
+    if (has_tail) tail_raw = reinterpret_cast<const Raw*>(x)[tail0 + tid];
+
+    uint32_t m = abs_bits_hi<IT>(tail_raw);
+#pragma unroll
+    for (int r = 0; r < kResVecs; ++r) {
+        const uint32_t w[4] = {v[r].x, v[r].y, v[r].z, v[r].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (sizeof(IT) == 4) m = umax(m, w[j] & 0x7fffffffu);
+            else m = umax(m, umax((w[j] << 16) & 0x7fff0000u, w[j] & 0x7fff0000u));
+        }
+    }
+    m = block_max_u32(m, red);    // valid in lane 0 of wave 0
+    if (tid < kWave) {
+        if (tid == 0) {
+            if constexpr (sizeof(IT) == 2 && !__is_same(IT, bf16_t)) m = __float_as_uint(f16_bits_to_float(m >> 16));
+            __hip_atomic_store(slots + blockIdx.x, (static_cast<uint64_t>(token) << 32) | m, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        uint32_t spins = 0, mm;
+        bool all_in;
+        do {
+            // all slots of one poll are requested together; the ones past the grid are read and ignored
+            uint64_t sv[kMaxSlots / kWave];
+#pragma unroll
+            for (int j = 0; j < kMaxSlots / kWave; ++j)
+                sv[j] = __hip_atomic_load(slots + tid + j * kWave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            bool ok = true;
+            mm = 0;
+#pragma unroll
+            for (int j = 0; j < kMaxSlots / kWave; ++j) {
+                const bool live = static_cast<uint32_t>(tid + j * kWave) < gridDim.x;
+                ok = ok && (!live || static_cast<uint32_t>(sv[j] >> 32) == token);
+                mm = umax(mm, live ? static_cast<uint32_t>(sv[j]) : 0u);
+            }
+            all_in = __all(ok);
+        } while (!all_in && ++spins < spin_limit);
+        mm = wave_max_u32(mm);
+        if (tid == 0) {
+            float am = __uint_as_float(mm);
+            if (!all_in) am = __uint_as_float(0x7fc00000u);    // the wait ran out: make the failure visible
+            else if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
+            const float s = scale_rule(am, old_scale, fp_max, margin);
+            s_scale = __float_as_uint(s);
+            if (blockIdx.x == 0) {
+                *amax = am;
+                *scale = s;
+                *scale_inv = 1.0f / s;
+            }
+        }
+    }
+    __syncthreads();
+    const float s = __uint_as_float(s_scale);
+
+#pragma unroll
+    for (int r = 0; r < kResVecs; ++r) {
+        // keep only the raw words live across the barrier, not values derived from them before it
+        asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
+        const uint32_t idx = v0 + r * kResThreads;
+        if (r < rounds && idx < nvec) {
+            float f[EPT];
+            In16<IT>::decode(v[r], f);
+            uint32_t w[EPT / 4];
+#pragma unroll
+            for (int j = 0; j < EPT / 4; ++j) w[j] = quant4<FMT>(f[4 * j] * s, f[4 * j + 1] * s, f[4 * j + 2] * s, f[4 * j + 3] * s);
+            if constexpr (EPT == 4) reinterpret_cast<uint32_t*>(out)[idx] = w[0];
+            else reinterpret_cast<uint2*>(out)[idx] = make_uint2(w[0], w[1]);
+        }
+    }
+    if (has_tail) {
+        float a;
+        if constexpr (sizeof(IT) == 4) a = __uint_as_float(tail_raw);
+        else if constexpr (__is_same(IT, bf16_t)) a = __uint_as_float(static_cast<uint32_t>(tail_raw) << 16);
+        else a = f16_bits_to_float(tail_raw);
+        out[tail0 + tid] = static_cast<uint8_t>(quant1<FMT>(a * s));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 template <int FMT, typename OT>
 __global__ __launch_bounds__(kCastThreads) void cast_from_fp8_kernel(const uint8_t* __restrict__ q,
                                                                       OT* __restrict__ out, size_t n,
@@ -416,6 +552,62 @@ __global__ __launch_bounds__(kCastThreads) void cast_transpose_kernel(const IT* 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Byte transpose with 16-byte accesses on both sides: a 128x128 tile goes through LDS (rows rotated
+// by their index so that neither side piles up on a bank), each lane gathers a 4-byte-wide, 16-row
+// column strip, transposes its four 4x4 byte blocks with byte permutes and writes 16 bytes of four
+// output rows.  Eight neighbouring lanes fill one 128-byte line on the way in and on the way out.
+// Needs R % 16 == 0, C % 16 == 0 and 16-byte aligned pointers.
+__device__ __forceinline__ void transpose4x4_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d, uint32_t* o) {
+    const uint32_t t0 = __builtin_amdgcn_perm(b, a, 0x05010400u), t1 = __builtin_amdgcn_perm(b, a, 0x07030602u);
+    const uint32_t t2 = __builtin_amdgcn_perm(d, c, 0x05010400u), t3 = __builtin_amdgcn_perm(d, c, 0x07030602u);
+    o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+    o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+    o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+__global__ __launch_bounds__(kCastThreads) void byte_transpose128_kernel(const uint8_t* __restrict__ in,
+                                                                          uint8_t* __restrict__ out_t, int R, int C) {
+    __shared__ uint4 tile[128 * 8];    // [row][8 chunks of 16 bytes], chunk index rotated per row
+    const int tid = threadIdx.x;
+    const int r0 = blockIdx.y * 128, c0 = blockIdx.x * 128;
+    {
+        const int ch = tid & 7;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int row = p * 32 + (tid >> 3);
+            uint4 t = make_uint4(0, 0, 0, 0);
+            if (r0 + row < R && c0 + ch * 16 < C)
+                t = *reinterpret_cast<const uint4*>(in + static_cast<size_t>(r0 + row) * C + c0 + ch * 16);
+            tile[row * 8 + ((ch + (row >> 4) + (row & 7)) & 7)] = t;
+        }
+    }
+    __syncthreads();
+    const int g = tid & 7, w = tid >> 3;    // rows 16g..16g+15 of the tile, byte columns 4w..4w+3
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(tile);
+    uint32_t o[4][4];                       // o[q][i]: column 4w+i, rows 16g+4q..+3
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t a[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = 4 * q + j, row = 16 * g + k;
+            a[j] = words[row * 32 + ((w + 4 * (g + (k & 7))) & 31)];
+        }
+        transpose4x4_bytes(a[0], a[1], a[2], a[3], o[q]);
+    }
+    if (r0 + 16 * g < R) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = c0 + 4 * w + i;
+            if (c < C)
+                *reinterpret_cast<uint4*>(out_t + static_cast<size_t>(c) * R + r0 + 16 * g) =
+                    make_uint4(o[0][i], o[1][i], o[2][i], o[3][i]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 __global__ void scaling_factor_kernel(const float* amax, const float* scale_in, int scale_in_n, float* scale_out, int n,
                                       float fp_max, int margin) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -500,6 +692,95 @@ static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const flo
     }
     set_error("unsupported input dtype %d", dtype);
     return MSAMP_ERR_DTYPE;
+}
+
+// One-pass (register-resident) in-time cast; returns 1 if it does not apply and the two-pass path must run.
+// Its workgroups wait for each other, so two such kernels must never share the chip half-resident:
+// the first stream to use it on a device keeps it, other streams take the two-pass path.
+static int g_intime_mode = -1;    // MSAMP_INTIME_MODE=0 in the environment: two-pass only
+static std::atomic<uint32_t> g_token{0};
+static std::mutex g_owner_mutex;
+static hipStream_t g_owner_stream[64];
+static bool g_owner_set[64];
+
+static bool owns_resident_kernel(hipStream_t st) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    std::lock_guard<std::mutex> lock(g_owner_mutex);
+    if (!g_owner_set[dev]) {
+        g_owner_set[dev] = true;
+        g_owner_stream[dev] = st;
+    }
+    return g_owner_stream[dev] == st;
+}
+
+// true if the runtime confirms kResBlocksPerCu workgroups of this kernel fit one CU (asked once per kernel)
+static bool fits_resident(const void* fn) {
+    static std::mutex mu;
+    static const void* known[16];
+    static bool fits[16];
+    static int n_known = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < n_known; ++i)
+        if (known[i] == fn) return fits[i];
+    int blocks = 0;
+    const bool ok = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, fn, kResThreads, 0) == hipSuccess &&
+                    blocks >= kResBlocksPerCu;
+    if (n_known < 16) {
+        known[n_known] = fn;
+        fits[n_known++] = ok;
+    }
+    return ok;
+}
+
+template <typename IT>
+static int launch_resident(const IT* x, size_t n, float* scale, float* amax, float* scale_inv, uint8_t* out,
+                           int fp8_type, int margin, int flags, void* ws, hipStream_t st) {
+    constexpr int EPT = 16 / sizeof(IT);
+    if (g_intime_mode < 0) {
+        const char* e = getenv("MSAMP_INTIME_MODE");
+        g_intime_mode = e ? atoi(e) : 1;
+    }
+    if (g_intime_mode == 0 || (flags & MSAMP_FLAG_TWO_PASS)) return 1;
+    if (!aligned(x, 16) || !aligned(out, EPT)) return 1;
+    const size_t nvec = n / EPT;
+    size_t max_blocks = static_cast<size_t>(cu_count()) * kResBlocksPerCu;
+    if (max_blocks > static_cast<size_t>(kMaxSlots)) max_blocks = kMaxSlots;
+    if (nvec == 0 || nvec > max_blocks * kResThreads * kResVecs) return 1;
+    if (!owns_resident_kernel(st)) return 1;
+    const void* fn = fp8_type == MSAMP_DT_E4M3
+                         ? reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E4M3>)
+                         : reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E5M2>);
+    if (!fits_resident(fn)) return 1;
+    // as many workgroups as there are runs of kResThreads vectors, up to the resident limit
+    size_t g = (nvec + kResThreads - 1) / kResThreads;
+    g = g > max_blocks ? max_blocks : g;
+    int rounds = static_cast<int>((nvec + g * kResThreads - 1) / (g * kResThreads));
+    g = (nvec + static_cast<size_t>(rounds) * kResThreads - 1) / (static_cast<size_t>(rounds) * kResThreads);
+    uint32_t token = ++g_token;
+    if (token == 0) token = ++g_token;
+    uint64_t* slots = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + kWsSlotBytes);
+    const float fp_max = fp8_max(fp8_type);
+    const uint32_t spin_limit = 1u << 20;    // a fraction of a second of polling
+#define LAUNCH(FMT) \
+    hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit)
+    if (fp8_type == MSAMP_DT_E4M3) LAUNCH(MSAMP_DT_E4M3); else LAUNCH(MSAMP_DT_E5M2);
+#undef LAUNCH
+    MSAMP_CHECK_LAUNCH("cast_intime_resident_kernel");
+    return MSAMP_OK;
+}
+
+static int dispatch_resident(const void* x, int dtype, size_t n, float* scale, float* amax, float* scale_inv, uint8_t* out,
+                             int fp8_type, int margin, int flags, void* ws, hipStream_t st) {
+    switch (dtype) {
+        case MSAMP_DT_F32:
+            return launch_resident(static_cast<const float*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st);
+        case MSAMP_DT_F16:
+            return launch_resident(static_cast<const f16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st);
+        case MSAMP_DT_BF16:
+            return launch_resident(static_cast<const bf16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st);
+    }
+    return 1;
 }
 
 static int finalize_amax(void* ws, float* amax, float* scale, float* scale_inv, float fp_max, int margin, int flags,
@@ -626,7 +907,9 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
                   "msamp_cast_to_fp8_intime: null pointer");
     MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_to_fp8_intime: workspace required");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
+    int rc = dispatch_resident(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, margin, flags, workspace, st);
+    if (rc <= 0) return rc;
+    rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
     if (rc != MSAMP_OK) return rc;
     const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags};
     return dispatch_cast(x, in_dtype, n, scale, nullptr, scale_inv, out, fp8_type, &it, st);
@@ -689,6 +972,12 @@ int msamp_fp8_transpose(const uint8_t* q, int rows, int cols, uint8_t* out, msam
     MSAMP_REQUIRE(rows >= 0 && cols >= 0, MSAMP_ERR_SHAPE, "msamp_fp8_transpose: shape %d x %d", rows, cols);
     if (rows == 0 || cols == 0) return MSAMP_OK;
     MSAMP_REQUIRE(q && out, MSAMP_ERR_NULL, "msamp_fp8_transpose: null pointer");
+    if (rows % 16 == 0 && cols % 16 == 0 && aligned(q, 16) && aligned(out, 16) && (rows + 127) / 128 <= 65535) {
+        hipLaunchKernelGGL(byte_transpose128_kernel, dim3((cols + 127) / 128, (rows + 127) / 128), dim3(kCastThreads), 0,
+                           static_cast<hipStream_t>(stream), q, out, rows, cols);
+        MSAMP_CHECK_LAUNCH("byte_transpose128_kernel");
+        return MSAMP_OK;
+    }
     return launch_ct<uint8_t, false>(q, rows, cols, nullptr, nullptr, nullptr, nullptr, out, MSAMP_DT_E4M3,
                                      static_cast<hipStream_t>(stream));
 }

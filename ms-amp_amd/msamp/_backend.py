@@ -16,7 +16,8 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 
 DT_F32, DT_F16, DT_BF16, DT_E4M3, DT_E5M2 = 2, 3, 4, 5, 6
 FLAG_NAN_TO_INF = 1
-WORKSPACE_BYTES = 8192
+FLAG_TWO_PASS = 2
+WORKSPACE_BYTES = 16384
 ADAMW_CHUNK = 16384
 
 _TORCH_TO_DT = {torch.float32: DT_F32, torch.float16: DT_F16, torch.bfloat16: DT_BF16}
@@ -156,14 +157,17 @@ def cast_to_fp8(x, scale, amax_cell, scale_inv, fp8_dt):
     return out
 
 
-def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_inf=False):
+def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_inf=False, two_pass=False):
+    """amax, scale rule, quantize and reciprocal in one call.  `two_pass` keeps the call off the
+    one-pass kernel whose workgroups wait for each other (same results either way)."""
     lib = load()
     _gpu(x, 'input')
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
     _check(
         lib.msamp_cast_to_fp8_intime(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
-            FLAG_NAN_TO_INF if nan_to_inf else 0, _ptr(workspace(x.device)), _stream()
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass else 0), _ptr(workspace(x.device)),
+            _stream()
         ), 'msamp_cast_to_fp8_intime'
     )
     return out

@@ -124,6 +124,39 @@ def test_in_time_cast_ragged_sizes(be, dtype, n):
         assert same_float(am[0], om['amax'][0]) and same_float(s, om['scale']) and same_float(si, om['scale_inv'])
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize('n', [512 * 4 + 3, 5_000_003, 512 * 512 * 16 * 4 + 8, 20_000_000])
+def test_in_time_cast_one_pass_matches_two_pass(be, dtype, n):
+    """The register-resident kernel (partly filled rounds, the largest tensor it takes, one past it)
+    against the two-pass kernels: same bytes, same meta; repeated calls reuse the workspace slots."""
+    g = torch.Generator().manual_seed(n % 1000)
+    x = (torch.randn(n, generator=g) * 5).to(dtype).cuda()
+    x[n // 3] = 300.0
+    for fp8_dt in (5, 6):
+        s1, si1, am1 = make_meta(scale=2.0)
+        q1 = be.cast_to_fp8_intime(x, s1, am1[0:1], si1, fp8_dt)
+        s2, si2, am2 = make_meta(scale=2.0)
+        q2 = be.cast_to_fp8_intime(x, s2, am2[0:1], si2, fp8_dt, two_pass=True)
+        assert torch.equal(q1, q2)
+        assert same_float(am1, am2) and same_float(s1, s2) and same_float(si1, si2)
+        assert am1[0].item() == 300.0
+
+
+def test_in_time_cast_on_a_second_stream(be):
+    """Only one stream per device runs the one-pass kernel; another stream gets the same answer."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1 << 20, generator=g).cuda()
+    s1, si1, am1 = make_meta()
+    q1 = be.cast_to_fp8_intime(x, s1, am1[0:1], si1, 5)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        s2, si2, am2 = make_meta()
+        q2 = be.cast_to_fp8_intime(x, s2, am2[0:1], si2, 5)
+    side.synchronize()
+    assert torch.equal(q1, q2) and same_float(am1, am2) and same_float(s1, s2) and same_float(si1, si2)
+
+
 def test_delayed_cast_accumulates_amax_and_skips_nan(be):
     g = torch.Generator().manual_seed(5)
     x = torch.randn(100000, generator=g).to(torch.bfloat16)
@@ -192,6 +225,18 @@ def test_fp8_transpose_is_involution_at_full_size(be):
     t = be.fp8_transpose(q)
     assert t.shape == (4096, 8192) and torch.equal(t, q.t().contiguous())
     assert torch.equal(be.fp8_transpose(t), q)
+
+
+@pytest.mark.parametrize('shape', [(16, 16), (144, 272), (4112, 48), (128, 128), (48, 1040), (130, 64), (64, 130)])
+def test_fp8_transpose_shapes(be, shape):
+    """Multiples of 16 take the 128x128-tile kernel (partial tiles at the edges), the rest the 64x64 one;
+    a misaligned view must not take the 16-byte path."""
+    g = torch.Generator().manual_seed(shape[0] + shape[1])
+    q = torch.randint(0, 256, shape, dtype=torch.uint8, generator=g).cuda()
+    assert torch.equal(be.fp8_transpose(q), q.t().contiguous())
+    flat = torch.randint(0, 256, (shape[0] * shape[1] + 1,), dtype=torch.uint8, generator=g).cuda()
+    view = flat[1:].view(shape)
+    assert torch.equal(be.fp8_transpose(view), view.t().contiguous())
 
 
 def test_scaled_16bit_payloads(be):
