@@ -79,11 +79,30 @@ int msamp_cast_to_fp8(const void* x, int in_dtype, size_t n, const float* scale,
 
 /* In-time cast: the whole of TypeCast.cast_to_fp8's in-time branch (cast.py:33-62) --
  * amax[0] = max|x|, *scale = rule(amax[0], *scale, fp_max(fp8_type), margin), quantize,
- * *scale_inv = 1 / *scale.  Two passes over x; the second runs back to front so that it
- * meets the cache lines the first pass left behind. */
+ * *scale_inv = 1 / *scale.  A tensor of up to 64 MiB (16-byte aligned) is read once by a
+ * kernel that holds it in registers while its workgroups agree on the amax; that kernel runs on
+ * one stream per device (the first to ask) and can be switched off with MSAMP_FLAG_TWO_PASS or
+ * MSAMP_INTIME_MODE=0 in the environment.  Otherwise two passes over x, the second back to
+ * front so that it meets the cache lines the first left behind.  Same results either way. */
 int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
                              uint8_t* out, int fp8_type, int margin, int flags, void* workspace,
                              msamp_stream_t stream);
+
+/* ScalingTensor.cast from a scaled 16/32-bit payload to FP8 (msamp/common/tensor/tensor.py:223-265):
+ * x holds value * old_scale and *amax = max|value| is known, so no reduction is needed:
+ * s = rule(*amax, 1, fp_max(fp8_type), margin); out[i] = fp8_sat_rne(float(x[i]) * (s * *old_scale_inv));
+ * *scale = s * *old_scale_inv; *scale_inv = 1 / s. */
+int msamp_cast_scaled_to_fp8(const void* x, int in_dtype, size_t n, const float* amax, const float* old_scale_inv,
+                             float* scale, float* scale_inv, uint8_t* out, int fp8_type, int margin,
+                             msamp_stream_t stream);
+
+/* TypeCast.cast_to_fp8 with the warm-up test of ScalingMeta.is_in_time_scaling (meta.py:58-72,
+ * cast.py:33) taken on the device: while *warmup_counter < window the call is the in-time cast,
+ * afterwards the delayed one (stored scale, max|x| folded into amax[0]).  The host needs no copy of
+ * the counter, so a training step has no device-to-host synchronisation. */
+int msamp_cast_to_fp8_gated(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
+                            uint8_t* out, int fp8_type, int margin, int flags, const int32_t* warmup_counter, int window,
+                            void* workspace, msamp_stream_t stream);
 
 /* tex.cast_from_fp8 (transformer_engine_wrapper.py:123-137): out[i] = otype(float(q[i]) * *scale_inv). */
 int msamp_cast_from_fp8(const uint8_t* q, int fp8_type, size_t n, const float* scale_inv, void* out, int out_dtype,
@@ -99,6 +118,11 @@ int msamp_cast_transpose_intime(const void* x, int in_dtype, int rows, int cols,
                                 float* scale_inv, uint8_t* out, uint8_t* out_t, int fp8_type, int margin, int flags,
                                 void* workspace, msamp_stream_t stream);
 
+/* msamp_cast_transpose with the same device-side warm-up test as msamp_cast_to_fp8_gated. */
+int msamp_cast_transpose_gated(const void* x, int in_dtype, int rows, int cols, float* scale, float* amax,
+                               float* scale_inv, uint8_t* out, uint8_t* out_t, int fp8_type, int margin, int flags,
+                               const int32_t* warmup_counter, int window, void* workspace, msamp_stream_t stream);
+
 /* tex.fp8_transpose (transformer_engine_wrapper.py:165-176): out[c][r] = q[r][c]. */
 int msamp_fp8_transpose(const uint8_t* q, int rows, int cols, uint8_t* out, msamp_stream_t stream);
 
@@ -107,11 +131,12 @@ int msamp_fp8_transpose(const uint8_t* q, int rows, int cols, uint8_t* out, msam
 int msamp_scale_cast(const void* x, int in_dtype, size_t n, const float* scale, void* out, int out_dtype,
                      msamp_stream_t stream);
 
-/* Device part of LBOptimizer._update_scaling_factors (optimizer.py:91-108) on flattened metas:
- * scales (n), amaxs (n x window, row-major).  bad[i] (nullable, n bytes) = 1 where amaxs[i][0]
- * was not finite (the caller resets that meta's host-side counter). */
-int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int n, int window, float fp_max, int margin,
-                       msamp_stream_t stream);
+/* LBOptimizer._update_scaling_factors (optimizer.py:83-108) on flattened metas: scales (n),
+ * amaxs (n x window, row-major).  A non-finite amaxs[i][0] is dropped, the scale comes from the
+ * window maximum, the window shifts.  bad[i] (nullable, n bytes) = 1 where amaxs[i][0] was not
+ * finite; counters[i] (nullable, n int32 on the device) += 1, or = 0 where bad. */
+int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int32_t* counters, int n, int window, float fp_max,
+                       int margin, msamp_stream_t stream);
 
 /* tex.te_gemm as Gemm.fp8_gemm calls it (gemm.py:121-144; transa=True, transb=False):
  * D[N][M] = (B[N][K] . A[M][K]^T) * *a_scale_inv * *b_scale_inv (+ bias[M]) (+ D if accumulate).

@@ -67,7 +67,20 @@ struct InTimeArgs {
     float fp_max;
     int margin;
     int flags;
+    const float* known_amax;       // kRescale: amax of the real values, already known
+    const float* old_scale_inv;    // kRescale: reciprocal scale of the stored payload
 };
+
+// Warm-up gate: the amax kernels of a gated cast run only while *counter < window (in-time scaling);
+// once the window is full they return at once and the cast that follows uses the stored scale.
+struct Gate {
+    const int32_t* counter;    // nullptr: always run
+    int window;
+};
+__device__ __forceinline__ bool gate_closed(const Gate& g) { return g.counter != nullptr && *g.counter >= g.window; }
+
+// where cast_to_fp8_kernel takes its scale from
+enum ScaleSource { kGivenScale = 0, kInTime = 1, kRescale = 2 };
 
 // every workgroup of the second pass derives the same amax and scale from the partial maxima
 __device__ __forceinline__ float resolve_in_time_scale(const InTimeArgs& a, uint32_t* red, float* scale_inv) {
@@ -94,18 +107,31 @@ __device__ __forceinline__ float resolve_in_time_scale(const InTimeArgs& a, uint
     return s_scale;
 }
 
-template <typename IT, int FMT, bool WITH_AMAX, bool INTIME>
-__global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __restrict__ x,
+// kRescale: the payload holds value * old_scale and max|value| is known, so the new scale is the rule of
+// that amax (fallback 1), the payload is multiplied by new_scale * old_scale_inv, and the meta gets
+// scale = that factor, scale_inv = 1 / new_scale.
+// Every workgroup ends with one atomic on the amax cell, and atomics on one address are served one
+// at a time (about 10 ns each): the launch with WITH_AMAX uses few, large workgroups (THREADS = 512,
+// two per CU) so that they stay a small part of the run time.
+template <typename IT, int FMT, bool WITH_AMAX, int INTIME, int THREADS = kCastThreads>
+__global__ __launch_bounds__(THREADS) void cast_to_fp8_kernel(const IT* __restrict__ x,
                                                                     uint8_t* __restrict__ out, size_t n,
                                                                     const float* __restrict__ scale_p, float* amax,
                                                                     float* scale_inv, int vec_ok, int reverse,
                                                                     InTimeArgs it) {
     constexpr int EPT = In16<IT>::EPT;
-    constexpr size_t TILE = static_cast<size_t>(kCastThreads) * EPT * kCastUnroll;
-    __shared__ uint32_t red[kCastThreads / kWave];
+    constexpr size_t TILE = static_cast<size_t>(THREADS) * EPT * kCastUnroll;
+    __shared__ uint32_t red[THREADS / kWave];
     float s;
-    if constexpr (INTIME) {
+    if constexpr (INTIME == kInTime) {
         s = resolve_in_time_scale(it, red, scale_inv);
+    } else if constexpr (INTIME == kRescale) {
+        const float s_new = scale_rule(*it.known_amax, 1.0f, it.fp_max, it.margin);
+        s = s_new * *it.old_scale_inv;
+        if (blockIdx.x == 0 && threadIdx.x == 0) {
+            *it.scale_out = s;
+            *scale_inv = 1.0f / s_new;
+        }
     } else {
         s = *scale_p;
     }
@@ -119,7 +145,7 @@ __global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __r
             float v[kCastUnroll][EPT];
 #pragma unroll
             for (int u = 0; u < kCastUnroll; ++u)
-                In16<IT>::load(x + base + (static_cast<size_t>(u) * kCastThreads + tid) * EPT, v[u]);
+                In16<IT>::load(x + base + (static_cast<size_t>(u) * THREADS + tid) * EPT, v[u]);
 #pragma unroll
             for (int u = 0; u < kCastUnroll; ++u) {
                 uint32_t w[EPT / 4];
@@ -129,7 +155,7 @@ __global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __r
                     if (WITH_AMAX) mx = fmaxf(fmaxf(mx, fabsf(a)), fmaxf(fmaxf(fabsf(b), fabsf(c)), fabsf(d)));
                     w[j] = quant4<FMT>(a * s, b * s, c * s, d * s);
                 }
-                uint8_t* o = out + base + (static_cast<size_t>(u) * kCastThreads + tid) * EPT;
+                uint8_t* o = out + base + (static_cast<size_t>(u) * THREADS + tid) * EPT;
                 if constexpr (EPT == 4) {
                     *reinterpret_cast<uint32_t*>(o) = w[0];
                 } else {
@@ -138,7 +164,7 @@ __global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __r
             }
         } else {
             const size_t end = (base + TILE < n) ? base + TILE : n;
-            for (size_t i = base + tid; i < end; i += kCastThreads) {
+            for (size_t i = base + tid; i < end; i += THREADS) {
                 const float a = Elem<IT>::load(x + i);
                 if (WITH_AMAX) mx = fmaxf(mx, fabsf(a));
                 out[i] = static_cast<uint8_t>(quant1<FMT>(a * s));
@@ -149,7 +175,7 @@ __global__ __launch_bounds__(kCastThreads) void cast_to_fp8_kernel(const IT* __r
         uint32_t m = block_max_u32(__float_as_uint(mx), red);
         if (tid == 0) amax_publish(amax, __uint_as_float(m));
     }
-    if constexpr (!INTIME) {
+    if constexpr (INTIME == kGivenScale) {
         if (scale_inv != nullptr && blockIdx.x == 0 && tid == 0) *scale_inv = 1.0f / s;
     }
 }
@@ -161,7 +187,8 @@ __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b 
 
 template <typename IT>
 __global__ __launch_bounds__(kCastThreads) void amax_partial_kernel(const IT* __restrict__ x, size_t n, uint32_t* ws,
-                                                                     const float* scale, int vec_ok) {
+                                                                     const float* scale, int vec_ok, Gate gate) {
+    if (gate_closed(gate)) return;
     constexpr int EPT = 16 / sizeof(IT);
     constexpr int UNROLL = 8;
     constexpr size_t TILE = static_cast<size_t>(kCastThreads) * EPT * UNROLL;
@@ -217,7 +244,8 @@ __global__ __launch_bounds__(kCastThreads) void amax_partial_kernel(const IT* __
 // reduce the partial maxima into amax[0] (and, if asked, run the scale rule) in one workgroup
 __global__ __launch_bounds__(kCastThreads) void amax_finalize_kernel(const uint32_t* ws, float* amax, float* scale,
                                                                       float* scale_inv, float fp_max, int margin, int flags,
-                                                                      int update_scale) {
+                                                                      int update_scale, Gate gate) {
+    if (gate_closed(gate)) return;
     __shared__ uint32_t red[kCastThreads / kWave];
     const int np = static_cast<int>(ws[1]);
     uint32_t m = 0;
@@ -608,6 +636,101 @@ __global__ __launch_bounds__(kCastThreads) void byte_transpose128_kernel(const u
 }
 
 // ---------------------------------------------------------------------------------------------
+// Cast + transpose with 16-byte loads and 128x128 tiles, for R % 16 == 0, C % 16 == 0 and 16-byte
+// aligned pointers.  A workgroup walks tiles in a grid-stride loop: it quantizes eight 16-byte loads
+// per lane at a time, writes the row-major bytes, parks them in LDS (same rotated layout as the byte
+// transpose), then each lane gathers a 4-byte-wide, 16-row strip, transposes its 4x4 byte blocks and
+// writes 16 bytes of four output rows.  Few long-lived workgroups mean few atomics on the amax cell.
+template <typename IT, int FMT, bool WITH_AMAX>
+__global__ __launch_bounds__(kCastThreads) void cast_transpose128_kernel(const IT* __restrict__ x,
+                                                                          uint8_t* __restrict__ out,
+                                                                          uint8_t* __restrict__ out_t, int R, int C,
+                                                                          const float* __restrict__ scale_p,
+                                                                          float* amax, float* scale_inv, int tiles_x,
+                                                                          int ntiles) {
+    constexpr int EPT = 16 / sizeof(IT);          // elements per 16-byte load: 8 or 4
+    constexpr int TPR = 128 / EPT;                // lanes per tile row: 16 or 32
+    constexpr int RPP = kCastThreads / TPR;       // rows per pass: 16 or 8
+    constexpr int PASSES = 128 / RPP;             // 8 or 16
+    constexpr int UNROLL = 8;
+    __shared__ uint4 tile[128 * 8];
+    __shared__ uint32_t red[kCastThreads / kWave];
+    uint32_t* words = reinterpret_cast<uint32_t*>(tile);
+    const int tid = threadIdx.x;
+    const float s = *scale_p;
+    float mx = 0.0f;
+    const int lc = tid % TPR, lr = tid / TPR;     // this lane's column group and row within a pass
+    const int g = tid & 7, w = tid >> 3;          // transposed side: rows 16g..16g+15, byte columns 4w..4w+3
+    for (int t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const int r0 = (t / tiles_x) * 128, c0 = (t % tiles_x) * 128;
+        const bool col_ok = c0 + lc * EPT < C;
+#pragma unroll
+        for (int p0 = 0; p0 < PASSES; p0 += UNROLL) {
+            uint4 v[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int row = (p0 + u) * RPP + lr;
+                v[u] = make_uint4(0, 0, 0, 0);
+                if (col_ok && r0 + row < R)
+                    v[u] = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(r0 + row) * C + c0 + lc * EPT);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const int row = (p0 + u) * RPP + lr;
+                float f[EPT];
+                In16<IT>::decode(v[u], f);
+                uint32_t q[EPT / 4];
+#pragma unroll
+                for (int j = 0; j < EPT / 4; ++j) {
+                    const float a = f[4 * j], b = f[4 * j + 1], c = f[4 * j + 2], d = f[4 * j + 3];
+                    if (WITH_AMAX) mx = fmaxf(fmaxf(mx, fabsf(a)), fmaxf(fmaxf(fabsf(b), fabsf(c)), fabsf(d)));
+                    q[j] = quant4<FMT>(a * s, b * s, c * s, d * s);
+                }
+                const bool ok = col_ok && r0 + row < R;
+                const int word = lc * (EPT / 4);    // word column of this lane's bytes within the tile row
+                const int pw = ((((word >> 2) + (row >> 4) + (row & 7)) & 7) << 2) | (word & 3);
+                if constexpr (EPT == 8) {
+                    if (ok && out != nullptr)
+                        *reinterpret_cast<uint2*>(out + static_cast<size_t>(r0 + row) * C + c0 + lc * EPT) = make_uint2(q[0], q[1]);
+                    *reinterpret_cast<uint2*>(words + row * 32 + pw) = make_uint2(q[0], q[1]);
+                } else {
+                    if (ok && out != nullptr)
+                        *reinterpret_cast<uint32_t*>(out + static_cast<size_t>(r0 + row) * C + c0 + lc * EPT) = q[0];
+                    words[row * 32 + pw] = q[0];
+                }
+            }
+        }
+        __syncthreads();
+        uint32_t o[4][4];    // o[q][i]: column 4w+i, rows 16g+4q..+3
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t a[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int k = 4 * q + j, row = 16 * g + k;
+                a[j] = words[row * 32 + ((w + 4 * (g + (k & 7))) & 31)];
+            }
+            transpose4x4_bytes(a[0], a[1], a[2], a[3], o[q]);
+        }
+        if (r0 + 16 * g < R) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = c0 + 4 * w + i;
+                if (c < C)
+                    *reinterpret_cast<uint4*>(out_t + static_cast<size_t>(c) * R + r0 + 16 * g) =
+                        make_uint4(o[0][i], o[1][i], o[2][i], o[3][i]);
+            }
+        }
+        __syncthreads();    // the tile is free for the next round
+    }
+    if constexpr (WITH_AMAX) {
+        uint32_t m = block_max_u32(__float_as_uint(mx), red);
+        if (tid == 0) amax_publish(amax, __uint_as_float(m));
+    }
+    if (scale_inv != nullptr && blockIdx.x == 0 && tid == 0) *scale_inv = 1.0f / s;
+}
+
+// ---------------------------------------------------------------------------------------------
 __global__ void scaling_factor_kernel(const float* amax, const float* scale_in, int scale_in_n, float* scale_out, int n,
                                       float fp_max, int margin) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -616,8 +739,8 @@ __global__ void scaling_factor_kernel(const float* amax, const float* scale_in, 
 
 __device__ __forceinline__ float nanmax(float a, float b) { return (a != a) ? a : ((b != b) ? b : fmaxf(a, b)); }
 
-__global__ void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad, int n, int window, float fp_max,
-                                    int margin) {
+__global__ void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad, int32_t* counters, int n, int window,
+                                    float fp_max, int margin) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float* row = amaxs + static_cast<size_t>(i) * window;
@@ -632,6 +755,7 @@ __global__ void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad, i
     row[0] = 0.0f;
     scales[i] = sf;
     if (bad != nullptr) bad[i] = is_bad ? 1 : 0;
+    if (counters != nullptr) counters[i] = is_bad ? 0 : counters[i] + 1;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -648,19 +772,30 @@ static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, f
     constexpr int EPT = In16<IT>::EPT;
     const int vec_ok = aligned(x, 16) && aligned(out, EPT);
     int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * kCastUnroll);
-    const InTimeArgs none = {nullptr, nullptr, nullptr, 0.0f, 0, 0};
+    const InTimeArgs none = {nullptr, nullptr, nullptr, 0.0f, 0, 0, nullptr, nullptr};
 #define LAUNCH(FMT, AM, INT) \
-    hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, AM, INT>), dim3(grid), dim3(kCastThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, INT ? 1 : 0, INT ? *it : none)
-    if (it != nullptr) {
+    hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, AM, INT>), dim3(grid), dim3(kCastThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, INT == kInTime ? 1 : 0, INT != kGivenScale ? *it : none)
+    if (it != nullptr && it->known_amax != nullptr) {
+        if (fp8_type == MSAMP_DT_E4M3) LAUNCH(MSAMP_DT_E4M3, false, kRescale); else LAUNCH(MSAMP_DT_E5M2, false, kRescale);
+    } else if (it != nullptr) {
         // second pass of an in-time cast: fewer, longer-lived workgroups (each one re-derives the scale),
         // walking the tensor back to front to meet what the first pass left in the caches
         const int cap = cu_count() * 4;
         grid = grid < cap ? grid : cap;
-        if (fp8_type == MSAMP_DT_E4M3) LAUNCH(MSAMP_DT_E4M3, false, true); else LAUNCH(MSAMP_DT_E5M2, false, true);
+        if (fp8_type == MSAMP_DT_E4M3) LAUNCH(MSAMP_DT_E4M3, false, kInTime); else LAUNCH(MSAMP_DT_E5M2, false, kInTime);
+    } else if (amax != nullptr) {
+        constexpr int kAmaxThreads = 512;
+        int g2 = grid_for(n, static_cast<size_t>(kAmaxThreads) * EPT * kCastUnroll);
+        const int cap = cu_count() * 2;
+        g2 = g2 < cap ? g2 : cap;
+#define LAUNCH_AMAX(FMT) \
+    hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, true, kGivenScale, kAmaxThreads>), dim3(g2), dim3(kAmaxThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, 0, none)
+        if (fp8_type == MSAMP_DT_E4M3) LAUNCH_AMAX(MSAMP_DT_E4M3); else LAUNCH_AMAX(MSAMP_DT_E5M2);
+#undef LAUNCH_AMAX
     } else if (fp8_type == MSAMP_DT_E4M3) {
-        if (amax) LAUNCH(MSAMP_DT_E4M3, true, false); else LAUNCH(MSAMP_DT_E4M3, false, false);
+        LAUNCH(MSAMP_DT_E4M3, false, kGivenScale);
     } else {
-        if (amax) LAUNCH(MSAMP_DT_E5M2, true, false); else LAUNCH(MSAMP_DT_E5M2, false, false);
+        LAUNCH(MSAMP_DT_E5M2, false, kGivenScale);
     }
 #undef LAUNCH
     MSAMP_CHECK_LAUNCH("cast_to_fp8_kernel");
@@ -668,27 +803,30 @@ static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, f
 }
 
 template <typename IT>
-static int launch_amax(const IT* x, size_t n, uint32_t* ws, const float* scale, hipStream_t st) {
+static int launch_amax(const IT* x, size_t n, uint32_t* ws, const float* scale, Gate gate, hipStream_t st) {
     constexpr int EPT = 16 / sizeof(IT);
     const int vec_ok = aligned(x, 16);
     int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * 8);
     const int cap = cu_count() * 4 < kMaxPartials ? cu_count() * 4 : kMaxPartials;
     grid = grid < cap ? grid : cap;
-    hipLaunchKernelGGL((amax_partial_kernel<IT>), dim3(grid), dim3(kCastThreads), 0, st, x, n, ws, scale, vec_ok);
+    hipLaunchKernelGGL((amax_partial_kernel<IT>), dim3(grid), dim3(kCastThreads), 0, st, x, n, ws, scale, vec_ok, gate);
     MSAMP_CHECK_LAUNCH("amax_partial_kernel");
     return MSAMP_OK;
 }
 
 // first pass: partial maxima of |x| into the workspace (plus the scale in force, for the rule's fallback)
-static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const float* scale, hipStream_t st) {
+constexpr Gate kNoGate = {nullptr, 0};
+
+static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const float* scale, hipStream_t st,
+                         Gate gate = kNoGate) {
     uint32_t* w = static_cast<uint32_t*>(ws);
     switch (dtype) {
         case MSAMP_DT_F32:
-            return launch_amax(static_cast<const float*>(x), n, w, scale, st);
+            return launch_amax(static_cast<const float*>(x), n, w, scale, gate, st);
         case MSAMP_DT_F16:
-            return launch_amax(static_cast<const f16_t*>(x), n, w, scale, st);
+            return launch_amax(static_cast<const f16_t*>(x), n, w, scale, gate, st);
         case MSAMP_DT_BF16:
-            return launch_amax(static_cast<const bf16_t*>(x), n, w, scale, st);
+            return launch_amax(static_cast<const bf16_t*>(x), n, w, scale, gate, st);
     }
     set_error("unsupported input dtype %d", dtype);
     return MSAMP_ERR_DTYPE;
@@ -784,9 +922,9 @@ static int dispatch_resident(const void* x, int dtype, size_t n, float* scale, f
 }
 
 static int finalize_amax(void* ws, float* amax, float* scale, float* scale_inv, float fp_max, int margin, int flags,
-                         int update_scale, hipStream_t st) {
+                         int update_scale, hipStream_t st, Gate gate = kNoGate) {
     hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(kCastThreads), 0, st, static_cast<const uint32_t*>(ws), amax, scale,
-                       scale_inv, fp_max, margin, flags, update_scale);
+                       scale_inv, fp_max, margin, flags, update_scale, gate);
     MSAMP_CHECK_LAUNCH("amax_finalize_kernel");
     return MSAMP_OK;
 }
@@ -812,6 +950,27 @@ static int launch_ct(const IT* x, int rows, int cols, const float* scale, float*
     const int vec_in = (cols % 4 == 0) && aligned(x, 4 * esz);
     const int vec_out = (cols % 4 == 0) && (out == nullptr || aligned(out, 4));
     const int vec_t = (rows % 4 == 0) && aligned(out_t, 4);
+    if constexpr (CAST) {
+        if (rows % 16 == 0 && cols % 16 == 0 && aligned(x, 16) && (out == nullptr || aligned(out, 16)) && aligned(out_t, 16)) {
+            const int tiles_x = (cols + 127) / 128;
+            const long long ntiles_ll = static_cast<long long>(tiles_x) * ((rows + 127) / 128);
+            if (ntiles_ll <= 0x7fffffffLL) {
+                const int ntiles = static_cast<int>(ntiles_ll);
+                const int cap = cu_count() * 2;
+                const int g = ntiles < cap ? ntiles : cap;
+#define LAUNCH128(FMT, AM) \
+    hipLaunchKernelGGL((cast_transpose128_kernel<IT, FMT, AM>), dim3(g), dim3(kCastThreads), 0, st, x, out, out_t, rows, cols, scale, amax, scale_inv, tiles_x, ntiles)
+                if (fp8_type == MSAMP_DT_E4M3) {
+                    if (amax) LAUNCH128(MSAMP_DT_E4M3, true); else LAUNCH128(MSAMP_DT_E4M3, false);
+                } else {
+                    if (amax) LAUNCH128(MSAMP_DT_E5M2, true); else LAUNCH128(MSAMP_DT_E5M2, false);
+                }
+#undef LAUNCH128
+                MSAMP_CHECK_LAUNCH("cast_transpose128_kernel");
+                return MSAMP_OK;
+            }
+        }
+    }
     dim3 grid((cols + 63) / 64, (rows + 63) / 64);
     MSAMP_REQUIRE(grid.y <= 65535u, MSAMP_ERR_SHAPE, "too many rows for one launch: %d", rows);
 #define LAUNCH(FMT, AM) \
@@ -911,8 +1070,19 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
     if (rc <= 0) return rc;
     rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
     if (rc != MSAMP_OK) return rc;
-    const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags};
+    const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags, nullptr, nullptr};
     return dispatch_cast(x, in_dtype, n, scale, nullptr, scale_inv, out, fp8_type, &it, st);
+}
+
+int msamp_cast_scaled_to_fp8(const void* x, int in_dtype, size_t n, const float* amax, const float* old_scale_inv,
+                             float* scale, float* scale_inv, uint8_t* out, int fp8_type, int margin,
+                             msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_scaled_to_fp8: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_scaled_to_fp8: in_dtype %d", in_dtype);
+    MSAMP_REQUIRE(amax && old_scale_inv && scale && scale_inv && ((x && out) || n == 0), MSAMP_ERR_NULL,
+                  "msamp_cast_scaled_to_fp8: null pointer");
+    const InTimeArgs it = {nullptr, scale, nullptr, fp8_max(fp8_type), margin, 0, amax, old_scale_inv};
+    return dispatch_cast(x, in_dtype, n, nullptr, nullptr, scale_inv, out, fp8_type, &it, static_cast<hipStream_t>(stream));
 }
 
 int msamp_cast_from_fp8(const uint8_t* q, int fp8_type, size_t n, const float* scale_inv, void* out, int out_dtype,
@@ -968,6 +1138,44 @@ int msamp_cast_transpose_intime(const void* x, int in_dtype, int rows, int cols,
     return dispatch_ct(x, in_dtype, rows, cols, scale, nullptr, nullptr, out, out_t, fp8_type, st);
 }
 
+int msamp_cast_to_fp8_gated(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
+                            uint8_t* out, int fp8_type, int margin, int flags, const int32_t* warmup_counter, int window,
+                            void* workspace, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_to_fp8_gated: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_to_fp8_gated: in_dtype %d", in_dtype);
+    MSAMP_REQUIRE(scale && amax && scale_inv && warmup_counter && ((x && out) || n == 0), MSAMP_ERR_NULL,
+                  "msamp_cast_to_fp8_gated: null pointer");
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_to_fp8_gated: workspace required");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const Gate gate = {warmup_counter, window};
+    // while warming up: amax[0] and the scale from this tensor; afterwards both kernels return at once
+    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st, gate);
+    if (rc != MSAMP_OK) return rc;
+    rc = finalize_amax(workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st, gate);
+    if (rc != MSAMP_OK) return rc;
+    // the delayed cast serves both cases: folding max|x| into an amax[0] that already holds it changes nothing
+    return dispatch_cast(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, nullptr, st);
+}
+
+int msamp_cast_transpose_gated(const void* x, int in_dtype, int rows, int cols, float* scale, float* amax,
+                               float* scale_inv, uint8_t* out, uint8_t* out_t, int fp8_type, int margin, int flags,
+                               const int32_t* warmup_counter, int window, void* workspace, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_transpose_gated: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_transpose_gated: in_dtype %d", in_dtype);
+    MSAMP_REQUIRE(rows >= 0 && cols >= 0, MSAMP_ERR_SHAPE, "msamp_cast_transpose_gated: shape %d x %d", rows, cols);
+    MSAMP_REQUIRE(scale && amax && scale_inv && warmup_counter, MSAMP_ERR_NULL, "msamp_cast_transpose_gated: null meta pointer");
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_transpose_gated: workspace required");
+    MSAMP_REQUIRE((x && out_t) || rows == 0 || cols == 0, MSAMP_ERR_NULL, "msamp_cast_transpose_gated: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t n = static_cast<size_t>(rows) * cols;
+    const Gate gate = {warmup_counter, window};
+    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st, gate);
+    if (rc != MSAMP_OK) return rc;
+    rc = finalize_amax(workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st, gate);
+    if (rc != MSAMP_OK || n == 0) return rc;
+    return dispatch_ct(x, in_dtype, rows, cols, scale, amax, scale_inv, out, out_t, fp8_type, st);
+}
+
 int msamp_fp8_transpose(const uint8_t* q, int rows, int cols, uint8_t* out, msamp_stream_t stream) {
     MSAMP_REQUIRE(rows >= 0 && cols >= 0, MSAMP_ERR_SHAPE, "msamp_fp8_transpose: shape %d x %d", rows, cols);
     if (rows == 0 || cols == 0) return MSAMP_OK;
@@ -998,13 +1206,13 @@ int msamp_scale_cast(const void* x, int in_dtype, size_t n, const float* scale, 
     }
 }
 
-int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int n, int window, float fp_max, int margin,
-                       msamp_stream_t stream) {
+int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int32_t* counters, int n, int window, float fp_max,
+                       int margin, msamp_stream_t stream) {
     MSAMP_REQUIRE(n >= 0 && window >= 1, MSAMP_ERR_SHAPE, "msamp_scale_update: n=%d window=%d", n, window);
     if (n == 0) return MSAMP_OK;
     MSAMP_REQUIRE(scales && amaxs, MSAMP_ERR_NULL, "msamp_scale_update: null pointer");
     hipLaunchKernelGGL(scale_update_kernel, dim3((n + 63) / 64), dim3(64), 0, static_cast<hipStream_t>(stream), scales,
-                       amaxs, bad, n, window, fp_max, margin);
+                       amaxs, bad, counters, n, window, fp_max, margin);
     MSAMP_CHECK_LAUNCH("scale_update_kernel");
     return MSAMP_OK;
 }

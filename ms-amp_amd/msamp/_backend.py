@@ -34,12 +34,15 @@ _SIGNATURES = {
     'msamp_compute_scaling_factor': ([_vp, _vp, _i, _vp, _i, _f, _i, _vp], _i),
     'msamp_cast_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp], _i),
     'msamp_cast_to_fp8_intime': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
+    'msamp_cast_scaled_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], _i),
     'msamp_cast_from_fp8': ([_vp, _i, _sz, _vp, _vp, _i, _vp], _i),
     'msamp_cast_transpose': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp], _i),
     'msamp_cast_transpose_intime': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
     'msamp_fp8_transpose': ([_vp, _i, _i, _vp, _vp], _i),
     'msamp_scale_cast': ([_vp, _i, _sz, _vp, _vp, _i, _vp], _i),
-    'msamp_scale_update': ([_vp, _vp, _vp, _i, _i, _f, _i, _vp], _i),
+    'msamp_scale_update': ([_vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp], _i),
+    'msamp_cast_to_fp8_gated': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp], _i),
+    'msamp_cast_transpose_gated': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp], _i),
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
@@ -91,7 +94,8 @@ def _ptr(t):
 
 
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    """Raw handle of torch's current stream on the current device."""
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())
 
 
 def _dt(t):
@@ -135,13 +139,19 @@ def compute_scaling_factor(amax_t, scale_t, fp_max, margin):
     return out
 
 
-def scale_update(scales, amaxs, fp_max, margin):
-    """In-place window update of flattened metas; returns the uint8 mask of non-finite current amaxs."""
+def scale_update(scales, amaxs, fp_max, margin, counters=None, want_mask=True):
+    """In-place window update of flattened metas.  `counters` (int32 on the GPU) are bumped, or reset where
+    the current amax was not finite; returns the uint8 mask of those entries if asked for."""
     lib = load()
     _gpu(scales, 'scales')
     n, window = amaxs.shape
-    bad = torch.empty(n, dtype=torch.uint8, device=scales.device)
-    _check(lib.msamp_scale_update(_ptr(scales), _ptr(amaxs), _ptr(bad), n, window, fp_max, margin, _stream()), 'msamp_scale_update')
+    if counters is not None:
+        _gpu(counters, 'counters')
+    bad = torch.empty(n, dtype=torch.uint8, device=scales.device) if want_mask else None
+    _check(
+        lib.msamp_scale_update(_ptr(scales), _ptr(amaxs), _ptr(bad), _ptr(counters), n, window, fp_max, margin, _stream()),
+        'msamp_scale_update'
+    )
     return bad
 
 
@@ -169,6 +179,35 @@ def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_
             (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass else 0), _ptr(workspace(x.device)),
             _stream()
         ), 'msamp_cast_to_fp8_intime'
+    )
+    return out
+
+
+def cast_to_fp8_gated(x, scale, amax_cell, scale_inv, fp8_dt, counter, window, margin=0, nan_to_inf=False):
+    """In-time cast while counter < window, delayed cast afterwards; the test runs on the GPU."""
+    lib = load()
+    _gpu(x, 'input')
+    _gpu(counter, 'warm-up counter')
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _check(
+        lib.msamp_cast_to_fp8_gated(
+            _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
+            FLAG_NAN_TO_INF if nan_to_inf else 0, _ptr(counter), window, _ptr(workspace(x.device)), _stream()
+        ), 'msamp_cast_to_fp8_gated'
+    )
+    return out
+
+
+def cast_scaled_to_fp8(x, amax_cell, old_scale_inv, scale, scale_inv, fp8_dt, margin=0):
+    """Requantize a scaled 16/32-bit payload whose amax is known; writes scale and scale_inv."""
+    lib = load()
+    _gpu(x, 'input')
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    _check(
+        lib.msamp_cast_scaled_to_fp8(
+            _ptr(x), _dt(x), x.numel(), _ptr(amax_cell), _ptr(old_scale_inv), _ptr(scale), _ptr(scale_inv), _ptr(out),
+            fp8_dt, margin, _stream()
+        ), 'msamp_cast_scaled_to_fp8'
     )
     return out
 
@@ -201,6 +240,22 @@ def cast_transpose(x, scale, amax_cell, scale_inv, fp8_dt, in_time=False, margin
             _stream()
         )
     _check(rc, 'msamp_cast_transpose')
+    return out, out_t
+
+
+def cast_transpose_gated(x, scale, amax_cell, scale_inv, fp8_dt, counter, window, margin=0, nan_to_inf=False):
+    lib = load()
+    _gpu(x, 'input')
+    _gpu(counter, 'warm-up counter')
+    rows, cols = x.shape
+    out = torch.empty((rows, cols), dtype=torch.uint8, device=x.device)
+    out_t = torch.empty((cols, rows), dtype=torch.uint8, device=x.device)
+    _check(
+        lib.msamp_cast_transpose_gated(
+            _ptr(x), _dt(x), rows, cols, _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), _ptr(out_t), fp8_dt,
+            margin, FLAG_NAN_TO_INF if nan_to_inf else 0, _ptr(counter), window, _ptr(workspace(x.device)), _stream()
+        ), 'msamp_cast_transpose_gated'
+    )
     return out, out_t
 
 

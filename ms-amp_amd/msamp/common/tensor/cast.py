@@ -38,8 +38,21 @@ class TypeCast:
         if input.dtype in (torch.uint8, torch.int8):
             raise ValueError('The input tensor is already quantized.')
         fp8_dt = int(meta.qtype)
-        in_time = meta.is_in_time_scaling()
         amax0 = meta.amax[0:1]
+        mode = meta.scaling_mode()
+        if mode == 'gated':
+            if not sync:
+                if fuse_transpose:
+                    if input.dim() != 2:
+                        raise ValueError('fuse_transpose needs a 2-D input.')
+                    return _backend.cast_transpose_gated(
+                        input, meta.scale, amax0, meta.scale_inv, fp8_dt, meta.amax_counter, meta.window_size
+                    )
+                return _backend.cast_to_fp8_gated(
+                    input, meta.scale, amax0, meta.scale_inv, fp8_dt, meta.amax_counter, meta.window_size
+                )
+            mode = 'in_time' if bool(meta.is_warmup()) else 'delayed'    # sync=True: decide on the host
+        in_time = mode == 'in_time'
         fused_in_time = in_time and not (sync and _world_size() > 1)
         sync_amax = None
         if not fused_in_time:

@@ -11,9 +11,11 @@ from msamp.common.dtype import Floating, Dtypes
 class ScalingMeta:
     """Scaling state of one quantized tensor.
 
-    scale, scale_inv: 0-d float32 on the GPU; amax: (window_size,) float32 on the GPU with
-    amax[0] the current value; amax_counter: 0-d int32 on the host, which is what lets the
-    warm-up / in-time decision be taken without a device synchronisation.
+    scale, scale_inv: 0-d float32; amax: (window_size,) float32 with amax[0] the current value;
+    amax_counter: 0-d int32 counting window updates.  All four live on the meta's device.  With the
+    counter on the GPU the casts take the warm-up test on the device (scaling_mode() == 'gated'), so
+    nothing in a training step waits for the GPU; is_warmup() / is_in_time_scaling() still answer on
+    the host, at the price of a synchronisation.
     """
     in_time_scaling: bool = True
 
@@ -22,7 +24,7 @@ class ScalingMeta:
         self.scale = scale if scale is not None else torch.ones((), device=device)
         self.scale_inv = scale_inv if scale_inv is not None else torch.ones((), device=device)
         self.amax = amax if amax is not None else torch.zeros((window_size, ), device=device)
-        self.amax_counter = torch.zeros((), dtype=torch.int32)
+        self.amax_counter = torch.zeros((), dtype=torch.int32, device=self.amax.device)
         self.window_size = window_size
         self.group = group
         self.locked = False
@@ -44,6 +46,16 @@ class ScalingMeta:
 
     def is_in_time_scaling(self):
         return ScalingMeta.in_time_scaling and (self.window_size == 1 or bool(self.is_warmup()))
+
+    def scaling_mode(self):
+        """'in_time', 'delayed', or 'gated' when only the GPU-resident counter can tell (no sync)."""
+        if not ScalingMeta.in_time_scaling:
+            return 'delayed'
+        if self.window_size == 1:
+            return 'in_time'
+        if self.amax_counter.is_cuda:
+            return 'gated'
+        return 'in_time' if bool(self.is_warmup()) else 'delayed'
 
     @staticmethod
     def in_time_scaling_context(enabled):
@@ -86,12 +98,14 @@ class ScalingMeta:
         self.scale = self.scale.cuda()
         self.scale_inv = self.scale_inv.cuda()
         self.amax = self.amax.cuda()
+        self.amax_counter = self.amax_counter.cuda()
         return self
 
     def cpu(self):
         self.scale = self.scale.cpu()
         self.scale_inv = self.scale_inv.cpu()
         self.amax = self.amax.cpu()
+        self.amax_counter = self.amax_counter.cpu()
         return self
 
     @property

@@ -192,14 +192,16 @@ class ScalingTensor:
             return self.float().cast(qtype)
         old = self.meta
         meta = ScalingMeta(qtype, amax=old.amax.clone(), window_size=old.window_size, device=old.amax.device)
+        if Dtypes.is_fp8_qtype(qtype):
+            # the whole recipe in one kernel
+            value = _backend.cast_scaled_to_fp8(
+                self.value.contiguous(), meta.amax, old.scale_inv, meta.scale, meta.scale_inv, int(qtype)
+            )
+            return ScalingTensor(value, meta)
         meta.reset_scaling_factor()
         scale_inv = torch.reciprocal(meta.scale)
         meta.scale.mul_(old.scale_inv)
-        value = self.value.contiguous()
-        if Dtypes.is_fp8_qtype(qtype):
-            value = _backend.cast_to_fp8(value, meta.scale, None, None, int(qtype))
-        else:
-            value = _backend.scale_cast(value, meta.scale, Dtypes.get_dtype_from_qtype(qtype))
+        value = _backend.scale_cast(self.value.contiguous(), meta.scale, Dtypes.get_dtype_from_qtype(qtype))
         meta.scale_inv.copy_(scale_inv)
         return ScalingTensor(value, meta)
 

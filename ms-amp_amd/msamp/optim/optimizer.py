@@ -52,21 +52,17 @@ class LBOptimizer(Optimizer):
             if not ScalingMeta.in_time_scaling:
                 names.append('wgrad')
         margin = 0
-        masks = []
         for name in names:
             meta = metas[name]
             fp_max = Floating.qfp_max[meta['qtype']]
-            masks.append(_backend.scale_update(meta['scales'], meta['amaxs'], fp_max, margin))
-        # the counters live on the host (they steer which cast kernel is enqueued next), so the
-        # non-finite masks come back in one device-to-host copy per step
-        bad = torch.cat(masks).cpu().bool()
-        offset = 0
-        for name in names:
-            counters = metas[name]['amax_counters']
-            n = counters.numel()
-            counters += 1
-            counters[bad[offset:offset + n]] = 0
-            offset += n
+            counters = meta['amax_counters']
+            if counters.is_cuda:
+                # counters live on the GPU and are updated by the same kernel: no device-to-host copy
+                _backend.scale_update(meta['scales'], meta['amaxs'], fp_max, margin, counters=counters, want_mask=False)
+            else:
+                bad = _backend.scale_update(meta['scales'], meta['amaxs'], fp_max, margin).cpu().bool()
+                counters += 1
+                counters[bad] = 0
 
     # ---- state (de)serialisation with order indices instead of tensors ---------------------------
     def state_dict(self):

@@ -157,6 +157,48 @@ def test_in_time_cast_on_a_second_stream(be):
     assert torch.equal(q1, q2) and same_float(am1, am2) and same_float(s1, s2) and same_float(si1, si2)
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('counter', [0, 3, 4, 100])
+def test_gated_casts_follow_the_device_counter(be, dtype, counter):
+    """Warm-up test on the GPU: counter < window -> the in-time cast, else the delayed cast; both byte
+    for byte, plain and with the fused transpose, NaN input included."""
+    window = 4
+    g = torch.Generator().manual_seed(counter)
+    x = (torch.randn(192, 320, generator=g) * 3).to(dtype)
+    x[5, 7] = float('nan')
+    xg = x.cuda()
+    cnt = torch.full((), counter, dtype=torch.int32, device='cuda')
+    in_time = counter < window
+    for fp8_dt in (5, 6):
+        s, si, am = make_meta(window=window, scale=2.0)
+        am[0] = 0.5
+        q = be.cast_to_fp8_gated(xg, s, am[0:1], si, fp8_dt, cnt, window)
+        s2, si2, am2 = make_meta(window=window, scale=2.0)
+        am2[0] = 0.5
+        if in_time:
+            want = be.cast_to_fp8_intime(xg, s2, am2[0:1], si2, fp8_dt)
+        else:
+            want = be.cast_to_fp8(xg, s2, am2[0:1], si2, fp8_dt)
+        assert torch.equal(q, want) and same_float(am, am2) and same_float(s, s2) and same_float(si, si2)
+        s, si, am = make_meta(window=window, scale=2.0)
+        q, qt = be.cast_transpose_gated(xg, s, am[0:1], si, fp8_dt, cnt, window)
+        s2, si2, am2 = make_meta(window=window, scale=2.0)
+        want, want_t = be.cast_transpose(xg, s2, am2[0:1], si2, fp8_dt, in_time=in_time)
+        assert torch.equal(q, want) and torch.equal(qt, want_t)
+        assert same_float(am, am2) and same_float(s, s2) and same_float(si, si2)
+    assert cnt.item() == counter
+
+
+def test_window_update_keeps_device_counters(be):
+    scales = torch.tensor([1.0, 2.0, 4.0], device='cuda')
+    amaxs = torch.tensor([[3.0, 1.0], [float('inf'), 2.0], [float('nan'), 0.0]], device='cuda')
+    counters = torch.tensor([5, 6, 7], dtype=torch.int32, device='cuda')
+    assert be.scale_update(scales, amaxs, 448.0, 0, counters=counters, want_mask=False) is None
+    assert counters.tolist() == [6, 0, 0]
+    assert amaxs.tolist() == [[0.0, 3.0], [0.0, 0.0], [0.0, 0.0]]
+    assert scales.tolist() == [128.0, 128.0, 4.0]
+
+
 def test_delayed_cast_accumulates_amax_and_skips_nan(be):
     g = torch.Generator().manual_seed(5)
     x = torch.randn(100000, generator=g).to(torch.bfloat16)
@@ -196,7 +238,7 @@ def test_in_time_nan_inf_and_sync_semantics(be):
     assert am[0].item() == 0.0 and s.item() == 4.0 and si.item() == 0.25 and q.sum().item() == 0
 
 
-@pytest.mark.parametrize('shape', [(64, 64), (100, 36), (17, 5), (1, 130), (257, 1), (512, 1024), (96, 4100)])
+@pytest.mark.parametrize('shape', [(64, 64), (100, 36), (17, 5), (1, 130), (257, 1), (512, 1024), (96, 4100), (144, 272), (4112, 48), (16, 1040)])
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
 def test_cast_transpose(be, shape, dtype):
     g = torch.Generator().manual_seed(shape[0] * 7 + shape[1])
