@@ -90,11 +90,12 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
 
 /* ScalingTensor.cast from a scaled 16/32-bit payload to FP8 (msamp/common/tensor/tensor.py:223-265):
  * x holds value * old_scale and *amax = max|value| is known, so no reduction is needed:
- * s = rule(*amax, 1, fp_max(fp8_type), margin); out[i] = fp8_sat_rne(float(x[i]) * (s * *old_scale_inv));
- * *scale = s * *old_scale_inv; *scale_inv = 1 / s. */
+ * s = rule(amax[0], 1, fp_max(fp8_type), margin); out[i] = fp8_sat_rne(float(x[i]) * (s * *old_scale_inv));
+ * *scale = s * *old_scale_inv; *scale_inv = 1 / s.  The rest of the new meta can be filled in the same
+ * launch: amax_out (nullable) receives amax[0..window), *counter_out (nullable) = 0. */
 int msamp_cast_scaled_to_fp8(const void* x, int in_dtype, size_t n, const float* amax, const float* old_scale_inv,
-                             float* scale, float* scale_inv, uint8_t* out, int fp8_type, int margin,
-                             msamp_stream_t stream);
+                             float* scale, float* scale_inv, float* amax_out, int window, int32_t* counter_out,
+                             uint8_t* out, int fp8_type, int margin, msamp_stream_t stream);
 
 /* TypeCast.cast_to_fp8 with the warm-up test of ScalingMeta.is_in_time_scaling (meta.py:58-72,
  * cast.py:33) taken on the device: while *warmup_counter < window the call is the in-time cast,

@@ -67,8 +67,11 @@ struct InTimeArgs {
     float fp_max;
     int margin;
     int flags;
-    const float* known_amax;       // kRescale: amax of the real values, already known
+    const float* known_amax;       // kRescale: amax window of the real values, already known
     const float* old_scale_inv;    // kRescale: reciprocal scale of the stored payload
+    float* amax_copy;              // kRescale, nullable: receives a copy of the amax window
+    int window;
+    int32_t* counter_out;          // kRescale, nullable: set to 0 (the new meta's update count)
 };
 
 // Warm-up gate: the amax kernels of a gated cast run only while *counter < window (in-time scaling);
@@ -131,6 +134,10 @@ __global__ __launch_bounds__(THREADS) void cast_to_fp8_kernel(const IT* __restri
         if (blockIdx.x == 0 && threadIdx.x == 0) {
             *it.scale_out = s;
             *scale_inv = 1.0f / s_new;
+            if (it.counter_out != nullptr) *it.counter_out = 0;
+        }
+        if (blockIdx.x == 0 && it.amax_copy != nullptr) {
+            for (int j = threadIdx.x; j < it.window; j += blockDim.x) it.amax_copy[j] = it.known_amax[j];
         }
     } else {
         s = *scale_p;
@@ -185,9 +192,22 @@ __global__ __launch_bounds__(THREADS) void cast_to_fp8_kernel(const IT* __restri
 // (no atomics, no fences: the kernel boundary orders it before the second pass).
 __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 
+// With fin.amax set, the workgroup that finishes last (a ticket counter in the workspace tells) also
+// reduces the partial maxima and applies the scale rule, which saves the finalize launch.
+struct Finish {
+    float* amax;    // nullptr: leave the reduction to a later kernel
+    float* scale;
+    float* scale_inv;
+    float fp_max;
+    int margin;
+    int flags;
+};
+constexpr int kWsTicket = 2;
+
 template <typename IT>
 __global__ __launch_bounds__(kCastThreads) void amax_partial_kernel(const IT* __restrict__ x, size_t n, uint32_t* ws,
-                                                                     const float* scale, int vec_ok, Gate gate) {
+                                                                     const float* scale, int vec_ok, Gate gate,
+                                                                     Finish fin) {
     if (gate_closed(gate)) return;
     constexpr int EPT = 16 / sizeof(IT);
     constexpr int UNROLL = 8;
@@ -238,6 +258,31 @@ __global__ __launch_bounds__(kCastThreads) void amax_partial_kernel(const IT* __
             ws[0] = scale != nullptr ? __float_as_uint(*scale) : __float_as_uint(1.0f);
             ws[1] = gridDim.x;
         }
+    }
+    if (fin.amax == nullptr) return;
+    __shared__ uint32_t s_last;
+    if (tid == 0) {
+        __threadfence();    // the partial maximum above is visible before the ticket is taken
+        const uint32_t ticket = atomicAdd(ws + kWsTicket, 1u);
+        s_last = ticket == gridDim.x - 1;
+        if (s_last) ws[kWsTicket] = 0;    // ready for the next call
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();    // see every other workgroup's partial maximum
+    uint32_t mm = 0;
+    for (int i = tid; i < static_cast<int>(gridDim.x); i += kCastThreads) {
+        const uint32_t v = __hip_atomic_load(ws + kWsPartials + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        mm = v > mm ? v : mm;
+    }
+    mm = block_max_u32(mm, red);
+    if (tid == 0) {
+        float a = __uint_as_float(mm);
+        if ((fin.flags & MSAMP_FLAG_NAN_TO_INF) && !(a < __uint_as_float(0x7f800000u))) a = __uint_as_float(0x7f800000u);
+        const float sc = scale_rule(a, *fin.scale, fin.fp_max, fin.margin);
+        *fin.amax = a;
+        *fin.scale = sc;
+        *fin.scale_inv = 1.0f / sc;
     }
 }
 
@@ -739,8 +784,37 @@ __global__ void scaling_factor_kernel(const float* amax, const float* scale_in, 
 
 __device__ __forceinline__ float nanmax(float a, float b) { return (a != a) ? a : ((b != b) ? b : fmaxf(a, b)); }
 
-__global__ void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad, int32_t* counters, int n, int window,
-                                    float fp_max, int margin) {
+// One wavefront per meta (window <= 64): lane j holds amaxs[i][j], so the row is read and written
+// with one load and one store per lane instead of a chain of dependent accesses.
+__global__ __launch_bounds__(256) void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad,
+                                                            int32_t* counters, int n, int window, float fp_max,
+                                                            int margin) {
+    const int lane = threadIdx.x & 63;
+    const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (i >= n) return;
+    float* row = amaxs + static_cast<size_t>(i) * window;
+    float v = lane < window ? row[lane] : 0.0f;
+    const float a0_raw = __shfl(v, 0);
+    const bool is_bad = !(fabsf(a0_raw) < __uint_as_float(0x7f800000u));
+    const float a0 = is_bad ? 0.0f : a0_raw;
+    if (lane == 0) v = a0;
+    // NaN-propagating maximum over the window, as torch.max does
+    float mx = v;
+#pragma unroll
+    for (int o = 32; o; o >>= 1) mx = nanmax(mx, __shfl_xor(mx, o));
+    // shift: row[j] <- row[j-1] for j >= 1 (row[1] gets the cleaned current value), row[0] <- 0
+    const float left = __shfl_up(v, 1);
+    if (lane < window) row[lane] = lane == 0 ? 0.0f : left;
+    if (lane == 0) {
+        scales[i] = scale_rule(mx, scales[i], fp_max, margin);
+        if (bad != nullptr) bad[i] = is_bad ? 1 : 0;
+        if (counters != nullptr) counters[i] = is_bad ? 0 : counters[i] + 1;
+    }
+}
+
+// any window: one lane per meta
+__global__ void scale_update_wide_kernel(float* scales, float* amaxs, uint8_t* bad, int32_t* counters, int n, int window,
+                                         float fp_max, int margin) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     float* row = amaxs + static_cast<size_t>(i) * window;
@@ -772,7 +846,7 @@ static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, f
     constexpr int EPT = In16<IT>::EPT;
     const int vec_ok = aligned(x, 16) && aligned(out, EPT);
     int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * kCastUnroll);
-    const InTimeArgs none = {nullptr, nullptr, nullptr, 0.0f, 0, 0, nullptr, nullptr};
+    const InTimeArgs none = {nullptr, nullptr, nullptr, 0.0f, 0, 0, nullptr, nullptr, nullptr, 0, nullptr};
 #define LAUNCH(FMT, AM, INT) \
     hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, AM, INT>), dim3(grid), dim3(kCastThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, INT == kInTime ? 1 : 0, INT != kGivenScale ? *it : none)
     if (it != nullptr && it->known_amax != nullptr) {
@@ -803,13 +877,13 @@ static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, f
 }
 
 template <typename IT>
-static int launch_amax(const IT* x, size_t n, uint32_t* ws, const float* scale, Gate gate, hipStream_t st) {
+static int launch_amax(const IT* x, size_t n, uint32_t* ws, const float* scale, Gate gate, Finish fin, hipStream_t st) {
     constexpr int EPT = 16 / sizeof(IT);
     const int vec_ok = aligned(x, 16);
     int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * 8);
     const int cap = cu_count() * 4 < kMaxPartials ? cu_count() * 4 : kMaxPartials;
     grid = grid < cap ? grid : cap;
-    hipLaunchKernelGGL((amax_partial_kernel<IT>), dim3(grid), dim3(kCastThreads), 0, st, x, n, ws, scale, vec_ok, gate);
+    hipLaunchKernelGGL((amax_partial_kernel<IT>), dim3(grid), dim3(kCastThreads), 0, st, x, n, ws, scale, vec_ok, gate, fin);
     MSAMP_CHECK_LAUNCH("amax_partial_kernel");
     return MSAMP_OK;
 }
@@ -817,16 +891,18 @@ static int launch_amax(const IT* x, size_t n, uint32_t* ws, const float* scale, 
 // first pass: partial maxima of |x| into the workspace (plus the scale in force, for the rule's fallback)
 constexpr Gate kNoGate = {nullptr, 0};
 
+constexpr Finish kNoFinish = {nullptr, nullptr, nullptr, 0.0f, 0, 0};
+
 static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const float* scale, hipStream_t st,
-                         Gate gate = kNoGate) {
+                         Gate gate = kNoGate, Finish fin = kNoFinish) {
     uint32_t* w = static_cast<uint32_t*>(ws);
     switch (dtype) {
         case MSAMP_DT_F32:
-            return launch_amax(static_cast<const float*>(x), n, w, scale, gate, st);
+            return launch_amax(static_cast<const float*>(x), n, w, scale, gate, fin, st);
         case MSAMP_DT_F16:
-            return launch_amax(static_cast<const f16_t*>(x), n, w, scale, gate, st);
+            return launch_amax(static_cast<const f16_t*>(x), n, w, scale, gate, fin, st);
         case MSAMP_DT_BF16:
-            return launch_amax(static_cast<const bf16_t*>(x), n, w, scale, gate, st);
+            return launch_amax(static_cast<const bf16_t*>(x), n, w, scale, gate, fin, st);
     }
     set_error("unsupported input dtype %d", dtype);
     return MSAMP_ERR_DTYPE;
@@ -1070,18 +1146,19 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
     if (rc <= 0) return rc;
     rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
     if (rc != MSAMP_OK) return rc;
-    const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags, nullptr, nullptr};
+    const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags, nullptr, nullptr, nullptr, 0, nullptr};
     return dispatch_cast(x, in_dtype, n, scale, nullptr, scale_inv, out, fp8_type, &it, st);
 }
 
 int msamp_cast_scaled_to_fp8(const void* x, int in_dtype, size_t n, const float* amax, const float* old_scale_inv,
-                             float* scale, float* scale_inv, uint8_t* out, int fp8_type, int margin,
-                             msamp_stream_t stream) {
+                             float* scale, float* scale_inv, float* amax_out, int window, int32_t* counter_out,
+                             uint8_t* out, int fp8_type, int margin, msamp_stream_t stream) {
     MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_cast_scaled_to_fp8: fp8_type %d", fp8_type);
     MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "msamp_cast_scaled_to_fp8: in_dtype %d", in_dtype);
     MSAMP_REQUIRE(amax && old_scale_inv && scale && scale_inv && ((x && out) || n == 0), MSAMP_ERR_NULL,
                   "msamp_cast_scaled_to_fp8: null pointer");
-    const InTimeArgs it = {nullptr, scale, nullptr, fp8_max(fp8_type), margin, 0, amax, old_scale_inv};
+    MSAMP_REQUIRE(amax_out == nullptr || window >= 1, MSAMP_ERR_SHAPE, "msamp_cast_scaled_to_fp8: window %d", window);
+    const InTimeArgs it = {nullptr, scale, nullptr, fp8_max(fp8_type), margin, 0, amax, old_scale_inv, amax_out, window, counter_out};
     return dispatch_cast(x, in_dtype, n, nullptr, nullptr, scale_inv, out, fp8_type, &it, static_cast<hipStream_t>(stream));
 }
 
@@ -1149,9 +1226,8 @@ int msamp_cast_to_fp8_gated(const void* x, int in_dtype, size_t n, float* scale,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const Gate gate = {warmup_counter, window};
     // while warming up: amax[0] and the scale from this tensor; afterwards both kernels return at once
-    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st, gate);
-    if (rc != MSAMP_OK) return rc;
-    rc = finalize_amax(workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st, gate);
+    const Finish fin = {amax, scale, scale_inv, fp8_max(fp8_type), margin, flags};
+    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st, gate, fin);
     if (rc != MSAMP_OK) return rc;
     // the delayed cast serves both cases: folding max|x| into an amax[0] that already holds it changes nothing
     return dispatch_cast(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, nullptr, st);
@@ -1169,9 +1245,8 @@ int msamp_cast_transpose_gated(const void* x, int in_dtype, int rows, int cols, 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const size_t n = static_cast<size_t>(rows) * cols;
     const Gate gate = {warmup_counter, window};
-    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st, gate);
-    if (rc != MSAMP_OK) return rc;
-    rc = finalize_amax(workspace, amax, scale, scale_inv, fp8_max(fp8_type), margin, flags, 1, st, gate);
+    const Finish fin = {amax, scale, scale_inv, fp8_max(fp8_type), margin, flags};
+    int rc = dispatch_amax(x, in_dtype, n, workspace, scale, st, gate, fin);
     if (rc != MSAMP_OK || n == 0) return rc;
     return dispatch_ct(x, in_dtype, rows, cols, scale, amax, scale_inv, out, out_t, fp8_type, st);
 }
@@ -1211,8 +1286,13 @@ int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int32_t* count
     MSAMP_REQUIRE(n >= 0 && window >= 1, MSAMP_ERR_SHAPE, "msamp_scale_update: n=%d window=%d", n, window);
     if (n == 0) return MSAMP_OK;
     MSAMP_REQUIRE(scales && amaxs, MSAMP_ERR_NULL, "msamp_scale_update: null pointer");
-    hipLaunchKernelGGL(scale_update_kernel, dim3((n + 63) / 64), dim3(64), 0, static_cast<hipStream_t>(stream), scales,
-                       amaxs, bad, counters, n, window, fp_max, margin);
+    if (window <= 64) {
+        hipLaunchKernelGGL(scale_update_kernel, dim3((n + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), scales,
+                           amaxs, bad, counters, n, window, fp_max, margin);
+    } else {
+        hipLaunchKernelGGL(scale_update_wide_kernel, dim3((n + 63) / 64), dim3(64), 0, static_cast<hipStream_t>(stream),
+                           scales, amaxs, bad, counters, n, window, fp_max, margin);
+    }
     MSAMP_CHECK_LAUNCH("scale_update_kernel");
     return MSAMP_OK;
 }

@@ -34,7 +34,7 @@ _SIGNATURES = {
     'msamp_compute_scaling_factor': ([_vp, _vp, _i, _vp, _i, _f, _i, _vp], _i),
     'msamp_cast_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp], _i),
     'msamp_cast_to_fp8_intime': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
-    'msamp_cast_scaled_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp], _i),
+    'msamp_cast_scaled_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp], _i),
     'msamp_cast_from_fp8': ([_vp, _i, _sz, _vp, _vp, _i, _vp], _i),
     'msamp_cast_transpose': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp], _i),
     'msamp_cast_transpose_intime': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
@@ -198,15 +198,19 @@ def cast_to_fp8_gated(x, scale, amax_cell, scale_inv, fp8_dt, counter, window, m
     return out
 
 
-def cast_scaled_to_fp8(x, amax_cell, old_scale_inv, scale, scale_inv, fp8_dt, margin=0):
-    """Requantize a scaled 16/32-bit payload whose amax is known; writes scale and scale_inv."""
+def cast_scaled_to_fp8(x, amax, old_scale_inv, scale, scale_inv, fp8_dt, margin=0, amax_out=None, counter_out=None):
+    """Requantize a scaled 16/32-bit payload whose amax is known; writes scale and scale_inv, and, if
+    given, copies the amax window to `amax_out` and zeroes `counter_out` (the rest of a fresh meta)."""
     lib = load()
     _gpu(x, 'input')
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    window = amax_out.numel() if amax_out is not None else 0
+    if window > amax.numel():
+        raise ValueError('amax_out is longer than the source amax window')
     _check(
         lib.msamp_cast_scaled_to_fp8(
-            _ptr(x), _dt(x), x.numel(), _ptr(amax_cell), _ptr(old_scale_inv), _ptr(scale), _ptr(scale_inv), _ptr(out),
-            fp8_dt, margin, _stream()
+            _ptr(x), _dt(x), x.numel(), _ptr(amax), _ptr(old_scale_inv), _ptr(scale), _ptr(scale_inv), _ptr(amax_out),
+            window, _ptr(counter_out), _ptr(out), fp8_dt, margin, _stream()
         ), 'msamp_cast_scaled_to_fp8'
     )
     return out

@@ -29,6 +29,21 @@ class ScalingMeta:
         self.group = group
         self.locked = False
 
+    @classmethod
+    def _uninitialized(cls, qtype, window_size, device, group=None):
+        """A meta whose four tensors are views of one uninitialised buffer, for callers whose kernel
+        writes every field (scale, scale_inv, counter, amax window) itself."""
+        self = cls.__new__(cls)
+        slab = torch.empty(3 + window_size, dtype=torch.float32, device=device)
+        self.qtype = qtype
+        self.scale, self.scale_inv = slab[0], slab[1]
+        self.amax_counter = slab[2:3].view(torch.int32).reshape(())
+        self.amax = slab[3:]
+        self.window_size = window_size
+        self.group = group
+        self.locked = False
+        return self
+
     @staticmethod
     def compute_scaling_factor(amax, scale, fp_max: float, margin: int):
         """Largest power of two sf with sf * amax <= fp_max (shifted down by `margin` binades).

@@ -191,13 +191,15 @@ class ScalingTensor:
         if Dtypes.is_fp8_qtype(self.meta.qtype):
             return self.float().cast(qtype)
         old = self.meta
-        meta = ScalingMeta(qtype, amax=old.amax.clone(), window_size=old.window_size, device=old.amax.device)
         if Dtypes.is_fp8_qtype(qtype):
-            # the whole recipe in one kernel
+            # the whole recipe, new meta included, in one kernel
+            meta = ScalingMeta._uninitialized(qtype, old.window_size, old.amax.device)
             value = _backend.cast_scaled_to_fp8(
-                self.value.contiguous(), meta.amax, old.scale_inv, meta.scale, meta.scale_inv, int(qtype)
+                self.value.contiguous(), old.amax, old.scale_inv, meta.scale, meta.scale_inv, int(qtype),
+                amax_out=meta.amax, counter_out=meta.amax_counter
             )
             return ScalingTensor(value, meta)
+        meta = ScalingMeta(qtype, amax=old.amax.clone(), window_size=old.window_size, device=old.amax.device)
         meta.reset_scaling_factor()
         scale_inv = torch.reciprocal(meta.scale)
         meta.scale.mul_(old.scale_inv)
