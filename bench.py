@@ -5,7 +5,7 @@ payload), dy[8192,4096] (bf16) in steady-state delayed scaling (amax history 16)
 weight cast, y = x W^T, fused cast+transpose of dy to E5M2, the two FP8 transposes, dx = dy W,
 dW = dy^T x, the in-time E4M3 cast of dW and the amax-window update.  `value` is the three GEMMs'
 2*M*N*K flops divided by the whole step time (inputs resident in HBM).  Beside it: the GEMM kernel's
-own roofline (HIP events around every GEMM launch inside the timed region), the cast+amax and fused
+own roofline (HIP events around the GEMM launches of every fourth step inside the timed region), the cast+amax and fused
 FP8-AdamW kernels against the HBM roofline, and the CPU oracle timed on the host cores.
 
 Prints one JSON line.  Synthetic data, random weights.
@@ -23,6 +23,7 @@ for _p in (ROOT, os.path.join(ROOT, 'ms-amp_amd')):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0
+GEMM_EVENT_STRIDE = 4
 FP8_PEAK_TFLOPS = 5000.0
 
 
@@ -84,9 +85,10 @@ def bench_fp8linear(steps, warmup):
         step()
     assert not model.scaling_metas['input'].is_in_time_scaling()
     torch.cuda.synchronize()
-    _Timed.enabled = True
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for i in range(steps):
+        # an event pair costs the stream a few microseconds: bracket the GEMMs of every fourth step only
+        _Timed.enabled = i % GEMM_EVENT_STRIDE == 0
         step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
@@ -249,6 +251,28 @@ def cpu_baseline():
     }
 
 
+def pmc_calibration_copy():
+    """One plain copy of known size -- scale_cast fp32 -> fp32 at scale 1 over 64 Mi elements: 256 MiB read,
+    256 MiB written -- so that a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this program holds a
+    dispatch of known traffic to scale the counters by.  Untimed."""
+    import torch
+    from msamp import _backend
+    src = torch.ones(64 * 1024 * 1024, device='cuda')
+    _backend.scale_cast(src, torch.ones((), device='cuda'), torch.float32)
+    torch.cuda.synchronize()
+
+
+def measured_gemm_traffic():
+    """HBM bytes per GEMM launch as last measured with rocprofv3 --pmc (profiles/fp8_gemm_hbm_traffic.json),
+    or None when no measurement is on file."""
+    path = os.path.join(ROOT, 'profiles', 'fp8_gemm_hbm_traffic.json')
+    try:
+        with open(path) as f:
+            return json.load(f)['traffic_bytes_per_launch']
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -266,6 +290,7 @@ def main():
         sys.exit(2)
     torch.cuda.set_device(0)
 
+    pmc_calibration_copy()
     lin = bench_fp8linear(args.steps, args.warmup)
     result = {
         'metric': 'FP8 GEMM TFLOPS, cast+amax GB/s, FP8-Adam Gparams/s on 1 MI355X',
@@ -284,7 +309,7 @@ def main():
                                'delayed scaling (history 16), outputs bf16, dW -> E4M3'},
         'roofline': {
             'kernel': 'fp8_gemm_kernel', 'bound': 'mfma', 'achieved': lin['gemm_tflops'], 'peak': FP8_PEAK_TFLOPS,
-            'unit': 'TFLOP/s', 'frac': lin['gemm_tflops'] / FP8_PEAK_TFLOPS, 'traffic': None,
+            'unit': 'TFLOP/s', 'frac': lin['gemm_tflops'] / FP8_PEAK_TFLOPS, 'traffic': measured_gemm_traffic(),
             'avg_launch_ms': lin['gemm_ms'], 'launches': lin['gemm_launches'],
         },
     }
