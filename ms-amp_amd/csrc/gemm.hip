@@ -437,20 +437,31 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
             }
         });
         __builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): the patch is written (same wave reads it back)
-        for (int pass = 0; pass < 32 / kRowsPerPass; ++pass) {
-            const int pr = pass * kRowsPerPass + lane / kChunksPerRow;
-            const int pc = lane % kChunksPerRow;
-            const int grow = row0 + wr * 128 + i * 32 + pr;
-            const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
-            const uint4 val = *reinterpret_cast<const uint4*>(patch + pr * kPitch + pc * 16);
-            if (grow >= NR || gcol >= NC) continue;
-            OT* out = D + static_cast<size_t>(grow) * NC + gcol;
-            if (plain && gcol + kElemsPerChunk <= NC) {
-                *reinterpret_cast<uint4*>(out) = val;
-            } else {
-                store_chunk_slow<OT>(out, val, gcol, NC, accumulate, bias, bias_dt);
+        constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
+        static_for<kPasses / 8>([&](auto gc) {
+            constexpr int p0 = decltype(gc)::value * 8;
+            uint4 val[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {    // eight reads in flight together
+                const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
+                val[u] = *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
             }
-        }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
+                const int pc = lane % kChunksPerRow;
+                const int grow = row0 + wr * 128 + i * 32 + pr;
+                const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
+                if (grow < NR && gcol < NC) {
+                    OT* out = D + static_cast<size_t>(grow) * NC + gcol;
+                    if (plain && gcol + kElemsPerChunk <= NC) {
+                        *reinterpret_cast<uint4*>(out) = val[u];
+                    } else {
+                        store_chunk_slow<OT>(out, val[u], gcol, NC, accumulate, bias, bias_dt);
+                    }
+                }
+            }
+        });
         __builtin_amdgcn_s_waitcnt(0xC07F);    // patch reads done before the next block overwrites it
     });
 }
