@@ -123,6 +123,39 @@ def test_fused_step_variants(be, kw):
     _check(dev[0], t, fp8.E4M3, fp8.E5M2, 3, **kw)
 
 
+def test_fused_step_maximum_comes_from_the_update_term(be):
+    """The amax pass bounds 16 elements at a time by max|p| + step * max|m'| / (sqrt(min v') / sbc2 + eps); here the
+    largest |p'| belongs to elements with a small weight and a large update (zero second moment, largest first
+    moment), spread over lanes that otherwise hold small values."""
+    n = 16384 * 6 + 48
+    t = _inputs(n, 55, fp8.E4M3, fp8.E5M2)
+    for idx in (5, 16384 * 2 + 17, n - 3):
+        t['v'][idx] = 0.0
+        t['m'][idx] = 0x7E if idx != 5 else 0xFE    # +-448 / scale
+        t['g'][idx] = 0
+        t['w'][idx] = 0x01                           # smallest positive weight code
+    for kw in (dict(lr=0.5), dict(lr=0.5, eps=0.0), dict()):
+        dev = _fused(be, [t], 5, 6, 2, **kw)
+        _check(dev[0], t, fp8.E4M3, fp8.E5M2, 2, **kw)
+
+
+def test_fused_step_nan_state_reaches_the_weight_amax(be):
+    """A NaN second moment makes that element's new weight NaN: the weight amax must say so (NaN), the scale stays,
+    and every other weight is what the oracle gives."""
+    n = 16384 * 3
+    t = _inputs(n, 56, fp8.E4M3, fp8.E5M2)
+    bad = 16384 + 4321
+    t['v'].view(torch.int16)[bad] = 0x7E00
+    dev = _fused(be, [t], 5, 6, 2)[0]
+    (w2, wm2, _, _, _, _), _ = oadam.step_tensor(t['w'], t['wm'], fp8.E4M3, t['g'], t['gm']['scale_inv'], fp8.E5M2, t['m'], t['mm'],
+                                                 t['v'], t['vm'], step=2, **HYPER)
+    assert torch.isnan(dev['wm'][2][0]).item() and torch.isnan(wm2['amax'][0]).item()
+    assert same_float(dev['wm'][0], wm2['scale']) and same_float(dev['wm'][0], t['wm']['scale'])
+    d = _code_distance(dev['w'], w2)
+    d[bad] = 0    # the sign of a NaN is not defined
+    assert d.max().item() <= 1 and dev['w'][bad].item() & 0x7F == 0x7F and w2[bad].item() & 0x7F == 0x7F
+
+
 def test_fused_step_grouping_does_not_change_results(be):
     sizes = [16384 * 3, 16384 * 5 + 9, 100, 16384 * 2]
     tensors = [_inputs(n, 300 + i, fp8.E4M3, fp8.E5M2) for i, n in enumerate(sizes)]
