@@ -962,6 +962,9 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
     if (max_blocks > static_cast<size_t>(kMaxSlots)) max_blocks = kMaxSlots;
     if (nvec == 0 || nvec > max_blocks * kResThreads * kResVecs) return 1;
     if (!owns_resident_kernel(st)) return 1;
+    // a captured launch would replay this call's token, and the slots of the previous replay still carry it
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return 1;
     const void* fn = fp8_type == MSAMP_DT_E4M3
                          ? reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E4M3>)
                          : reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E5M2>);

@@ -195,6 +195,91 @@ def test_historical_window_quantization():
     assert not model.scaling_metas['input'].is_in_time_scaling()
 
 
+def _linear_step_record(model, opt, x, dy):
+    metas = model.scaling_metas
+    return dict(
+        dx=x.grad.clone(), dw=model.weight.grad.value.clone(), dw_scale_inv=model.weight.grad.meta.scale_inv.clone(),
+        metas={k: (m.scale.clone(), m.scale_inv.clone(), m.amax.clone(), m.amax_counter.clone()) for k, m in metas.items()}
+    )
+
+
+def test_training_step_replays_from_a_graph():
+    """Nothing in forward + backward + window update waits for the GPU or decides on the host, so one captured graph
+    serves the warm-up (in-time scaling) and the steady state (delayed scaling) alike: 24 steps with changing inputs,
+    every replay against the eager run, bit for bit, with eager work in between."""
+    tokens, d_in, d_out, steps = 256, 128, 192, 24
+    torch.manual_seed(3)
+    w0 = (torch.randn(d_out, d_in) * 0.05).bfloat16()
+    xs = [(torch.randn(tokens, d_in) * (1 + (i % 5))).bfloat16().cuda() for i in range(steps)]
+    dys = [(torch.randn(tokens, d_out) * 1e-3 * (1 + (i % 3))).bfloat16().cuda() for i in range(steps)]
+
+    def build():
+        model_state.clear()
+        lin = torch.nn.Linear(d_in, d_out, bias=False).cuda().bfloat16()
+        with torch.no_grad():
+            lin.weight.copy_(w0)
+        model = LinearReplacer.replace(lin, Dtypes.kbfloat16)
+        return model, LBAdamW(model.parameters())
+
+    # eager
+    model, opt = build()
+    want = []
+    for i in range(steps):
+        x = xs[i].clone().requires_grad_(True)
+        y = model(x)
+        y.backward(dys[i])
+        opt._update_scaling_factors()
+        rec = _linear_step_record(model, opt, x, dys[i])
+        rec['y'] = y.detach().clone()
+        want.append(rec)
+        model.weight.grad = None
+
+    # graph: three eager steps on a side stream (allocator warm-up), then capture the fourth and replay the rest
+    model, opt = build()
+    x = xs[0].clone().requires_grad_(True)
+    dy = dys[0].clone()
+    n_eager = 3
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(n_eager):
+            with torch.no_grad():
+                x.copy_(xs[i])
+                dy.copy_(dys[i])
+            y = model(x)
+            y.backward(dy)
+            opt._update_scaling_factors()
+            x.grad = None
+            model.weight.grad = None
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        x.copy_(xs[n_eager])
+        dy.copy_(dys[n_eager])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = model(x)
+        y.backward(dy)
+        model_state.ready_to_scale_tensor = True
+        opt._update_scaling_factors()
+    for i in range(n_eager, steps):
+        with torch.no_grad():
+            x.copy_(xs[i])
+            dy.copy_(dys[i])
+        graph.replay()
+        got = _linear_step_record(model, opt, x, dy)
+        torch.cuda.synchronize()
+        w = want[i]
+        assert torch.equal(y, w['y']) and torch.equal(got['dx'], w['dx']), i
+        assert torch.equal(got['dw'], w['dw']) and same_float(got['dw_scale_inv'], w['dw_scale_inv']), i
+        for k in w['metas']:
+            for a, b in zip(got['metas'][k], w['metas'][k]):
+                assert same_float(a.float(), b.float()), (i, k)
+        # eager work between replays
+        assert torch.isfinite((xs[i].float() @ w0.float().cuda().t()).sum()).item()
+    assert model.scaling_metas['input'].amax_counter.item() == steps
+
+
 def test_optimizer_state_dict_round_trip():
     torch.manual_seed(7)
     x = torch.randn(4, 4, device='cuda')
