@@ -211,7 +211,8 @@ def cpu_baseline():
     from oracle import adamw as oadam, cast as ocast, fp8
     from tests.gpu_util import c1_input
     from tests.test_gpu_adam import _inputs
-    cores = os.cpu_count()
+    # the box sets OMP_NUM_THREADS to its CPU share; never spread over more threads than that
+    cores = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', '16') or 16))
     torch.set_num_threads(cores)
 
     def med(fn, runs=5, warm=2):
