@@ -346,7 +346,7 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
     constexpr int EPT = 16 / sizeof(IT);
     using Raw = typename std::conditional<sizeof(IT) == 4, uint32_t, uint16_t>::type;
     __shared__ uint32_t red[kResThreads / kWave];
-    __shared__ uint32_t s_scale;
+    __shared__ uint32_t s_scale, s_amax;
     const int tid = threadIdx.x;
     // the host keeps the vector count within 32 bits (at most one register file of vectors)
     const uint32_t nvec = static_cast<uint32_t>(n / EPT);
@@ -410,6 +410,7 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
             else if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
             const float s = scale_rule(am, old_scale, fp_max, margin);
             s_scale = __float_as_uint(s);
+            s_amax = __float_as_uint(am);
             if (blockIdx.x == 0) {
                 *amax = am;
                 *scale = s;
@@ -419,20 +420,41 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
     }
     __syncthreads();
     const float s = __uint_as_float(s_scale);
+    // With a positive finite amax and the scale the rule derived from it, every |x| * s stays within the
+    // format and nothing is NaN: the clamp and the NaN patch can go.
+    const bool in_range = __uint_as_float(s_amax) * s <= fp_max && __uint_as_float(s_amax) > 0.0f;
 
+    if (in_range) {
 #pragma unroll
-    for (int r = 0; r < kResVecs; ++r) {
-        // keep only the raw words live across the barrier, not values derived from them before it
-        asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
-        const uint32_t idx = v0 + r * kResThreads;
-        if (r < rounds && idx < nvec) {
-            float f[EPT];
-            In16<IT>::decode(v[r], f);
-            uint32_t w[EPT / 4];
+        for (int r = 0; r < kResVecs; ++r) {
+            // keep only the raw words live across the barrier, not values derived from them before it
+            asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
+            const uint32_t idx = v0 + r * kResThreads;
+            if (r < rounds && idx < nvec) {
+                float f[EPT];
+                In16<IT>::decode(v[r], f);
+                uint32_t w[EPT / 4];
 #pragma unroll
-            for (int j = 0; j < EPT / 4; ++j) w[j] = quant4<FMT>(f[4 * j] * s, f[4 * j + 1] * s, f[4 * j + 2] * s, f[4 * j + 3] * s);
-            if constexpr (EPT == 4) reinterpret_cast<uint32_t*>(out)[idx] = w[0];
-            else reinterpret_cast<uint2*>(out)[idx] = make_uint2(w[0], w[1]);
+                for (int j = 0; j < EPT / 4; ++j)
+                    w[j] = quant4_in_range<FMT>(f[4 * j] * s, f[4 * j + 1] * s, f[4 * j + 2] * s, f[4 * j + 3] * s);
+                if constexpr (EPT == 4) reinterpret_cast<uint32_t*>(out)[idx] = w[0];
+                else reinterpret_cast<uint2*>(out)[idx] = make_uint2(w[0], w[1]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < kResVecs; ++r) {
+            asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
+            const uint32_t idx = v0 + r * kResThreads;
+            if (r < rounds && idx < nvec) {
+                float f[EPT];
+                In16<IT>::decode(v[r], f);
+                uint32_t w[EPT / 4];
+#pragma unroll
+                for (int j = 0; j < EPT / 4; ++j) w[j] = quant4<FMT>(f[4 * j] * s, f[4 * j + 1] * s, f[4 * j + 2] * s, f[4 * j + 3] * s);
+                if constexpr (EPT == 4) reinterpret_cast<uint32_t*>(out)[idx] = w[0];
+                else reinterpret_cast<uint2*>(out)[idx] = make_uint2(w[0], w[1]);
+            }
         }
     }
     if (has_tail) {

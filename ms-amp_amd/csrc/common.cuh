@@ -118,6 +118,15 @@ __device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
     return w;
 }
 
+// the same for values known to be finite and within the format's range: no clamp, no NaN patch
+template <int FMT>
+__device__ __forceinline__ uint32_t quant4_in_range(float a, float b, float c, float d) {
+    uint32_t w = 0;
+    w = cvt_pk<FMT>(a, b, w, false);
+    w = cvt_pk<FMT>(c, d, w, true);
+    return w;
+}
+
 template <int FMT>
 __device__ __forceinline__ uint32_t quant1(float a) {
     uint32_t w = cvt_pk<FMT>(sat<FMT>(a), 0.0f, 0u, false) & 0xffu;
