@@ -2,8 +2,9 @@
 
 A step is one forward + backward of a single FP8Linear at x[8192,4096] (bf16), W[4096,4096] (bf16
 payload), dy[8192,4096] (bf16) in steady-state delayed scaling (amax history 16): input cast to E4M3,
-weight cast, y = x W^T, fused cast+transpose of dy to E5M2, the two FP8 transposes, dx = dy W,
-dW = dy^T x, the in-time E4M3 cast of dW and the amax-window update.  `value` is the three GEMMs'
+weight cast, y = x W^T, cast of dy to E5M2, dx = dy W and dW = dy^T x (the kernel reads W, x and dy
+K-major in place, so no transposed copies are made), the in-time E4M3 cast of dW and the amax-window
+update.  `value` is the three GEMMs'
 2*M*N*K flops divided by the whole step time (inputs resident in HBM).  Beside it: the GEMM kernel's
 own roofline (HIP events around the GEMM launches of every fourth step inside the timed region), the cast+amax and fused
 FP8-AdamW kernels against the HBM roofline, and the CPU oracle timed on the host cores.
@@ -296,7 +297,7 @@ def main():
     result = {
         'metric': 'FP8 GEMM TFLOPS, cast+amax GB/s, FP8-Adam Gparams/s on 1 MI355X',
         'value': lin['step_tflops'],
-        'unit': 'TFLOP/s (3 GEMMs of one FP8Linear fwd+bwd / whole step incl. casts and transposes)',
+        'unit': 'TFLOP/s (3 GEMMs of one FP8Linear fwd+bwd / whole step incl. casts and window update)',
         'n_gpus': 1,
         'steps': args.steps,
         'warmup': max(args.warmup, 17),

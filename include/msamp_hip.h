@@ -147,6 +147,16 @@ int msamp_fp8_gemm(const uint8_t* a, int a_type, const float* a_scale_inv, const
                    const float* b_scale_inv, void* d, int d_dtype, int m, int n, int k, int accumulate,
                    const void* bias, int bias_dtype, msamp_stream_t stream);
 
+/* The same product with operands handed over K-major: a_kmajor != 0 means `a` points at A^T, i.e. [K][M]
+ * with M contiguous, likewise b_kmajor for [K][N].  The backward GEMMs of a linear layer
+ * (nn/functional.py:84-111 of the reference) then read W, x and dy as they are, and the explicit FP8
+ * transposes (transformer_engine_wrapper.py:165-176) are not needed.  Results are bit-identical to
+ * msamp_fp8_gemm on transposed copies.  Supported: a K-major alone, or both; k % 128 == 0 and the row
+ * count of every K-major operand (m, and n if b_kmajor) a multiple of 256; otherwise MSAMP_ERR_SHAPE. */
+int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
+                          int b_type, const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int m, int n, int k,
+                          int accumulate, const void* bias, int bias_dtype, msamp_stream_t stream);
+
 /* msamp_adamw.adamw_fp8_stage1_compute (adamw.cu:99-127): fp32 param/grad, quantized moments;
  * updates param in place and atomically maxes |m'|, |v'| into the two amax cells.
  * exp_avg_dtype: E4M3/E5M2/F16/F32, exp_avg_sq_dtype: F16/F32/E4M3/E5M2. */

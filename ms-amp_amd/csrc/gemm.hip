@@ -185,7 +185,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
             for (int r = 0; r < 16; ++r) {
                 const int row = row0 + wr * WR + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
                 if (row < NR) {
-                    store_out<OT>(D + static_cast<size_t>(row) * NC + col, acc[i][j][r] * alpha + bv, accumulate != 0);
+                    store_out<OT>(D + static_cast<size_t>(row) * NC + col, fmaf(acc[i][j][r], alpha, bv), accumulate != 0);
                 }
             }
         }
@@ -215,26 +215,17 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
-// one 16-byte chunk of an output row, element by element: ragged right edge, bias, accumulate
+// four consecutive elements of an output row straight from the accumulators, one by one: ragged edges,
+// bias and accumulation, all in float32 with a single rounding to the output type
 template <typename OT>
-__device__ __noinline__ void store_chunk_slow(OT* out, uint4 val, int gcol, int NC, int accumulate, const void* bias,
-                                              int bias_dt) {
-    constexpr int kEsz = static_cast<int>(sizeof(OT));
-    constexpr int kElems = 16 / kEsz;
-    for (int e = 0; e < kElems; ++e) {
-        if (gcol + e >= NC) break;
-        const int wi = e * kEsz / 4;
-        const uint32_t word = wi == 0 ? val.x : (wi == 1 ? val.y : (wi == 2 ? val.z : val.w));
-        float v;
-        if constexpr (kEsz == 4) {
-            v = __uint_as_float(word);
-        } else if constexpr (__is_same(OT, bf16_t)) {
-            v = bf16_bits_to_float((word >> ((e & 1) * 16)) & 0xffffu);
-        } else {
-            v = f16_bits_to_float((word >> ((e & 1) * 16)) & 0xffffu);
-        }
-        if (bias != nullptr) v += load_bias(bias, bias_dt, gcol + e);
-        store_out<OT>(out + e, v, accumulate != 0);
+__device__ __noinline__ void store_quad_slow(OT* D, int row, int col, int NR, int NC, float alpha, float v0, float v1,
+                                             float v2, float v3, int accumulate, const void* bias, int bias_dt) {
+    if (row >= NR) return;
+    const float v[4] = {v0, v1, v2, v3};
+    for (int e = 0; e < 4; ++e) {
+        if (col + e >= NC) break;
+        const float bv = bias != nullptr ? load_bias(bias, bias_dt, col + e) : 0.0f;
+        store_out<OT>(D + static_cast<size_t>(row) * NC + col + e, fmaf(v[e], alpha, bv), accumulate != 0);
     }
 }
 
@@ -261,7 +252,17 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int XF, int YF, typename OT>
+//  * XT / YT: that operand is handed over K-major, T[K][rows] with the rows contiguous (the transpose of
+//    what the product needs), so that callers need not materialize transposed copies.  Its slice sits in
+//    LDS as 128 k-rows of 256 bytes (same 32 KiB), filled by the same eight 1 KiB loads, and its
+//    fragments come from the transposing LDS read: a 16-lane group reads eight k-rows of 16 bytes and
+//    lane i receives byte i of each, i.e. eight consecutive k for its row -- four such reads make the
+//    32-byte operand of the MFMA.  The 16-byte position inside a k-row is XOR-ed with k % 8 (on the global
+//    side again) so that the eight k-rows of one read fall into different banks.  Needs that operand's
+//    row count to be a multiple of 256.
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
                                                                      const uint8_t* __restrict__ Y, OT* __restrict__ D,
                                                                      int NR, int NC, int K,
@@ -283,6 +284,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     const int chunk = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
     const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)smem)));
+    // K-major operand: one wave instruction fills 4 k-rows of 256 bytes; lane l lands in k-row l/16,
+    // position l%16, and fetches the logical chunk position ^ (k-row % 8)
+    const int chunk_t = (lane & 15) ^ ((wave & 1) * 4 + (lane >> 4));
     uint32_t xoff[8], yoff[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -290,12 +294,17 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         int gx = row0 + r, gy = col0 + r;
         gx = gx < NR ? gx : NR - 1;
         gy = gy < NC ? gy : NC - 1;
-        xoff[i] = static_cast<uint32_t>(gx) * static_cast<uint32_t>(K) + chunk * 16;
-        yoff[i] = static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
+        const int krow = (i * 4 + wave) * 4 + (lane >> 4);
+        xoff[i] = XT ? static_cast<uint32_t>(krow) * static_cast<uint32_t>(NR) + row0 + chunk_t * 16
+                     : static_cast<uint32_t>(gx) * static_cast<uint32_t>(K) + chunk * 16;
+        yoff[i] = YT ? static_cast<uint32_t>(krow) * static_cast<uint32_t>(NC) + col0 + chunk_t * 16
+                     : static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
     }
     // one of the 16 loads of a slice (0..7: X rows, 8..15: Y rows), so they can be spread between MFMAs
     auto dma = [&](int kt, int stage, int which) {
-        const uint8_t* src = (which < 8 ? X : Y) + static_cast<size_t>(kt) * kBK;
+        const bool is_x = which < 8;
+        const size_t slice = static_cast<size_t>(kt) * kBK;
+        const uint8_t* src = is_x ? X + (XT ? slice * NR : slice) : Y + (YT ? slice * NC : slice);
         const uint32_t off = which < 8 ? xoff[which] : yoff[which - 8];
         const uint32_t dst = lds_base + stage * kDmaStage + (which < 8 ? 0 : kDmaTile * kBK) + ((which & 7) * 4 + wave) * 1024;
         // Written as assembly so that the compiler does not see an LDS write it cannot tell apart from
@@ -305,16 +314,37 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + off) : "memory", "m0");
     };
 
-    // ---- LDS -> fragments: this lane's row inside a 32-row block and its swizzled 16-byte chunks
+    // ---- LDS -> fragments.  Row-major operand: this lane's row inside a 32-row block and its swizzled
+    // 16-byte chunks.  K-major operand: the address this lane contributes to a transposing read.
     const int fsw = (lane & 7) ^ ((lane >> 3) & 1);
     const int off_a = ((2 * lh) ^ fsw) << 4;    // sub-step 0, low half; high half is ^16, sub-step 1 is ^64
     const int xrow = (wr * 128 + l32) * kBK;
     const int yrow = kDmaTile * kBK + (wc * 128 + l32) * kBK;
-    // fragment half h (0..15): X blocks 0..3 then Y blocks 0..3, low then high 16 bytes
-    auto frag_half = [&](int stage, int ks, int h) -> v4i {
-        const int blk = (h >> 1) & 3;
-        const int base = (h < 8 ? xrow : yrow) + blk * 32 * kBK + ((off_a ^ (ks * 64)) ^ ((h & 1) * 16));
-        return *reinterpret_cast<const v4i*>(smem + stage * kDmaStage + base);
+    const int i16 = lane & 15, tj = i16 >> 1, g1 = (lane >> 4) & 1;
+    const int t_lane = (lh * 32 + tj) * 256 + (i16 & 1) * 8;    // k-row and 8-byte half of this lane's address
+    // A sub-step needs 8 fragments of 8 registers (X blocks 0..3, Y blocks 0..3).  They arrive in pieces:
+    // two 16-byte reads per fragment of a row-major operand, four 8-byte transposing reads otherwise.
+    constexpr int kPX = XT ? 16 : 8, kPY = YT ? 16 : 8, kPieces = kPX + kPY;
+    auto read_piece = [&](int* dst, int stage, int ks, int p) {
+        const bool is_x = p < kPX;
+        const int q = is_x ? p : p - kPX;
+        const uint8_t* base = smem + stage * kDmaStage;
+        if ((is_x && !XT) || (!is_x && !YT)) {
+            const int blk = q >> 1, hf = q & 1;
+            const v4i val = *reinterpret_cast<const v4i*>(base + (is_x ? xrow : yrow) + blk * 32 * kBK +
+                                                          ((off_a ^ (ks * 64)) ^ (hf * 16)));
+            int* d = dst + ((is_x ? 0 : 4) + blk) * 8 + hf * 4;
+            d[0] = val[0], d[1] = val[1], d[2] = val[2], d[3] = val[3];
+        } else {
+            const int blk = q >> 2, qq = q & 3;
+            const int wq = is_x ? wr : wc;
+            const int addr = (is_x ? 0 : kDmaTile * kBK) + t_lane + (ks * 64 + qq * 8) * 256 + wq * 128 +
+                             (((blk * 2 + g1) ^ tj) << 4);
+            const v2i val = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                (__attribute__((address_space(3))) v2i*)(base + addr));
+            int* d = dst + ((is_x ? 0 : 4) + blk) * 8 + qq * 2;
+            d[0] = val[0], d[1] = val[1];
+        }
     };
 
     v16f acc[4][4];
@@ -326,13 +356,13 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     const int nk = K / kBK;
-    v4i fa[16], fb[16];    // fragment halves [X0..X3, Y0..Y3] x {low, high}, two buffers
+    int fa[64], fb[64];    // fragments [X0..X3, Y0..Y3] x 8 registers, two buffers
 
     // One sub-step: 16 MFMAs on `cur`, 16 fragment-half reads into `nxt`, 8 tile loads.
     // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row l%32, four
     // consecutive D columns per register quad -- the layout the epilogue wants.
     // EARLY: the loads go out two per MFMA during the first four MFMAs (they are needed soonest).
-    auto sub_step = [&](const v4i* cur, v4i* nxt, int rd_stage, int rd_ks, bool do_read, int ld_kt, int ld_stage,
+    auto sub_step = [&](const int* cur, int* nxt, int rd_stage, int rd_ks, bool do_read, int ld_kt, int ld_stage,
                         int ld_first, bool do_load, bool early) {
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
@@ -341,10 +371,15 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int n = i * 4 + j;
-                const v8i fx = __builtin_shufflevector(cur[2 * i], cur[2 * i + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-                const v8i fy = __builtin_shufflevector(cur[8 + 2 * j], cur[8 + 2 * j + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+                const int* cx = cur + i * 8;
+                const int* cy = cur + (4 + j) * 8;
+                const v8i fx = {cx[0], cx[1], cx[2], cx[3], cx[4], cx[5], cx[6], cx[7]};
+                const v8i fy = {cy[0], cy[1], cy[2], cy[3], cy[4], cy[5], cy[6], cy[7]};
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fy, fx, acc[i][j], cb, bl, 0, 0, 0, 0);
-                if (do_read) nxt[n] = frag_half(rd_stage, rd_ks, n);
+                if (do_read) {
+#pragma unroll
+                    for (int p = n * kPieces / 16; p < (n + 1) * kPieces / 16; ++p) read_piece(nxt, rd_stage, rd_ks, p);
+                }
                 if (do_load) {
                     if (early) {
                         if (n < 4) {
@@ -357,11 +392,11 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 }
             }
         }
-#pragma unroll
-        for (int n = 0; n < 16; ++n) {
+        static_for<16>([&](auto nc) {
+            constexpr int n = decltype(nc)::value;
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // one LDS read
-        }
+            __builtin_amdgcn_sched_group_barrier(0x100, (n + 1) * kPieces / 16 - n * kPieces / 16, 0);    // its LDS reads
+        });
     };
 
     // prologue: slice 0 and the X half of slice 1; wait for slice 0; read its first fragments
@@ -376,7 +411,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     }
     __syncthreads();
 #pragma unroll
-    for (int n = 0; n < 16; ++n) fa[n] = frag_half(0, 0, n);
+    for (int p = 0; p < kPieces; ++p) read_piece(fa, 0, 0, p);
 
     // slice kt lives in stage kt & 1.  Sub-step 0: MFMAs on its first half, read its second half, send the
     // Y half of slice kt+1 on its way (its X half went out during the previous sub-step 1).  Barrier: slice
@@ -417,6 +452,21 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     constexpr int kChunksPerRow = 128 * kEsz / 16;      // 16 (2-byte) or 32 (float)
     constexpr int kRowsPerPass = 64 / kChunksPerRow;    // 4 or 2
     constexpr int kElemsPerChunk = 16 / kEsz;           // 8 or 4
+    if (!plain) {
+        static_for<4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            static_for<4>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    store_quad_slow<OT>(D, row0 + wr * 128 + i * 32 + l32, col0 + wc * 128 + j * 32 + q * 8 + lh * 4, NR, NC,
+                                        alpha, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                        acc[i][j][4 * q + 3], accumulate, bias, bias_dt);
+                }
+            });
+        });
+        return;
+    }
     static_for<4>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
         static_for<4>([&](auto jc) {
@@ -452,26 +502,19 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 const int pc = lane % kChunksPerRow;
                 const int grow = row0 + wr * 128 + i * 32 + pr;
                 const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
-                if (grow < NR && gcol < NC) {
-                    OT* out = D + static_cast<size_t>(grow) * NC + gcol;
-                    if (plain && gcol + kElemsPerChunk <= NC) {
-                        *reinterpret_cast<uint4*>(out) = val[u];
-                    } else {
-                        store_chunk_slow<OT>(out, val[u], gcol, NC, accumulate, bias, bias_dt);
-                    }
-                }
+                if (grow < NR && gcol < NC) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = val[u];
             }
         });
         __builtin_amdgcn_s_waitcnt(0xC07F);    // patch reads done before the next block overwrites it
     });
 }
 
-template <int XF, int YF, typename OT>
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
 static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                            const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     constexpr int smem = 2 * kDmaStage;
     static bool configured = false;
-    auto kern = fp8_gemm_dma_kernel<XF, YF, OT>;
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT>;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel)");
@@ -535,9 +578,61 @@ static int pick_out(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, in
     }
 }
 
+// K-major operands: only the direct-to-LDS kernel reads them, so the shape must suit it
+static bool kmajor_shape_ok(int NR, int NC, int K, bool xt, bool yt) {
+    const bool fits32 = static_cast<unsigned long long>(NR) * K < (1ull << 32) && static_cast<unsigned long long>(NC) * K < (1ull << 32);
+    return K % kBK == 0 && fits32 && (!xt || NR % kDmaTile == 0) && (!yt || NC % kDmaTile == 0);
+}
+
+template <int XF, int YF, bool XT, bool YT>
+static int pick_out_kmajor(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, int NR, int NC, int K, const float* xs,
+                           const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    switch (d_dtype) {
+        case MSAMP_DT_F32:
+            return launch_gemm_dma<XF, YF, float, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+        case MSAMP_DT_F16:
+            return launch_gemm_dma<XF, YF, f16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+        default:
+            return launch_gemm_dma<XF, YF, bf16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    }
+}
+
+template <bool XT, bool YT>
+static int pick_types_kmajor(const uint8_t* X, int x_type, const uint8_t* Y, int y_type, void* D, int d_dtype, int NR, int NC,
+                             int K, const float* xs, const float* ys, int accumulate, const void* bias, int bias_dt,
+                             hipStream_t st) {
+    if (x_type == MSAMP_DT_E4M3 && y_type == MSAMP_DT_E4M3)
+        return pick_out_kmajor<MSAMP_DT_E4M3, MSAMP_DT_E4M3, XT, YT>(X, Y, D, d_dtype, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    if (x_type == MSAMP_DT_E4M3)
+        return pick_out_kmajor<MSAMP_DT_E4M3, MSAMP_DT_E5M2, XT, YT>(X, Y, D, d_dtype, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    if (y_type == MSAMP_DT_E4M3)
+        return pick_out_kmajor<MSAMP_DT_E5M2, MSAMP_DT_E4M3, XT, YT>(X, Y, D, d_dtype, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    return pick_out_kmajor<MSAMP_DT_E5M2, MSAMP_DT_E5M2, XT, YT>(X, Y, D, d_dtype, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+}
+
 }    // namespace msamp
 
 using namespace msamp;
+
+extern "C" int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
+                                     int b_type, const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int m, int n,
+                                     int k, int accumulate, const void* bias, int bias_dtype, msamp_stream_t stream) {
+    if (!a_kmajor && !b_kmajor)
+        return msamp_fp8_gemm(a, a_type, a_scale_inv, b, b_type, b_scale_inv, d, d_dtype, m, n, k, accumulate, bias, bias_dtype, stream);
+    MSAMP_REQUIRE(is_fp8(a_type) && is_fp8(b_type), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_kmajor: operand types %d, %d", a_type, b_type);
+    MSAMP_REQUIRE(is_hp(d_dtype), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_kmajor: output dtype %d", d_dtype);
+    MSAMP_REQUIRE(bias == nullptr || is_hp(bias_dtype), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_kmajor: bias dtype %d", bias_dtype);
+    MSAMP_REQUIRE(a_kmajor, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_kmajor: b may be K-major only together with a");
+    MSAMP_REQUIRE(m > 0 && n > 0 && k > 0 && kmajor_shape_ok(n, m, k, b_kmajor != 0, true), MSAMP_ERR_SHAPE,
+                  "msamp_fp8_gemm_kmajor: m=%d n=%d k=%d (k %% 128 and the K-major operands' rows %% 256 must be 0)", m, n, k);
+    MSAMP_REQUIRE(a && b && d && a_scale_inv && b_scale_inv, MSAMP_ERR_NULL, "msamp_fp8_gemm_kmajor: null pointer");
+    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16), MSAMP_ERR_SHAPE, "msamp_fp8_gemm_kmajor: operands must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // X = b (rows of D), Y = a (columns of D)
+    if (b_kmajor)
+        return pick_types_kmajor<true, true>(b, b_type, a, a_type, d, d_dtype, n, m, k, b_scale_inv, a_scale_inv, accumulate, bias, bias_dtype, st);
+    return pick_types_kmajor<false, true>(b, b_type, a, a_type, d, d_dtype, n, m, k, b_scale_inv, a_scale_inv, accumulate, bias, bias_dtype, st);
+}
 
 extern "C" int msamp_fp8_gemm(const uint8_t* a, int a_type, const float* a_scale_inv, const uint8_t* b, int b_type,
                               const float* b_scale_inv, void* d, int d_dtype, int m, int n, int k, int accumulate,

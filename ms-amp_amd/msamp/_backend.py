@@ -44,6 +44,7 @@ _SIGNATURES = {
     'msamp_cast_to_fp8_gated': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp], _i),
     'msamp_cast_transpose_gated': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp], _i),
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
@@ -285,11 +286,33 @@ def scale_cast(x, scale, out_dtype):
 
 
 # ---- GEMM ---------------------------------------------------------------------------------------
-def fp8_gemm(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, out, accumulate=False, bias=None):
-    """out[N,M] (+)= (b[N,K] . a[M,K]^T) * a_scale_inv * b_scale_inv (+ bias[M])."""
+def gemm_kmajor_supported(m, n, k, a_kmajor, b_kmajor):
+    """Shapes the kernel reads K-major operands for (see msamp_fp8_gemm_kmajor)."""
+    if b_kmajor and not a_kmajor:
+        return False
+    return k % 128 == 0 and (not a_kmajor or m % 256 == 0) and (not b_kmajor or n % 256 == 0) and \
+        m * k < 2**32 and n * k < 2**32
+
+
+def fp8_gemm(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, out, accumulate=False, bias=None, a_kmajor=False, b_kmajor=False):
+    """out[N,M] (+)= (b[N,K] . a[M,K]^T) * a_scale_inv * b_scale_inv (+ bias[M]).
+    With a_kmajor / b_kmajor the tensor handed over is the transpose, [K,M] / [K,N]."""
     lib = load()
     _gpu(a, 'mat_a')
     _gpu(b, 'mat_b')
+    if a_kmajor or b_kmajor:
+        k, m = a.shape if a_kmajor else a.shape[::-1]
+        kb, n = b.shape if b_kmajor else b.shape[::-1]
+        if kb != k or tuple(out.shape) != (n, m):
+            raise ValueError(f'shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}, out {tuple(out.shape)}')
+        _check(
+            lib.msamp_fp8_gemm_kmajor(
+                _ptr(a), a_dt, _ptr(a_scale_inv), 1 if a_kmajor else 0, _ptr(b), b_dt, _ptr(b_scale_inv),
+                1 if b_kmajor else 0, _ptr(out), _dt(out), m, n, k, 1 if accumulate else 0, _ptr(bias),
+                _dt(bias) if bias is not None else DT_F32, _stream()
+            ), 'msamp_fp8_gemm_kmajor'
+        )
+        return out
     m, k = a.shape
     n = b.shape[0]
     if b.shape[1] != k or tuple(out.shape) != (n, m):

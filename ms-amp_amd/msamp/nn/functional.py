@@ -30,22 +30,40 @@ class _FP8GemmFunction(torch.autograd.Function):
     def backward(ctx, output_grad):
         output_grad = output_grad.contiguous()
         metas = ctx.metas
-        ograd_fp8, ograd_fp8_t = output_grad.fused_cast_transpose(Dtypes.kfloat8_e5m2, meta=metas['ograd'])
+        tokens, d_out = output_grad.shape
+        d_in = ctx.input_fp8.shape[1]
+        need_dgrad, need_wgrad = ctx.input_fp8.requires_grad, ctx.weight.requires_grad
+        # The reference materializes dy^T, W^T and x^T (fused cast-transpose + two FP8 transposes) because its
+        # GEMM reads K-contiguous operands only.  This kernel also reads [K, rows] operands in place, so when
+        # the shapes allow, dy is only cast and W, x, dy go to the GEMMs as they are (same results).
+        in_place = (not need_dgrad or Gemm.kmajor_supported(d_in, tokens, d_out, True, False)) and \
+            (not need_wgrad or Gemm.kmajor_supported(d_in, d_out, tokens, True, True))
+        if in_place:
+            ograd_fp8 = output_grad.cast(Dtypes.kfloat8_e5m2, meta=metas['ograd'])
+            ograd_fp8_t = None
+        else:
+            ograd_fp8, ograd_fp8_t = output_grad.fused_cast_transpose(Dtypes.kfloat8_e5m2, meta=metas['ograd'])
 
         input_grad = None
-        if ctx.input_fp8.requires_grad:
-            weight_fp8_t = ctx.weight_fp8.fp8_transpose()
-            input_grad = Gemm.fp8_gemm(weight_fp8_t, ograd_fp8, ctx.output_qtype, use_split_accumulator=True)
+        if need_dgrad:
+            if in_place:
+                input_grad = Gemm.fp8_gemm(ctx.weight_fp8, ograd_fp8, ctx.output_qtype, use_split_accumulator=True, a_kmajor=True)
+            else:
+                weight_fp8_t = ctx.weight_fp8.fp8_transpose()
+                input_grad = Gemm.fp8_gemm(weight_fp8_t, ograd_fp8, ctx.output_qtype, use_split_accumulator=True)
 
-        if ctx.weight.requires_grad:
-            input_fp8_t = ctx.input_fp8.fp8_transpose()
+        if need_wgrad:
+            if in_place:
+                mat_a, mat_b, layout = ctx.input_fp8, ograd_fp8, dict(a_kmajor=True, b_kmajor=True)
+            else:
+                mat_a, mat_b, layout = ctx.input_fp8.fp8_transpose(), ograd_fp8_t, {}
             if ctx.weight.grad is None:
-                wgrad = Gemm.fp8_gemm(input_fp8_t, ograd_fp8_t, ctx.output_qtype, use_split_accumulator=True)
+                wgrad = Gemm.fp8_gemm(mat_a, mat_b, ctx.output_qtype, use_split_accumulator=True, **layout)
             else:
                 # gradient accumulation: add into the dequantized previous gradient
                 old_wgrad = ctx.weight.grad.to(ctx.output_dtype)
                 wgrad = Gemm.fp8_gemm(
-                    input_fp8_t, ograd_fp8_t, ctx.output_qtype, accumulate=True, out=old_wgrad, use_split_accumulator=True
+                    mat_a, mat_b, ctx.output_qtype, accumulate=True, out=old_wgrad, use_split_accumulator=True, **layout
                 )
                 del old_wgrad
             if model_state.use_fp8_ddp:

@@ -18,20 +18,52 @@ class Gemm:
         return (value + base - 1) // base * base
 
     @classmethod
+    def kmajor_supported(cls, m, n, k, a_kmajor=True, b_kmajor=False):
+        """True if fp8_gemm reads K-major operands of this problem in place (else it transposes them first)."""
+        return _backend.gemm_kmajor_supported(m, n, k, a_kmajor, b_kmajor)
+
+    @classmethod
     @torch.no_grad()
-    def fp8_gemm(cls, mat_a, mat_b, out_qtype, bias=None, accumulate=False, out=None, use_split_accumulator=False):
+    def fp8_gemm(
+        cls, mat_a, mat_b, out_qtype, bias=None, accumulate=False, out=None, use_split_accumulator=False, a_kmajor=False,
+        b_kmajor=False
+    ):
         """out[N, M] = (mat_b[N, K] @ mat_a[M, K].T) * a.scale_inv * b.scale_inv.
 
         mat_a, mat_b: contiguous FP8 ScalingTensors on the GPU.  The kernel accumulates in fp32
         over the full K (use_split_accumulator has nothing to switch) and writes out_qtype; with
         `accumulate` it adds into `out`.  Only K needs padding (to a multiple of 16 bytes, with
         FP8 zeros); ragged M and N are handled inside the kernel.
+
+        a_kmajor / b_kmajor (not in the reference): the tensor passed is the transpose of the operand,
+        [K, M] / [K, N], as the backward pass of a linear layer has them; the kernel reads it in place
+        when the shape allows, otherwise it is transposed first.  Same result either way.
         """
         assert isinstance(mat_a, ScalingTensor)
         assert isinstance(mat_b, ScalingTensor)
         assert mat_a.is_cuda and mat_a.is_contiguous()
         assert mat_b.is_cuda and mat_b.is_contiguous()
         assert Dtypes.is_fp8_qtype(mat_a.qtype) and Dtypes.is_fp8_qtype(mat_b.qtype)
+
+        if a_kmajor or b_kmajor:
+            K, M = mat_a.shape if a_kmajor else mat_a.shape[::-1]
+            N = mat_b.shape[1] if b_kmajor else mat_b.shape[0]
+            if cls.kmajor_supported(M, N, K, a_kmajor, b_kmajor):
+                out_dtype = Dtypes.get_dtype_from_qtype(out_qtype)
+                if out is None:
+                    assert not accumulate, 'accumulate needs an output tensor'
+                    out = torch.empty(N, M, dtype=out_dtype, device=mat_a.device)
+                else:
+                    assert out.is_cuda and out.is_contiguous() and out.dtype == out_dtype
+                _backend.fp8_gemm(
+                    mat_a.value, int(mat_a.qtype), mat_a.meta.scale_inv, mat_b.value, int(mat_b.qtype), mat_b.meta.scale_inv,
+                    out, accumulate, bias, a_kmajor=a_kmajor, b_kmajor=b_kmajor
+                )
+                return out
+            if a_kmajor:
+                mat_a = mat_a.fp8_transpose()
+            if b_kmajor:
+                mat_b = mat_b.fp8_transpose()
 
         M, K = mat_a.shape
         N = len(mat_b)

@@ -280,6 +280,38 @@ def test_training_step_replays_from_a_graph():
     assert model.scaling_metas['input'].amax_counter.item() == steps
 
 
+def test_backward_without_transposed_copies_matches_the_explicit_path(monkeypatch):
+    """At shapes the kernel reads K-major operands for, the backward pass skips dy^T, W^T and x^T; gradients and
+    metas must equal, bit for bit, what the path with the three explicit transposes gives."""
+    from msamp.operators.gemm import Gemm
+    tokens, d_in, d_out = 512, 256, 768
+    torch.manual_seed(9)
+    w0 = (torch.randn(d_out, d_in) * 0.05).bfloat16()
+    x0 = torch.randn(tokens, d_in).bfloat16().cuda()
+    dy = (torch.randn(tokens, d_out) * 1e-3).bfloat16().cuda()
+    assert Gemm.kmajor_supported(d_in, tokens, d_out, True, False) and Gemm.kmajor_supported(d_in, d_out, tokens, True, True)
+
+    def run(accumulate_twice):
+        model_state.clear()
+        lin = torch.nn.Linear(d_in, d_out, bias=False).cuda().bfloat16()
+        with torch.no_grad():
+            lin.weight.copy_(w0)
+        model = LinearReplacer.replace(lin, Dtypes.kbfloat16)
+        x = x0.clone().requires_grad_(True)
+        for _ in range(2 if accumulate_twice else 1):    # the second pass accumulates into the FP8 weight gradient
+            model(x).backward(dy)
+        g = model.weight.grad
+        return x.grad.clone(), g.value.clone(), g.meta.scale_inv.clone(), {k: m.amax.clone() for k, m in model.scaling_metas.items()}
+
+    for twice in (False, True):
+        fast = run(twice)
+        with monkeypatch.context() as mp:
+            mp.setattr(Gemm, 'kmajor_supported', classmethod(lambda cls, *a, **k: False))
+            slow = run(twice)
+        assert torch.equal(fast[0], slow[0]) and torch.equal(fast[1], slow[1]) and same_float(fast[2], slow[2])
+        assert all(same_float(fast[3][k], slow[3][k]) for k in fast[3])
+
+
 def test_optimizer_state_dict_round_trip():
     torch.manual_seed(7)
     x = torch.randn(4, 4, device='cuda')

@@ -118,6 +118,42 @@ def test_large_tiles_ragged_edges_accumulate_bias(be, m, n, k, out_dtype):
     assert (buf[0] == 7).all() and (buf[n + 1] == 7).all() and torch.equal(buf[1:n + 1], got)
 
 
+@pytest.mark.parametrize('a_dt,b_dt', [(5, 5), (5, 6), (6, 5)])
+@pytest.mark.parametrize('m,n,k', [(256, 256, 128), (512, 768, 384), (1024, 300, 256), (4096, 4096, 512)])
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16])
+def test_kmajor_operands_match_transposed_copies(be, a_dt, b_dt, m, n, k, out_dtype):
+    """Operands handed over as [K, rows] must give exactly what the row-major kernel gives on their transposed
+    copies (same products, same order): `a` alone K-major for any n, both K-major when n is a multiple of 256;
+    with bias and accumulation as well."""
+    a = _rand_fp8((m, k), a_dt, 11 * m + k).cuda()
+    b = _rand_fp8((n, k), b_dt, 13 * n + k, spread=0.5).cuda()
+    a_t, b_t = a.t().contiguous(), b.t().contiguous()
+    sa, sb = torch.tensor(0.25, device='cuda'), torch.tensor(2.0, device='cuda')
+    want = be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'))
+    got = be.fp8_gemm(a_t, a_dt, sa, b, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'), a_kmajor=True)
+    assert torch.equal(got, want)
+    assert be.gemm_kmajor_supported(m, n, k, True, True) == (n % 256 == 0)
+    if n % 256 == 0:
+        got = be.fp8_gemm(a_t, a_dt, sa, b_t, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'), a_kmajor=True,
+                          b_kmajor=True)
+        assert torch.equal(got, want)
+        bias = torch.randn(m, device='cuda').to(out_dtype)
+        base = torch.randn(n, m, device='cuda').to(out_dtype)
+        want2 = be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, base.clone(), accumulate=True, bias=bias)
+        got2 = be.fp8_gemm(a_t, a_dt, sa, b_t, b_dt, sb, base.clone(), accumulate=True, bias=bias, a_kmajor=True, b_kmajor=True)
+        assert torch.equal(got2, want2)
+
+
+def test_kmajor_rejects_unsupported_shapes(be):
+    a = _rand_fp8((128, 100), 5, 1).cuda()    # [K=128, M=100]: M is not a multiple of 256
+    b = _rand_fp8((64, 128), 5, 2).cuda()
+    one = torch.ones((), device='cuda')
+    with pytest.raises(RuntimeError):
+        be.fp8_gemm(a, 5, one, b, 5, one, torch.empty(64, 100, device='cuda'), a_kmajor=True)
+    assert not be.gemm_kmajor_supported(100, 64, 128, True, False)
+    assert not be.gemm_kmajor_supported(256, 256, 128, False, True)
+
+
 def test_k_not_multiple_of_16_is_padded_by_the_operator():
     import msamp    # noqa: F401
     from msamp.common.dtype import Dtypes
