@@ -105,6 +105,14 @@ int msamp_cast_to_fp8_gated(const void* x, int in_dtype, size_t n, float* scale,
                             uint8_t* out, int fp8_type, int margin, int flags, const int32_t* warmup_counter, int window,
                             void* workspace, msamp_stream_t stream);
 
+/* Arithmetic.add_to_fp8 (msamp/operators/arithmetic/arithmetic.py:15-35, vectorized_pointwise.h:184-301): in place,
+ * q <- in-time cast of (T(dequant(q)) + other), T = other's dtype, the sum rounded to T as torch adds two T tensors;
+ * amax[0] = max|sum|, *scale by the rule (fallback the old *scale), *scale_inv = 1 / *scale.  Equal, bit for bit, to
+ * (q.to(T) + other).cast(qtype, meta) -- the identity the reference's own test demands (tests/operators/
+ * test_arithmetic.py:25-42). */
+int msamp_add_to_fp8(uint8_t* q, int fp8_type, size_t n, float* scale, float* scale_inv, float* amax, const void* other,
+                     int other_dtype, void* workspace, msamp_stream_t stream);
+
 /* tex.cast_from_fp8 (transformer_engine_wrapper.py:123-137): out[i] = otype(float(q[i]) * *scale_inv). */
 int msamp_cast_from_fp8(const uint8_t* q, int fp8_type, size_t n, const float* scale_inv, void* out, int out_dtype,
                         msamp_stream_t stream);

@@ -1121,6 +1121,100 @@ static int launch_scale_cast_out(const IT* x, size_t n, const float* scale, void
     return MSAMP_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// add_to_fp8: q <- cast_in_time(IT(dequant(q)) + other), in place (operators/arithmetic/arithmetic.py:15-35,
+// vectorized_pointwise.h:184-301).  t = IT(float(q) * scale_inv) + other with the sum rounded to IT, as
+// torch adds two IT tensors; amax = max|t|; scale by the rule; q = fp8(float(t) * scale).  Two passes over
+// q and other; the old scale_inv travels in workspace word kWsOldScaleInv because the second pass replaces it.
+constexpr int kWsOldScaleInv = 6;
+
+template <typename IT>
+__device__ __forceinline__ float round_to(float v) {
+    if constexpr (sizeof(IT) == 4) return v;
+    else if constexpr (__is_same(IT, bf16_t)) return bf16_bits_to_float(float_to_bf16_bits(v));
+    else return f16_bits_to_float(float_to_f16_bits(v));
+}
+
+template <typename IT, int FMT>
+__device__ __forceinline__ float add_term(uint32_t code, float other, float si) {
+    return round_to<IT>(round_to<IT>(dequant1<FMT>(code) * si) + other);
+}
+
+template <typename IT, int FMT>
+__global__ __launch_bounds__(kCastThreads) void add_amax_partial_kernel(const uint8_t* __restrict__ q,
+                                                                         const IT* __restrict__ other, size_t n,
+                                                                         uint32_t* ws, const float* scale,
+                                                                         const float* scale_inv, int vec_ok) {
+    __shared__ uint32_t red[kCastThreads / kWave];
+    const float si = *scale_inv;
+    uint32_t m = 0;
+    const size_t stride = static_cast<size_t>(gridDim.x) * kCastThreads * 4;
+    for (size_t i = (static_cast<size_t>(blockIdx.x) * kCastThreads + threadIdx.x) * 4; i < n; i += stride) {
+        if (i + 4 <= n && vec_ok) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(q + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float t = add_term<IT, FMT>((w >> (8 * j)) & 0xffu, Elem<IT>::load(other + i + j), si);
+                m = umax(m, __float_as_uint(t) & 0x7fffffffu);
+            }
+        } else {
+            for (size_t e = i; e < n && e < i + 4; ++e) {
+                const float t = add_term<IT, FMT>(q[e], Elem<IT>::load(other + e), si);
+                m = umax(m, __float_as_uint(t) & 0x7fffffffu);
+            }
+        }
+    }
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0) {
+        ws[kWsPartials + blockIdx.x] = m;
+        if (blockIdx.x == 0) {
+            ws[0] = __float_as_uint(*scale);
+            ws[1] = gridDim.x;
+            ws[kWsOldScaleInv] = __float_as_uint(si);
+        }
+    }
+}
+
+template <typename IT, int FMT>
+__global__ __launch_bounds__(kCastThreads) void add_cast_kernel(uint8_t* __restrict__ q, const IT* __restrict__ other,
+                                                                 size_t n, float* scale_inv, InTimeArgs it, int vec_ok) {
+    __shared__ uint32_t red[kCastThreads / kWave];
+    const float si = __uint_as_float(it.ws[kWsOldScaleInv]);
+    const float s = resolve_in_time_scale(it, red, scale_inv);
+    const size_t stride = static_cast<size_t>(gridDim.x) * kCastThreads * 4;
+    for (size_t i = (static_cast<size_t>(blockIdx.x) * kCastThreads + threadIdx.x) * 4; i < n; i += stride) {
+        if (i + 4 <= n && vec_ok) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(q + i);
+            float t[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) t[j] = add_term<IT, FMT>((w >> (8 * j)) & 0xffu, Elem<IT>::load(other + i + j), si);
+            *reinterpret_cast<uint32_t*>(q + i) = quant4<FMT>(t[0] * s, t[1] * s, t[2] * s, t[3] * s);
+        } else {
+            for (size_t e = i; e < n && e < i + 4; ++e)
+                q[e] = static_cast<uint8_t>(quant1<FMT>(add_term<IT, FMT>(q[e], Elem<IT>::load(other + e), si) * s));
+        }
+    }
+}
+
+template <typename IT>
+static int launch_add_to_fp8(uint8_t* q, int fp8_type, const IT* other, size_t n, float* scale, float* scale_inv, float* amax,
+                             uint32_t* ws, hipStream_t st) {
+    int grid = grid_for(n, static_cast<size_t>(kCastThreads) * 4 * 4);
+    const int cap = cu_count() * 4 < kMaxPartials ? cu_count() * 4 : kMaxPartials;
+    grid = grid < cap ? grid : cap;
+    const InTimeArgs it = {ws, scale, amax, fp8_max(fp8_type), 0, 0, nullptr, nullptr, nullptr, 0, nullptr};
+    const int vec_ok = aligned(q, 4);
+    if (fp8_type == MSAMP_DT_E4M3) {
+        hipLaunchKernelGGL((add_amax_partial_kernel<IT, MSAMP_DT_E4M3>), dim3(grid), dim3(kCastThreads), 0, st, q, other, n, ws, scale, scale_inv, vec_ok);
+        hipLaunchKernelGGL((add_cast_kernel<IT, MSAMP_DT_E4M3>), dim3(grid), dim3(kCastThreads), 0, st, q, other, n, scale_inv, it, vec_ok);
+    } else {
+        hipLaunchKernelGGL((add_amax_partial_kernel<IT, MSAMP_DT_E5M2>), dim3(grid), dim3(kCastThreads), 0, st, q, other, n, ws, scale, scale_inv, vec_ok);
+        hipLaunchKernelGGL((add_cast_kernel<IT, MSAMP_DT_E5M2>), dim3(grid), dim3(kCastThreads), 0, st, q, other, n, scale_inv, it, vec_ok);
+    }
+    MSAMP_CHECK_LAUNCH("add_to_fp8 kernels");
+    return MSAMP_OK;
+}
+
 }    // namespace msamp
 
 using namespace msamp;
@@ -1185,6 +1279,24 @@ int msamp_cast_scaled_to_fp8(const void* x, int in_dtype, size_t n, const float*
     MSAMP_REQUIRE(amax_out == nullptr || window >= 1, MSAMP_ERR_SHAPE, "msamp_cast_scaled_to_fp8: window %d", window);
     const InTimeArgs it = {nullptr, scale, nullptr, fp8_max(fp8_type), margin, 0, amax, old_scale_inv, amax_out, window, counter_out};
     return dispatch_cast(x, in_dtype, n, nullptr, nullptr, scale_inv, out, fp8_type, &it, static_cast<hipStream_t>(stream));
+}
+
+int msamp_add_to_fp8(uint8_t* q, int fp8_type, size_t n, float* scale, float* scale_inv, float* amax, const void* other,
+                     int other_dtype, void* workspace, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_add_to_fp8: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(is_hp(other_dtype), MSAMP_ERR_DTYPE, "msamp_add_to_fp8: other_dtype %d", other_dtype);
+    MSAMP_REQUIRE(scale && scale_inv && amax && ((q && other) || n == 0), MSAMP_ERR_NULL, "msamp_add_to_fp8: null pointer");
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_add_to_fp8: workspace required");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint32_t* ws = static_cast<uint32_t*>(workspace);
+    switch (other_dtype) {
+        case MSAMP_DT_F32:
+            return launch_add_to_fp8(q, fp8_type, static_cast<const float*>(other), n, scale, scale_inv, amax, ws, st);
+        case MSAMP_DT_F16:
+            return launch_add_to_fp8(q, fp8_type, static_cast<const f16_t*>(other), n, scale, scale_inv, amax, ws, st);
+        default:
+            return launch_add_to_fp8(q, fp8_type, static_cast<const bf16_t*>(other), n, scale, scale_inv, amax, ws, st);
+    }
 }
 
 int msamp_cast_from_fp8(const uint8_t* q, int fp8_type, size_t n, const float* scale_inv, void* out, int out_dtype,

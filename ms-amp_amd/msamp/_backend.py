@@ -35,6 +35,7 @@ _SIGNATURES = {
     'msamp_cast_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp], _i),
     'msamp_cast_to_fp8_intime': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
     'msamp_cast_scaled_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp], _i),
+    'msamp_add_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp, _vp], _i),
     'msamp_cast_from_fp8': ([_vp, _i, _sz, _vp, _vp, _i, _vp], _i),
     'msamp_cast_transpose': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp], _i),
     'msamp_cast_transpose_intime': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
@@ -215,6 +216,20 @@ def cast_scaled_to_fp8(x, amax, old_scale_inv, scale, scale_inv, fp8_dt, margin=
         ), 'msamp_cast_scaled_to_fp8'
     )
     return out
+
+
+def add_to_fp8(q, fp8_dt, scale, scale_inv, amax_cell, other):
+    """In place: q <- in-time cast of (dequant(q) in other's dtype + other); rewrites scale, scale_inv, amax."""
+    lib = load()
+    _gpu(q, 'fp8 tensor')
+    _gpu(other, 'other')
+    _check(
+        lib.msamp_add_to_fp8(
+            _ptr(q), fp8_dt, q.numel(), _ptr(scale), _ptr(scale_inv), _ptr(amax_cell), _ptr(other), _dt(other),
+            _ptr(workspace(q.device)), _stream()
+        ), 'msamp_add_to_fp8'
+    )
+    return q
 
 
 def cast_from_fp8(q, scale_inv, fp8_dt, out_dtype):

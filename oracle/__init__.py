@@ -16,6 +16,9 @@ Pinning status of each function (what fixes its output besides its own formula):
   the special-value table read from msamp/common/tensor/meta.py:51-56.
 * ``scaling.update_scaling_factors``: the window sequence of
   tests/optim/test_adamw.py:203-220.
+* ``arithmetic.add_to_fp8``: the identity the reference's test demands
+  (tests/operators/test_arithmetic.py:25-42: equal to dequantize, add, in-time cast) and a
+  hand-worked case.
 * ``gemm.fp8_gemm``: definition (fp32 matmul of dequantized operands) and the exact
   case of tests/operators/test_gemm.py:45-56.
 * ``adamw.*``: textbook AdamW against ``torch.optim.AdamW`` to the reference's own
