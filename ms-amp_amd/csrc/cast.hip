@@ -336,7 +336,9 @@ __device__ __forceinline__ uint32_t abs_bits_hi(uint32_t raw) {    // raw elemen
     else return (raw << 16) & 0x7fff0000u;
 }
 
-template <typename IT, int FMT>
+// R = vectors per lane the kernel is built for (the host picks the smallest of 4 / 8 / 16 that covers the
+// tensor, so that a small tensor does not pay for loads it has no use for).
+template <typename IT, int FMT, int R>
 __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void cast_intime_resident_kernel(const IT* __restrict__ x,
                                                                            uint8_t* __restrict__ out, size_t n,
                                                                            float* scale, float* amax, float* scale_inv,
@@ -354,9 +356,9 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
     const uint32_t v0 = blockIdx.x * static_cast<uint32_t>(rounds) * kResThreads + tid;
     const float old_scale = *scale;    // read before any workgroup can pass the meeting and replace it
 
-    uint4 v[kResVecs];
+    uint4 v[R];
 #pragma unroll
-    for (int r = 0; r < kResVecs; ++r) {
+    for (int r = 0; r < R; ++r) {
         // unconditional (clamped) loads, so that all of them are in flight together; a vector read
         // twice changes no maximum, and the store phase skips the duplicates
         const uint32_t idx = v0 + r * kResThreads;
@@ -370,7 +372,7 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
 
     uint32_t m = abs_bits_hi<IT>(tail_raw);
 #pragma unroll
-    for (int r = 0; r < kResVecs; ++r) {
+    for (int r = 0; r < R; ++r) {
         const uint32_t w[4] = {v[r].x, v[r].y, v[r].z, v[r].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -426,7 +428,7 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
 
     if (in_range) {
 #pragma unroll
-        for (int r = 0; r < kResVecs; ++r) {
+        for (int r = 0; r < R; ++r) {
             // keep only the raw words live across the barrier, not values derived from them before it
             asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
             const uint32_t idx = v0 + r * kResThreads;
@@ -443,7 +445,7 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
         }
     } else {
 #pragma unroll
-        for (int r = 0; r < kResVecs; ++r) {
+        for (int r = 0; r < R; ++r) {
             asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
             const uint32_t idx = v0 + r * kResThreads;
             if (r < rounds && idx < nvec) {
@@ -987,10 +989,7 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
     // a captured launch would replay this call's token, and the slots of the previous replay still carry it
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return 1;
-    const void* fn = fp8_type == MSAMP_DT_E4M3
-                         ? reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E4M3>)
-                         : reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E5M2>);
-    if (!fits_resident(fn)) return 1;
+    if (!fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E4M3, kResVecs>))) return 1;
     // as many workgroups as there are runs of kResThreads vectors, up to the resident limit
     size_t g = (nvec + kResThreads - 1) / kResThreads;
     g = g > max_blocks ? max_blocks : g;
@@ -1001,9 +1000,12 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
     uint64_t* slots = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + kWsSlotBytes);
     const float fp_max = fp8_max(fp8_type);
     const uint32_t spin_limit = 1u << 20;    // a fraction of a second of polling
-#define LAUNCH(FMT) \
-    hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit)
-    if (fp8_type == MSAMP_DT_E4M3) LAUNCH(MSAMP_DT_E4M3); else LAUNCH(MSAMP_DT_E5M2);
+#define LAUNCH(FMT, R) \
+    hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT, R>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit)
+#define LAUNCH_R(FMT) \
+    do { if (rounds <= 4) LAUNCH(FMT, 4); else if (rounds <= 8) LAUNCH(FMT, 8); else LAUNCH(FMT, kResVecs); } while (0)
+    if (fp8_type == MSAMP_DT_E4M3) LAUNCH_R(MSAMP_DT_E4M3); else LAUNCH_R(MSAMP_DT_E5M2);
+#undef LAUNCH_R
 #undef LAUNCH
     MSAMP_CHECK_LAUNCH("cast_intime_resident_kernel");
     return MSAMP_OK;
