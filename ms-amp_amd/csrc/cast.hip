@@ -328,7 +328,7 @@ constexpr int kResVecs = 16;
 constexpr int kResBlocksPerCu = 2;
 constexpr int kWsSlotBytes = 8192;
 constexpr int kMaxSlots = 512;
-static_assert(kWsSlotBytes + kMaxSlots * 8 <= MSAMP_WORKSPACE_BYTES, "slots exceed the workspace");
+static_assert(kWsSlotBytes + (kMaxSlots + 2) * 8 <= MSAMP_WORKSPACE_BYTES, "slots exceed the workspace");
 
 template <typename IT>
 __device__ __forceinline__ uint32_t abs_bits_hi(uint32_t raw) {    // raw element bits -> ordered key
@@ -387,37 +387,55 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
             __hip_atomic_store(slots + blockIdx.x, (static_cast<uint64_t>(token) << 32) | m, __ATOMIC_RELAXED,
                                __HIP_MEMORY_SCOPE_AGENT);
         }
-        uint32_t spins = 0, mm;
-        bool all_in;
-        do {
-            // all slots of one poll are requested together; the ones past the grid are read and ignored
-            uint64_t sv[kMaxSlots / kWave];
+        // Workgroup 0 collects: it alone polls the slots (everyone polling them costs the workgroups still
+        // loading a good part of their bandwidth), derives amax and scale and posts both, tagged with the
+        // token, in two words behind the slots; the others poll only those.
+        uint64_t* post = slots + kMaxSlots;
+        if (blockIdx.x == 0) {
+            uint32_t spins = 0, mm;
+            bool all_in;
+            do {
+                // all slots of one poll are requested together; the ones past the grid are read and ignored
+                uint64_t sv[kMaxSlots / kWave];
 #pragma unroll
-            for (int j = 0; j < kMaxSlots / kWave; ++j)
-                sv[j] = __hip_atomic_load(slots + tid + j * kWave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            bool ok = true;
-            mm = 0;
+                for (int j = 0; j < kMaxSlots / kWave; ++j)
+                    sv[j] = __hip_atomic_load(slots + tid + j * kWave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                bool ok = true;
+                mm = 0;
 #pragma unroll
-            for (int j = 0; j < kMaxSlots / kWave; ++j) {
-                const bool live = static_cast<uint32_t>(tid + j * kWave) < gridDim.x;
-                ok = ok && (!live || static_cast<uint32_t>(sv[j] >> 32) == token);
-                mm = umax(mm, live ? static_cast<uint32_t>(sv[j]) : 0u);
-            }
-            all_in = __all(ok);
-        } while (!all_in && ++spins < spin_limit);
-        mm = wave_max_u32(mm);
-        if (tid == 0) {
-            float am = __uint_as_float(mm);
-            if (!all_in) am = __uint_as_float(0x7fc00000u);    // the wait ran out: make the failure visible
-            else if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
-            const float s = scale_rule(am, old_scale, fp_max, margin);
-            s_scale = __float_as_uint(s);
-            s_amax = __float_as_uint(am);
-            if (blockIdx.x == 0) {
+                for (int j = 0; j < kMaxSlots / kWave; ++j) {
+                    const bool live = static_cast<uint32_t>(tid + j * kWave) < gridDim.x;
+                    ok = ok && (!live || static_cast<uint32_t>(sv[j] >> 32) == token);
+                    mm = umax(mm, live ? static_cast<uint32_t>(sv[j]) : 0u);
+                }
+                all_in = __all(ok);
+            } while (!all_in && ++spins < spin_limit);
+            mm = wave_max_u32(mm);
+            if (tid == 0) {
+                float am = __uint_as_float(mm);
+                if (!all_in) am = __uint_as_float(0x7fc00000u);    // the wait ran out: make the failure visible
+                else if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
+                const float s = scale_rule(am, old_scale, fp_max, margin);
+                const uint64_t tag = static_cast<uint64_t>(token) << 32;
+                __hip_atomic_store(post, tag | __float_as_uint(am), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(post + 1, tag | __float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                s_scale = __float_as_uint(s);
+                s_amax = __float_as_uint(am);
                 *amax = am;
                 *scale = s;
                 *scale_inv = 1.0f / s;
             }
+        } else if (tid == 0) {
+            uint32_t spins = 0;
+            uint64_t pa, ps;
+            bool posted;
+            do {
+                pa = __hip_atomic_load(post, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ps = __hip_atomic_load(post + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                posted = static_cast<uint32_t>(pa >> 32) == token && static_cast<uint32_t>(ps >> 32) == token;
+            } while (!posted && ++spins < spin_limit);
+            s_amax = posted ? static_cast<uint32_t>(pa) : 0x7fc00000u;
+            s_scale = posted ? static_cast<uint32_t>(ps) : 0x7fc00000u;
         }
     }
     __syncthreads();
