@@ -276,6 +276,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wr = wave >> 1, wc = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
+    // the output factor is fetched now: left to the epilogue, the two scalar loads sit on its critical path
+    float alpha_early = (*x_scale_inv) * (*y_scale_inv);
+    asm volatile("" : "+v"(alpha_early));
 
     // ---- global -> LDS.  A stage holds 256 X rows then 256 Y rows, 128 bytes per row.  One wave
     // instruction fills 8 rows (1 KiB, lane-contiguous): lane l lands in row l/8, 16-byte position l%8,
@@ -363,7 +366,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // consecutive D columns per register quad -- the layout the epilogue wants.
     // EARLY: the loads go out two per MFMA during the first four MFMAs (they are needed soonest).
     auto sub_step = [&](const int* cur, int* nxt, int rd_stage, int rd_ks, bool do_read, int ld_kt, int ld_stage,
-                        int ld_first, bool do_load, bool early) {
+                        int ld_first, bool do_load, int early) {
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
 #pragma unroll
@@ -381,7 +384,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     for (int p = n * kPieces / 16; p < (n + 1) * kPieces / 16; ++p) read_piece(nxt, rd_stage, rd_ks, p);
                 }
                 if (do_load) {
-                    if (early) {
+                    if (early == 2) {
+                        dma(ld_kt, ld_stage, n);    // the whole slice, one load per MFMA
+                    } else if (early == 1) {
                         if (n < 4) {
                             dma(ld_kt, ld_stage, ld_first + 2 * n);
                             dma(ld_kt, ld_stage, ld_first + 2 * n + 1);
@@ -399,6 +404,49 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         });
     };
 
+#ifndef MSAMP_GEMM_SCHED
+#define MSAMP_GEMM_SCHED 1
+#endif
+#if MSAMP_GEMM_SCHED == 1
+    // prologue: slices 0 and 1; wait for slice 0; read its first fragments
+#pragma unroll
+    for (int w = 0; w < 16; ++w) dma(0, 0, w);
+    if (nk > 1) {
+#pragma unroll
+        for (int w = 0; w < 16; ++w) dma(1, 1, w);
+        wait_vmcnt<16>();
+    } else {
+        wait_vmcnt<0>();
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < kPieces; ++p) read_piece(fa, 0, 0, p);
+    // slice kt lives in stage kt & 1 and slice kt+1 is already on its way.  Sub-step 0: MFMAs on the first half,
+    // read the second half.  Barrier: slice kt+1 has landed, nobody needs the LDS copy of slice kt.  Sub-step 1:
+    // MFMAs on the second half, read the first half of slice kt+1, refill this stage with all of slice kt+2.
+    int kt = 0;
+    for (; kt + 3 < nk; kt += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            sub_step(fa, fb, u, 1, true, 0, 0, 0, false, 0);
+            wait_vmcnt<0>();
+            __syncthreads();
+            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, 0, true, 2);
+        }
+    }
+    for (; kt < nk; kt += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k1 = kt + u;
+            if (k1 < nk) {
+                sub_step(fa, fb, u, 1, true, 0, 0, 0, false, 0);
+                wait_vmcnt<0>();
+                __syncthreads();
+                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, 0, k1 + 2 < nk, 2);
+            }
+        }
+    }
+#else
     // prologue: slice 0 and the X half of slice 1; wait for slice 0; read its first fragments
 #pragma unroll
     for (int w = 0; w < 16; ++w) dma(0, 0, w);
@@ -421,10 +469,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     for (; kt + 3 < nk; kt += 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            sub_step(fa, fb, u, 1, true, kt + u + 1, u ^ 1, 8, true, true);
+            sub_step(fa, fb, u, 1, true, kt + u + 1, u ^ 1, 8, true, 1);
             wait_vmcnt<0>();
             __syncthreads();
-            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, 0, true, false);
+            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, 0, true, 0);
         }
     }
     for (; kt < nk; kt += 2) {
@@ -432,13 +480,14 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         for (int u = 0; u < 2; ++u) {
             const int k1 = kt + u;
             if (k1 < nk) {
-                sub_step(fa, fb, u, 1, true, k1 + 1, u ^ 1, 8, k1 + 1 < nk, true);
+                sub_step(fa, fb, u, 1, true, k1 + 1, u ^ 1, 8, k1 + 1 < nk, 1);
                 wait_vmcnt<0>();
                 __syncthreads();
-                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, 0, k1 + 2 < nk, false);
+                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, 0, k1 + 2 < nk, 0);
             }
         }
     }
+#endif
     wait_vmcnt<0>();
     __syncthreads();    // LDS is reused below
 
@@ -446,7 +495,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     constexpr int kEsz = static_cast<int>(sizeof(OT));
     constexpr int kPitch = 128 * kEsz + 16;    // bytes per patch row (padding staggers the banks)
     uint8_t* patch = smem + wave * (32 * kPitch);
-    const float alpha = (*x_scale_inv) * (*y_scale_inv);
+    const float alpha = alpha_early;
     const bool vec_ok = (NC % (16 / kEsz) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
     const bool plain = vec_ok && !accumulate && bias == nullptr;
     constexpr int kChunksPerRow = 128 * kEsz / 16;      // 16 (2-byte) or 32 (float)
@@ -486,26 +535,29 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 }
             }
         });
-        __builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0): the patch is written (same wave reads it back)
+        // no wait between the writes above and the reads below, nor before the next block's writes: the patch is
+        // private to this wave and the LDS serves one wave's requests in order
         constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
         static_for<kPasses / 8>([&](auto gc) {
             constexpr int p0 = decltype(gc)::value * 8;
-            uint4 val[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {    // eight reads in flight together
+            // eight reads in flight together, then the eight stores (named values: an array here ends up in scratch)
+            auto rd = [&](int u) {
                 const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
-                val[u] = *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
+                return *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
+            };
+            const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3), val4 = rd(4), val5 = rd(5), val6 = rd(6),
+                        val7 = rd(7);
+            auto st = [&](int u, const uint4& v) {
                 const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
                 const int pc = lane % kChunksPerRow;
                 const int grow = row0 + wr * 128 + i * 32 + pr;
                 const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
-                if (grow < NR && gcol < NC) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = val[u];
-            }
+                if (grow < NR && gcol < NC) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
+            };
+            st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
         });
-        __builtin_amdgcn_s_waitcnt(0xC07F);    // patch reads done before the next block overwrites it
+        // keep the blocks apart: hoisting the next blocks' accumulator reads up here runs out of registers
+        __builtin_amdgcn_sched_barrier(0);
     });
 }
 
