@@ -488,8 +488,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         }
     }
 #endif
-    wait_vmcnt<0>();
-    __syncthreads();    // LDS is reused below
+    // No barrier here: the last LDS reads of every wave were issued (and awaited) before the barrier of the last
+    // slice, and no load is in flight, so each wave may start on its patch as soon as its own MFMAs are done.
 
     // ---- epilogue: per 32-row block, accumulators -> this wave's LDS patch -> 16-byte row stores
     constexpr int kEsz = static_cast<int>(sizeof(OT));
@@ -556,8 +556,6 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
             };
             st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
         });
-        // keep the blocks apart: hoisting the next blocks' accumulator reads up here runs out of registers
-        __builtin_amdgcn_sched_barrier(0);
     });
 }
 
