@@ -163,14 +163,12 @@ __device__ __forceinline__ void prepare(float w_raw, float g_raw, float m_old, f
     float gj = g_raw * g_si;
     if (k.maximize) gj = -gj;
     g_plain = gj;
-    if (k.use_decay) {
-        if (k.adam_mode) {
-            const float t = k.wd * pj;
-            gj = gj + t;
-        } else {
-            pj = pj * k.decay;
-        }
-    }
+    // both decay forms are evaluated and one is selected: branches here, once per element of a fully
+    // unrolled step, cost far more registers than the two spare multiplies cost time
+    const float t = k.wd * pj;
+    const float g_l2 = gj + t, p_dec = pj * k.decay;
+    gj = (k.use_decay && k.adam_mode) ? g_l2 : gj;
+    pj = (k.use_decay && !k.adam_mode) ? p_dec : pj;
     moments(m_old, v_old, gj, inv_m, inv_v, k, m_new, v_new);
 }
 
@@ -197,6 +195,33 @@ __device__ __forceinline__ void load16(const msamp_adamw_tensor& d, size_t i, fl
     load_w16<MSAMP_DT_F16>(d.exp_avg_sq, i, v);
 }
 
+// One lane's 16 elements of the first pass (p, g, m, v hold the dequantized stored values on entry).
+__device__ __forceinline__ void amax_step(float* p, const float* g, float* m, float* v, float w_si, float g_si, float inv_m,
+                                          float inv_v, const AdamConsts& k, float& floor_p, uint32_t& mxp, float& mxm,
+                                          float& mxv) {
+    float hi[kEPT];
+    float lo_max = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kEPT; ++j) {
+        float pj, g_plain, m_new, v_new, p_est, err;
+        prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+        estimate(pj, m_new, v_new, k, p_est, err);
+        mxm = fmaxf(mxm, fabsf(m_new));
+        mxv = fmaxf(mxv, fabsf(v_new));
+        p[j] = pj, m[j] = m_new, v[j] = v_new;
+        hi[j] = fabsf(p_est) + err;
+        lo_max = fmaxf(lo_max, fabsf(p_est) - err);    // NaN estimates are skipped here, caught below
+    }
+    floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
+#pragma unroll
+    for (int j = 0; j < kEPT; ++j) {
+        if (!(hi[j] < floor_p)) {
+            const uint32_t ab = __float_as_uint(param_update(p[j], m[j], v[j], k)) & 0x7fffffffu;
+            mxp = ab > mxp ? ab : mxp;
+        }
+    }
+}
+
 // First pass: exact max |m'| and |v'| (they are cheap), and the exact max |p'| found by bounding:
 // every element gets the cheap estimate; only elements whose upper bound reaches the best lower bound
 // seen so far (by this wavefront, or already published for the tensor) are evaluated exactly.  The
@@ -221,28 +246,9 @@ __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_te
 #pragma unroll 1
         for (int s = 0; s < kSteps; ++s) {
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
-            float p[kEPT], g[kEPT], m[kEPT], v[kEPT], hi[kEPT];
+            float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            float lo_max = 0.0f;
-#pragma unroll
-            for (int j = 0; j < kEPT; ++j) {
-                float pj, g_plain, m_new, v_new, p_est, err;
-                prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
-                estimate(pj, m_new, v_new, k, p_est, err);
-                mxm = fmaxf(mxm, fabsf(m_new));
-                mxv = fmaxf(mxv, fabsf(v_new));
-                p[j] = pj, m[j] = m_new, v[j] = v_new;
-                hi[j] = fabsf(p_est) + err;
-                lo_max = fmaxf(lo_max, fabsf(p_est) - err);    // NaN estimates are skipped here, caught below
-            }
-            floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
-#pragma unroll
-            for (int j = 0; j < kEPT; ++j) {
-                if (!(hi[j] < floor_p)) {
-                    const uint32_t ab = __float_as_uint(param_update(p[j], m[j], v[j], k)) & 0x7fffffffu;
-                    mxp = ab > mxp ? ab : mxp;
-                }
-            }
+            amax_step(p, g, m, v, w_si, g_si, inv_m, inv_v, k, floor_p, mxp, mxm, mxv);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
@@ -327,6 +333,50 @@ __device__ __forceinline__ uint32_t quant_weight_exact(float pj, float m_new, fl
     }
 }
 
+// One lane's 16 elements of the second pass: requantized weight, exp_avg and exp_avg_sq are stored at element i.
+template <int WDT>
+__device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i, float* p, const float* g, float* m,
+                                           float* v, float w_si, float g_si, float inv_m, float inv_v, float ws, float ms,
+                                           float vs, bool raw_moments, const AdamConsts& k) {
+    uint32_t wq[kEPT];
+#pragma unroll
+    for (int j = 0; j < kEPT; ++j) {
+        float pj, g_plain, m_new, v_new, p_est, err;
+        prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+        estimate(pj, m_new, v_new, k, p_est, err);
+        const float lo = (p_est - err) * ws, hi = (p_est + err) * ws;
+        bool same;
+        uint32_t code;
+        if constexpr (WDT == MSAMP_DT_F16) {
+            code = float_to_f16_bits(lo);
+            same = code == float_to_f16_bits(hi);
+        } else {
+            const uint32_t two = cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(hi), 0u, false);
+            code = two & 0xffu;
+            same = code == ((two >> 8) & 0xffu);
+        }
+        if (!(same && err < __uint_as_float(0x7f800000u))) code = quant_weight_exact<WDT>(pj, m_new, v_new, ws, k);
+        wq[j] = code;
+        if (raw_moments) moments(m[j], v[j], g_plain, inv_m, inv_v, k, m_new, v_new);
+        m[j] = m_new * ms;
+        v[j] = v_new * vs;
+    }
+    if constexpr (WDT == MSAMP_DT_F16) {
+        uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(d.weight) + i);
+        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
+        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
+    } else {
+        uint4 o;
+        o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
+        o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
+        o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
+        o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(d.weight) + i) = o;
+    }
+    store_w16<MSAMP_DT_E4M3>(d.exp_avg, i, m);
+    store_w16<MSAMP_DT_F16>(d.exp_avg_sq, i, v);
+}
+
 // Second pass: recompute m', v' exactly and requantize them; for the weight, quantize both ends of the
 // estimate's error interval -- when they give the same code (rounding is monotonic) that code is the
 // exact answer, otherwise (or for anything non-finite) the element takes the exact chain.
@@ -348,43 +398,7 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            uint32_t wq[kEPT];
-#pragma unroll
-            for (int j = 0; j < kEPT; ++j) {
-                float pj, g_plain, m_new, v_new, p_est, err;
-                prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
-                estimate(pj, m_new, v_new, k, p_est, err);
-                const float lo = (p_est - err) * ws, hi = (p_est + err) * ws;
-                bool same;
-                uint32_t code;
-                if constexpr (WDT == MSAMP_DT_F16) {
-                    code = float_to_f16_bits(lo);
-                    same = code == float_to_f16_bits(hi);
-                } else {
-                    const uint32_t two = cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(hi), 0u, false);
-                    code = two & 0xffu;
-                    same = code == ((two >> 8) & 0xffu);
-                }
-                if (!(same && err < __uint_as_float(0x7f800000u))) code = quant_weight_exact<WDT>(pj, m_new, v_new, ws, k);
-                wq[j] = code;
-                if (raw_moments) moments(m[j], v[j], g_plain, inv_m, inv_v, k, m_new, v_new);
-                m[j] = m_new * ms;
-                v[j] = v_new * vs;
-            }
-            if constexpr (WDT == MSAMP_DT_F16) {
-                uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(d.weight) + i);
-                o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
-                o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
-            } else {
-                uint4 o;
-                o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
-                o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
-                o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
-                o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-                *reinterpret_cast<uint4*>(static_cast<uint8_t*>(d.weight) + i) = o;
-            }
-            store_w16<MSAMP_DT_E4M3>(d.exp_avg, i, m);
-            store_w16<MSAMP_DT_F16>(d.exp_avg_sq, i, v);
+            write_step<WDT>(d, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, raw_moments, k);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {

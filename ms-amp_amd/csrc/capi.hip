@@ -1,6 +1,10 @@
 // Library-wide pieces of the C ABI: version and the thread-local error string.
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
+
+#include <atomic>
+#include <mutex>
 
 #include "common.cuh"
 
@@ -18,6 +22,43 @@ void set_error(const char* fmt, ...) {
 int hip_fail(hipError_t e, const char* what) {
     set_error("%s: %s", what, hipGetErrorString(e));
     return MSAMP_ERR_HIP - static_cast<int>(e);
+}
+
+// ---- kernels whose workgroups wait for each other ---------------------------------------------
+// Two such kernels half-resident on one chip could wait for each other forever, so they are kept to
+// one stream per device (the first that asks), out of stream capture (a replay would reuse the
+// token), and can be switched off altogether with MSAMP_INTIME_MODE=0 in the environment.
+static std::atomic<uint32_t> g_token{0};
+static std::mutex g_owner_mutex;
+static hipStream_t g_owner_stream[64];
+static bool g_owner_set[64];
+static int g_waiting_kernels = -1;
+
+bool waiting_kernels_allowed(hipStream_t st) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    {
+        std::lock_guard<std::mutex> lock(g_owner_mutex);
+        if (g_waiting_kernels < 0) {
+            const char* e = getenv("MSAMP_INTIME_MODE");
+            g_waiting_kernels = e ? (atoi(e) != 0) : 1;
+        }
+        if (!g_waiting_kernels) return false;
+        if (!g_owner_set[dev]) {
+            g_owner_set[dev] = true;
+            g_owner_stream[dev] = st;
+        }
+        if (g_owner_stream[dev] != st) return false;
+    }
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(st, &capture) == hipSuccess && capture == hipStreamCaptureStatusNone;
+}
+
+uint32_t next_tokens(uint32_t count) {
+    for (;;) {
+        const uint32_t first = g_token.fetch_add(count) + 1;
+        if (first != 0 && first + count - 1 >= first) return first;    // skip 0 and a range that wraps
+    }
 }
 
 }    // namespace msamp

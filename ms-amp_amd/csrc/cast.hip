@@ -950,26 +950,6 @@ static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const flo
     return MSAMP_ERR_DTYPE;
 }
 
-// One-pass (register-resident) in-time cast; returns 1 if it does not apply and the two-pass path must run.
-// Its workgroups wait for each other, so two such kernels must never share the chip half-resident:
-// the first stream to use it on a device keeps it, other streams take the two-pass path.
-static int g_intime_mode = -1;    // MSAMP_INTIME_MODE=0 in the environment: two-pass only
-static std::atomic<uint32_t> g_token{0};
-static std::mutex g_owner_mutex;
-static hipStream_t g_owner_stream[64];
-static bool g_owner_set[64];
-
-static bool owns_resident_kernel(hipStream_t st) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-    std::lock_guard<std::mutex> lock(g_owner_mutex);
-    if (!g_owner_set[dev]) {
-        g_owner_set[dev] = true;
-        g_owner_stream[dev] = st;
-    }
-    return g_owner_stream[dev] == st;
-}
-
 // true if the runtime confirms kResBlocksPerCu workgroups of this kernel fit one CU (asked once per kernel)
 static bool fits_resident(const void* fn) {
     static std::mutex mu;
@@ -989,32 +969,25 @@ static bool fits_resident(const void* fn) {
     return ok;
 }
 
+// One-pass (register-resident) in-time cast; returns 1 if it does not apply and the two-pass path must run.
 template <typename IT>
 static int launch_resident(const IT* x, size_t n, float* scale, float* amax, float* scale_inv, uint8_t* out,
                            int fp8_type, int margin, int flags, void* ws, hipStream_t st) {
     constexpr int EPT = 16 / sizeof(IT);
-    if (g_intime_mode < 0) {
-        const char* e = getenv("MSAMP_INTIME_MODE");
-        g_intime_mode = e ? atoi(e) : 1;
-    }
-    if (g_intime_mode == 0 || (flags & MSAMP_FLAG_TWO_PASS)) return 1;
+    if (flags & MSAMP_FLAG_TWO_PASS) return 1;
     if (!aligned(x, 16) || !aligned(out, EPT)) return 1;
     const size_t nvec = n / EPT;
     size_t max_blocks = static_cast<size_t>(cu_count()) * kResBlocksPerCu;
     if (max_blocks > static_cast<size_t>(kMaxSlots)) max_blocks = kMaxSlots;
     if (nvec == 0 || nvec > max_blocks * kResThreads * kResVecs) return 1;
-    if (!owns_resident_kernel(st)) return 1;
-    // a captured launch would replay this call's token, and the slots of the previous replay still carry it
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone) return 1;
+    if (!waiting_kernels_allowed(st)) return 1;
     if (!fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E4M3, kResVecs>))) return 1;
     // as many workgroups as there are runs of kResThreads vectors, up to the resident limit
     size_t g = (nvec + kResThreads - 1) / kResThreads;
     g = g > max_blocks ? max_blocks : g;
     int rounds = static_cast<int>((nvec + g * kResThreads - 1) / (g * kResThreads));
     g = (nvec + static_cast<size_t>(rounds) * kResThreads - 1) / (static_cast<size_t>(rounds) * kResThreads);
-    uint32_t token = ++g_token;
-    if (token == 0) token = ++g_token;
+    const uint32_t token = next_tokens(1);
     uint64_t* slots = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + kWsSlotBytes);
     const float fp_max = fp8_max(fp8_type);
     const uint32_t spin_limit = 1u << 20;    // a fraction of a second of polling

@@ -16,6 +16,10 @@ constexpr int kWave = 64;
 // ---- error reporting -------------------------------------------------------------------------
 void set_error(const char* fmt, ...);
 int hip_fail(hipError_t e, const char* what);
+// true if a kernel whose workgroups wait for each other may be launched on this stream now
+bool waiting_kernels_allowed(hipStream_t st);
+// `count` consecutive non-zero tokens, unique in this process
+uint32_t next_tokens(uint32_t count);
 
 #define MSAMP_REQUIRE(cond, code, ...)  \
     do {                                \
