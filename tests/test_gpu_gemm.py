@@ -202,3 +202,52 @@ def test_config2_fp8linear_shapes_sampled(be):
     assert rel_fro(dw[r2.cuda()][:, cols.cuda()], want) < TOL_F32
     dw2 = _run(be, xt, 5, 2 * xs, dyt, 6, dys, out_dtype=torch.float32)
     assert torch.equal(dw2, 2 * dw)
+
+
+def _gpu_codes(shape, fp8_dt, seed):
+    """Random finite FP8 payload made on the GPU (magnitude codes below the top binade, random sign)."""
+    g = torch.Generator(device='cuda').manual_seed(seed)
+    top = 0x70 if fp8_dt == 5 else 0x74
+    mag = torch.randint(0, top, shape, generator=g, device='cuda', dtype=torch.uint8)
+    sign = torch.randint(0, 2, shape, generator=g, device='cuda', dtype=torch.uint8) << 7
+    return mag | sign
+
+
+@pytest.mark.parametrize('tokens,d_out,d_in', [(16384, 11008, 4096), (16384, 4096, 11008), (16384, 12288, 4096),
+                                               (16384, 8192, 28672), (16384, 10240, 8192)])
+def test_llama_layer_shapes_sampled(be, tokens, d_out, d_in):
+    """Forward, dgrad and wgrad of the Llama-7B / 70B projection shapes (K up to 28672), operands handed over the way
+    the layer holds them (dgrad and wgrad read K-major operands in place).  Sampled rows and columns against the
+    oracle; exact linearity in the output factor over the whole matrix."""
+    x = _gpu_codes((tokens, d_in), 5, 1)
+    w = _gpu_codes((d_out, d_in), 5, 2)
+    dy = _gpu_codes((tokens, d_out), 6, 3)
+    xs, ws, dys = 2.0**-7, 2.0**-9, 2.0**-14
+    one = lambda v: torch.tensor(v, device='cuda')
+    rows = torch.tensor([0, 255, 256, 8191, tokens - 1])
+    cols = torch.tensor([0, 31, 257, d_out - 1])
+    cin = torch.tensor([0, 129, 4000, d_in - 1])
+    cpu = lambda t, idx, dim=0: t.index_select(dim, idx.cuda()).cpu()
+    # forward y[tokens, d_out] = x W^T
+    y = torch.empty(tokens, d_out, dtype=torch.bfloat16, device='cuda')
+    be.fp8_gemm(w, 5, one(ws), x, 5, one(xs), y)
+    want = ogemm.fp8_gemm(cpu(w, cols), torch.tensor(ws), fp8.E4M3, cpu(x, rows), torch.tensor(xs), fp8.E4M3)
+    assert rel_fro(y[rows.cuda()][:, cols.cuda()].float(), want) < TOL_16
+    y2 = torch.empty_like(y)
+    be.fp8_gemm(w, 5, one(2 * ws), x, 5, one(xs), y2)
+    assert torch.equal(y2, 2 * y)
+    del y, y2
+    # dgrad dx[tokens, d_in] = dy W: a = W^T, handed over as W (K-major)
+    assert be.gemm_kmajor_supported(d_in, tokens, d_out, True, False)
+    dx = torch.empty(tokens, d_in, dtype=torch.bfloat16, device='cuda')
+    be.fp8_gemm(w, 5, one(ws), dy, 6, one(dys), dx, a_kmajor=True)
+    want = ogemm.fp8_gemm(cpu(w, cin, 1).t().contiguous(), torch.tensor(ws), fp8.E4M3, cpu(dy, rows), torch.tensor(dys), fp8.E5M2)
+    assert rel_fro(dx[rows.cuda()][:, cin.cuda()].float(), want) < TOL_16
+    del dx
+    # wgrad dW[d_out, d_in] = dy^T x: a = x^T, b = dy^T, handed over as x and dy (both K-major)
+    assert be.gemm_kmajor_supported(d_in, d_out, tokens, True, True)
+    dw = torch.empty(d_out, d_in, dtype=torch.float32, device='cuda')
+    be.fp8_gemm(x, 5, one(xs), dy, 6, one(dys), dw, a_kmajor=True, b_kmajor=True)
+    want = ogemm.fp8_gemm(cpu(x, cin, 1).t().contiguous(), torch.tensor(xs), fp8.E4M3, cpu(dy, cols, 1).t().contiguous(),
+                          torch.tensor(dys), fp8.E5M2)
+    assert rel_fro(dw[cols.cuda()][:, cin.cuda()], want) < TOL_F32
