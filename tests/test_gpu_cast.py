@@ -108,6 +108,41 @@ def test_config1_in_time_cast_full_size(be, fp8_dt):
     assert torch.equal(q, q2) and am2[0].item() == am[0].item()
 
 
+def test_config5_weight_cast_full_size(be):
+    """In-time cast of one Llama-70B MLP weight, bf16 [28672, 8192] = 234 881 024 elements drawn N(0, 0.01) with
+    0.01 % of them multiplied by 50.  The oracle checks a slice; the whole tensor is checked through properties that do
+    not depend on its size: the amax is the maximum, the scale follows the rule, dequantizing and casting again with
+    the same scale gives the same bytes, and no code exceeds the code of the largest element."""
+    rows, cols = 28672, 8192
+    g = torch.Generator(device='cuda').manual_seed(5)
+    x = torch.randn(rows, cols, generator=g, device='cuda') * 0.01
+    n = x.numel()
+    idx = torch.randint(0, n, (n // 10000, ), generator=g, device='cuda')
+    x.view(-1)[idx] *= 50
+    x = x.bfloat16()
+    for fp8_dt in (5, 6):
+        s, si, am = make_meta()
+        q = be.cast_to_fp8_intime(x, s, am[0:1], si, fp8_dt)
+        assert am[0].item() == x.abs().max().item()
+        fp_max = 448.0 if fp8_dt == 5 else 57344.0
+        assert same_float(s.cpu(), scaling.compute_scaling_factor(am[0].cpu(), torch.tensor(1.0), fp_max, 0))
+        assert same_float(si.cpu(), 1.0 / s.cpu())
+        # a slice against the oracle, quantized with the tensor's scale
+        part = slice(1234567, 1234567 + (1 << 20))
+        om = oracle_meta()
+        om['scale'].copy_(s.cpu())
+        want = ocast.cast_to_fp8(x.view(-1)[part].cpu(), om, FMT[fp8_dt], in_time=False)
+        assert torch.equal(q.view(-1)[part].cpu(), want)
+        # idempotence: dequantize, cast with the same (stored) scale -> same bytes
+        back = be.cast_from_fp8(q, si, fp8_dt, torch.float32)
+        s2, si2, am2 = make_meta()
+        s2.copy_(s)
+        q2 = be.cast_to_fp8(back, s2, am2[0:1], si2, fp8_dt)
+        assert torch.equal(q, q2)
+        assert (q & 0x7F).max().item() == (q.view(-1)[x.view(-1).abs().argmax()] & 0x7F).item()
+        del back, q2
+
+
 @pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('n', [1, 3, 1000, 4097, 16384 * 3 + 5, 1 << 20])
 def test_in_time_cast_ragged_sizes(be, dtype, n):
