@@ -167,6 +167,25 @@ def test_fused_step_grouping_does_not_change_results(be):
             assert all(torch.equal(x, y) for x, y in zip(a['wm'] + a['mm'] + a['vm'], b['wm'] + b['mm'] + b['vm']))
 
 
+def test_config3_full_size_every_tensor_matches(be):
+    """1.0e9 parameters as 238 tensors of [4096, 1024] and a tail of 1 755 648 elements, one fused step.  Every full
+    tensor holds the same bytes, so all of them must come out identical to the first, which is checked against the
+    oracle; the tail (a prefix of the same bytes, its own metas) is checked against the oracle too."""
+    per, total = 4096 * 1024, 1_000_000_000
+    n_full, tail = total // per, total % per
+    base = _inputs(per, 77, fp8.E4M3, fp8.E5M2)
+    last = {k: (v[:tail].clone() if isinstance(v, torch.Tensor) else {kk: vv.clone() for kk, vv in v.items()})
+            for k, v in base.items()}
+    tensors = [base] * n_full + [last]
+    dev = _fused(be, tensors, 5, 6, 2)
+    _check(dev[0], base, fp8.E4M3, fp8.E5M2, 2)
+    _check(dev[-1], last, fp8.E4M3, fp8.E5M2, 2)
+    first = dev[0]
+    for d in dev[1:n_full]:
+        assert torch.equal(d['w'], first['w']) and torch.equal(d['m'], first['m']) and torch.equal(d['v'], first['v'])
+        assert all(torch.equal(x, y) for x, y in zip(d['wm'] + d['mm'] + d['vm'], first['wm'] + first['mm'] + first['vm']))
+
+
 def test_fused_step_is_deterministic(be):
     t = _inputs(16384 * 9, 21, fp8.E4M3, fp8.E5M2)
     a = _fused(be, [t], 5, 6, 2)[0]
