@@ -4,12 +4,16 @@
 // multiply-adds, so the second pass reproduces the first one bit for bit.
 #include "common.cuh"
 
+#include <cmath>
+#include <limits>
+
 namespace msamp {
 
 constexpr int kAdamThreads = 256;
 
 struct AdamConsts {
     float beta1, beta2, omb1, omb2, eps, step_size, sbc2, inv_sbc2, decay, wd;
+    float bound_rsq, bound_eps;    // first pass: |update| <= step_size * |m'| * min(bound_rsq * rsq(v'), bound_eps)
     int adam_mode, maximize, use_decay;
 };
 
@@ -154,21 +158,24 @@ __device__ __forceinline__ float load_w1(const void* base, size_t i) {
 
 // ---- element-wise pieces shared by both passes ------------------------------------------------
 // Exact part: dequantized weight (decayed), gradient (negated / with the Adam-mode L2 term) and the
-// new moments, all as the reference evaluates them.
+// new moments, all as the reference evaluates them.  Two uniform choices are folded into factors, which
+// changes no bit: `g_si` arrives negated when the step maximizes (negation commutes with rounding), and
+// `k.decay` is 1 when no decoupled decay applies.  L2 (Adam mode with a non-zero weight decay) is a
+// template parameter: it adds the decay term to the gradient instead.
+template <bool L2>
 __device__ __forceinline__ void prepare(float w_raw, float g_raw, float m_old, float v_old, float w_si, float g_si,
                                         float inv_m, float inv_v, const AdamConsts& k, float& pj, float& g_plain,
                                         float& m_new, float& v_new) {
 #pragma clang fp contract(off)
     pj = w_raw * w_si;
     float gj = g_raw * g_si;
-    if (k.maximize) gj = -gj;
     g_plain = gj;
-    // both decay forms are evaluated and one is selected: branches here, once per element of a fully
-    // unrolled step, cost far more registers than the two spare multiplies cost time
-    const float t = k.wd * pj;
-    const float g_l2 = gj + t, p_dec = pj * k.decay;
-    gj = (k.use_decay && k.adam_mode) ? g_l2 : gj;
-    pj = (k.use_decay && !k.adam_mode) ? p_dec : pj;
+    if constexpr (L2) {
+        const float t = k.wd * pj;
+        gj = gj + t;
+    } else {
+        pj = pj * k.decay;
+    }
     moments(m_old, v_old, gj, inv_m, inv_v, k, m_new, v_new);
 }
 
@@ -196,6 +203,11 @@ __device__ __forceinline__ void load16(const msamp_adamw_tensor& d, size_t i, fl
 }
 
 // One lane's 16 elements of the first pass (p, g, m, v hold the dequantized stored values on entry).
+// Only bounds on |p'| are needed here: |p| - D <= |p'| <= |p| + D with D >= |step * m' / (sqrt(v') / sbc2 + eps)|,
+// and since eps >= 0 the quotient is at most sbc2 / sqrt(v') and at most 1 / eps.  k.bound_rsq and k.bound_eps hold
+// |step| times those two factors, widened by 4e-6 for the roundings of both chains (the exact one has six, the
+// hardware reciprocal square root is good to one ulp).  A NaN or negative v' keeps its NaN through the selection.
+template <bool L2>
 __device__ __forceinline__ void amax_step(float* p, const float* g, float* m, float* v, float w_si, float g_si, float inv_m,
                                           float inv_v, const AdamConsts& k, float& floor_p, uint32_t& mxp, float& mxm,
                                           float& mxv) {
@@ -203,19 +215,23 @@ __device__ __forceinline__ void amax_step(float* p, const float* g, float* m, fl
     float lo_max = 0.0f;
 #pragma unroll
     for (int j = 0; j < kEPT; ++j) {
-        float pj, g_plain, m_new, v_new, p_est, err;
-        prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
-        estimate(pj, m_new, v_new, k, p_est, err);
+        float pj, g_plain, m_new, v_new;
+        prepare<L2>(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+        const float t = k.bound_rsq * __builtin_amdgcn_rsqf(v_new);
+        const float lim = k.bound_eps < t ? k.bound_eps : t;
+        const float dmax = fabsf(m_new) * lim;
         mxm = fmaxf(mxm, fabsf(m_new));
         mxv = fmaxf(mxv, fabsf(v_new));
         p[j] = pj, m[j] = m_new, v[j] = v_new;
-        hi[j] = fabsf(p_est) + err;
-        lo_max = fmaxf(lo_max, fabsf(p_est) - err);    // NaN estimates are skipped here, caught below
+        hi[j] = fabsf(pj) + dmax;
+        lo_max = fmaxf(lo_max, fabsf(pj) - dmax);    // NaN bounds are skipped here, caught below
     }
     floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
+    // the additions above and the last subtraction of the exact chain round once each: leave room for them
+    const float skip_below = floor_p * 0.999999f;
 #pragma unroll
     for (int j = 0; j < kEPT; ++j) {
-        if (!(hi[j] < floor_p)) {
+        if (!(hi[j] < skip_below)) {
             const uint32_t ab = __float_as_uint(param_update(p[j], m[j], v[j], k)) & 0x7fffffffu;
             mxp = ab > mxp ? ab : mxp;
         }
@@ -223,10 +239,10 @@ __device__ __forceinline__ void amax_step(float* p, const float* g, float* m, fl
 }
 
 // First pass: exact max |m'| and |v'| (they are cheap), and the exact max |p'| found by bounding:
-// every element gets the cheap estimate; only elements whose upper bound reaches the best lower bound
+// every element gets cheap bounds; only elements whose upper bound reaches the best lower bound
 // seen so far (by this wavefront, or already published for the tensor) are evaluated exactly.  The
 // element that attains the true maximum always passes that test, so the result is the exact maximum.
-template <int WDT, int GDT>
+template <int WDT, int GDT, bool L2>
 __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_tensor* __restrict__ tensors,
                                                                    const int32_t* __restrict__ block_map,
                                                                    AdamConsts k) {
@@ -235,7 +251,7 @@ __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_te
     msamp_adamw_tensor& d = tensors[t];
     const size_t n = d.numel;
     const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
-    const float w_si = *d.w_scale_inv, g_si = *d.g_scale_inv;
+    const float w_si = *d.w_scale_inv, g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv;
     const float inv_m = 1.0f / *d.m_scale, inv_v = 1.0f / *d.v_scale;
     uint32_t mxp = 0;    // exact |p'| bit patterns of the candidates (NaN patterns compare highest)
     float mxm = 0.0f, mxv = 0.0f;
@@ -248,12 +264,12 @@ __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_te
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            amax_step(p, g, m, v, w_si, g_si, inv_m, inv_v, k, floor_p, mxp, mxm, mxv);
+            amax_step<L2>(p, g, m, v, w_si, g_si, inv_m, inv_v, k, floor_p, mxp, mxm, mxv);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
             float pj, g_plain, m_new, v_new;
-            prepare(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), load_w1<MSAMP_DT_E4M3>(d.exp_avg, i),
+            prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), load_w1<MSAMP_DT_E4M3>(d.exp_avg, i),
                     load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i), w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
             const uint32_t ab = __float_as_uint(param_update(pj, m_new, v_new, k)) & 0x7fffffffu;
             mxp = ab > mxp ? ab : mxp;
@@ -334,15 +350,15 @@ __device__ __forceinline__ uint32_t quant_weight_exact(float pj, float m_new, fl
 }
 
 // One lane's 16 elements of the second pass: requantized weight, exp_avg and exp_avg_sq are stored at element i.
-template <int WDT>
+template <int WDT, bool L2>
 __device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i, float* p, const float* g, float* m,
                                            float* v, float w_si, float g_si, float inv_m, float inv_v, float ws, float ms,
-                                           float vs, bool raw_moments, const AdamConsts& k) {
+                                           float vs, const AdamConsts& k) {
     uint32_t wq[kEPT];
 #pragma unroll
     for (int j = 0; j < kEPT; ++j) {
         float pj, g_plain, m_new, v_new, p_est, err;
-        prepare(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+        prepare<L2>(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
         estimate(pj, m_new, v_new, k, p_est, err);
         const float lo = (p_est - err) * ws, hi = (p_est + err) * ws;
         bool same;
@@ -357,7 +373,7 @@ __device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i
         }
         if (!(same && err < __uint_as_float(0x7f800000u))) code = quant_weight_exact<WDT>(pj, m_new, v_new, ws, k);
         wq[j] = code;
-        if (raw_moments) moments(m[j], v[j], g_plain, inv_m, inv_v, k, m_new, v_new);
+        if constexpr (L2) moments(m[j], v[j], g_plain, inv_m, inv_v, k, m_new, v_new);    // stored moments ignore the L2 term
         m[j] = m_new * ms;
         v[j] = v_new * vs;
     }
@@ -380,7 +396,7 @@ __device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i
 // Second pass: recompute m', v' exactly and requantize them; for the weight, quantize both ends of the
 // estimate's error interval -- when they give the same code (rounding is monotonic) that code is the
 // exact answer, otherwise (or for anything non-finite) the element takes the exact chain.
-template <int WDT, int GDT>
+template <int WDT, int GDT, bool L2>
 __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_tensor* __restrict__ tensors,
                                                                     const int32_t* __restrict__ block_map,
                                                                     AdamConsts k) {
@@ -389,25 +405,24 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
     msamp_adamw_tensor& d = tensors[t];
     const size_t n = d.numel;
     const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
-    const float w_si = d.saved[0], g_si = *d.g_scale_inv, inv_m = d.saved[1], inv_v = d.saved[2];
+    const float w_si = d.saved[0], g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv, inv_m = d.saved[1], inv_v = d.saved[2];
     const float ws = *d.w_scale, ms = *d.m_scale, vs = *d.v_scale;
-    const bool raw_moments = k.use_decay && k.adam_mode;    // stored moments ignore the L2 term (see prepare)
     if (base + MSAMP_ADAMW_CHUNK <= n) {
 #pragma unroll 1
         for (int s = 0; s < kSteps; ++s) {
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            write_step<WDT>(d, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, raw_moments, k);
+            write_step<WDT, L2>(d, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
             const float m_old = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v_old = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
             float pj, g_plain, m_new, v_new;
-            prepare(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
+            prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
                     g_plain, m_new, v_new);
             store_w1<WDT>(d.weight, i, param_update(pj, m_new, v_new, k) * ws);
-            if (raw_moments) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
+            if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
             store_w1<MSAMP_DT_E4M3>(d.exp_avg, i, m_new * ms);
             store_w1<MSAMP_DT_F16>(d.exp_avg_sq, i, v_new * vs);
         }
@@ -507,25 +522,41 @@ int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int3
     k.eps = static_cast<float>(eps);
     host_consts(static_cast<float>(lr), k.beta1, k.beta2, step, bias_correction, &k.step_size, &k.sbc2);
     k.inv_sbc2 = 1.0f / k.sbc2;
-    k.decay = static_cast<float>(1.0 - lr * weight_decay);
     k.wd = static_cast<float>(weight_decay);
     k.adam_mode = adam_mode, k.maximize = maximize, k.use_decay = weight_decay != 0.0;
+    const bool l2 = k.use_decay && adam_mode;    // Adam mode: the decay joins the gradient, the weight is not decayed
+    k.decay = (k.use_decay && !adam_mode) ? static_cast<float>(1.0 - lr * weight_decay) : 1.0f;
+    // factors of the first pass' bound on |update|, rounded up and widened; a negative eps (the bound assumes
+    // eps >= 0) or anything non-finite makes them infinite, and then every element takes the exact chain
+    const float inf = std::numeric_limits<float>::infinity();
+    const double widen = 1.0 + 4e-6, abs_step = fabs(static_cast<double>(k.step_size));
+    k.bound_rsq = k.eps >= 0.0f ? nextafterf(static_cast<float>(abs_step * k.sbc2 * widen), inf) : inf;
+    k.bound_eps = k.eps > 0.0f ? nextafterf(static_cast<float>(abs_step / k.eps * widen), inf) : inf;
+    if (!(k.bound_rsq >= 0.0f)) k.bound_rsq = inf;
+    if (!(k.bound_eps >= 0.0f)) k.bound_eps = inf;
     const float w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
     hipStream_t st = static_cast<hipStream_t>(stream);
+#define FUSED_LAUNCH_WG(KERNEL, NB, BM, W, G)                                                                          \
+    do {                                                                                                              \
+        if (l2)                                                                                                       \
+            hipLaunchKernelGGL((KERNEL<W, G, true>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k);            \
+        else                                                                                                          \
+            hipLaunchKernelGGL((KERNEL<W, G, false>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k);           \
+    } while (0)
 #define FUSED_LAUNCH(KERNEL, NB, BM)                                                                                  \
     do {                                                                                                              \
         if (weight_dtype == MSAMP_DT_E4M3 && grad_dtype == MSAMP_DT_E4M3)                                             \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E4M3, MSAMP_DT_E4M3>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
+            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E4M3, MSAMP_DT_E4M3);                                            \
         else if (weight_dtype == MSAMP_DT_E4M3)                                                                       \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E4M3, MSAMP_DT_E5M2>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
+            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E4M3, MSAMP_DT_E5M2);                                            \
         else if (weight_dtype == MSAMP_DT_E5M2 && grad_dtype == MSAMP_DT_E4M3)                                        \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E5M2, MSAMP_DT_E4M3>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
+            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E5M2, MSAMP_DT_E4M3);                                            \
         else if (weight_dtype == MSAMP_DT_E5M2)                                                                       \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_E5M2, MSAMP_DT_E5M2>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
+            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E5M2, MSAMP_DT_E5M2);                                            \
         else if (grad_dtype == MSAMP_DT_E4M3)                                                                         \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_F16, MSAMP_DT_E4M3>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
+            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_F16, MSAMP_DT_E4M3);                                             \
         else                                                                                                          \
-            hipLaunchKernelGGL((KERNEL<MSAMP_DT_F16, MSAMP_DT_E5M2>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k); \
+            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_F16, MSAMP_DT_E5M2);                                             \
     } while (0)
     // Groups of whole tensors, each small enough that what the first pass read (5 B/param) and what
     // the second writes (4 B/param) stay in the 256 MB Infinity Cache: the second pass then re-reads
@@ -557,6 +588,7 @@ int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int3
         t0 = t1, b0 = b1;
     }
 #undef FUSED_LAUNCH
+#undef FUSED_LAUNCH_WG
     return MSAMP_OK;
 }
 
