@@ -186,6 +186,19 @@ def test_config3_full_size_every_tensor_matches(be):
         assert all(torch.equal(x, y) for x, y in zip(d['wm'] + d['mm'] + d['vm'], first['wm'] + first['mm'] + first['vm']))
 
 
+def test_fused_step_sparse_gradient_and_zero_state(be):
+    """Nine gradients in ten are exactly zero and the moments start at zero: for those elements m' = v' = 0 and the
+    first pass' bound has to come from eps alone (the reciprocal square root of zero is infinite)."""
+    n = 16384 * 5 + 321
+    t = _inputs(n, 91, fp8.E4M3, fp8.E5M2, zero_state=True)
+    g = torch.Generator().manual_seed(92)
+    t['g'][torch.rand(n, generator=g) < 0.9] = 0
+    t['g'][7] = 0x80    # a negative zero as well
+    for step, kw in ((1, dict()), (1, dict(adam_mode=True)), (3, dict(maximize=True))):
+        dev = _fused(be, [t], 5, 6, step, **kw)
+        _check(dev[0], t, fp8.E4M3, fp8.E5M2, step, **kw)
+
+
 def test_fused_step_is_deterministic(be):
     t = _inputs(16384 * 9, 21, fp8.E4M3, fp8.E5M2)
     a = _fused(be, [t], 5, 6, 2)[0]
