@@ -10,6 +10,8 @@
 // workgroups of one XCD (one L2) work on neighbouring tiles.
 #include "common.cuh"
 
+#include <atomic>
+
 #include <type_traits>
 
 namespace msamp {
@@ -563,12 +565,12 @@ template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
 static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                            const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     constexpr int smem = 2 * kDmaStage;
-    static bool configured = false;
+    static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
     auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT>;
-    if (!configured) {
+    if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel)");
-        configured = true;
+        configured.store(true, std::memory_order_release);
     }
     const int tiles = ((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
     hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys,
@@ -581,12 +583,12 @@ template <int BR, int BC, int XF, int YF, typename OT, bool KGUARD>
 static int launch_gemm_k(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                        const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     constexpr int smem = 2 * (BR + BC) * kBK;
-    static bool configured = false;
+    static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
     auto kern = fp8_gemm_kernel<BR, BC, XF, YF, OT, KGUARD>;
-    if (!configured) {
+    if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_kernel)");
-        configured = true;
+        configured.store(true, std::memory_order_release);
     }
     const int tiles = ((NR + BR - 1) / BR) * ((NC + BC - 1) / BC);
     hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys,

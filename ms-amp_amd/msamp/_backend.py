@@ -169,6 +169,13 @@ def cast_to_fp8(x, scale, amax_cell, scale_inv, fp8_dt):
     return out
 
 
+def _shared_device():
+    """True when other kernels may hold part of the GPU for long (a process group with peers keeps RCCL kernels
+    resident beside the compute stream): kernels whose workgroups wait for each other then stay off."""
+    import torch.distributed as dist
+    return dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1
+
+
 def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_inf=False, two_pass=False):
     """amax, scale rule, quantize and reciprocal in one call.  `two_pass` keeps the call off the
     one-pass kernel whose workgroups wait for each other (same results either way)."""
@@ -178,7 +185,8 @@ def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_
     _check(
         lib.msamp_cast_to_fp8_intime(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
-            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass else 0), _ptr(workspace(x.device)),
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _shared_device() else 0),
+            _ptr(workspace(x.device)),
             _stream()
         ), 'msamp_cast_to_fp8_intime'
     )
@@ -194,7 +202,8 @@ def cast_to_fp8_gated(x, scale, amax_cell, scale_inv, fp8_dt, counter, window, m
     _check(
         lib.msamp_cast_to_fp8_gated(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
-            FLAG_NAN_TO_INF if nan_to_inf else 0, _ptr(counter), window, _ptr(workspace(x.device)), _stream()
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _shared_device() else 0), _ptr(counter), window,
+            _ptr(workspace(x.device)), _stream()
         ), 'msamp_cast_to_fp8_gated'
     )
     return out

@@ -213,3 +213,15 @@ def test_adamw_descriptor_layout_matches_header():
     assert 8 * n_ptr + 8 + 12 + 12 + 8 == 8 * _backend.ADAMW_DESC_WORDS
     assert int(re.search(r'#define MSAMP_ADAMW_CHUNK (\d+)', header).group(1)) == _backend.ADAMW_CHUNK
     assert int(re.search(r'#define MSAMP_WORKSPACE_BYTES (\d+)', header).group(1)) == _backend.WORKSPACE_BYTES
+
+
+def test_one_pass_kernels_stay_off_under_a_process_group(monkeypatch):
+    """Kernels whose workgroups wait for each other are only asked for when no other rank exists."""
+    import torch.distributed as dist
+    from msamp import _backend
+    assert _backend._shared_device() is False
+    monkeypatch.setattr(dist, 'is_initialized', lambda: True)
+    monkeypatch.setattr(dist, 'get_world_size', lambda group=None: 2)
+    assert _backend._shared_device() is True
+    monkeypatch.setattr(dist, 'get_world_size', lambda group=None: 1)
+    assert _backend._shared_device() is False
