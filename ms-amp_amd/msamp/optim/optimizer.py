@@ -12,7 +12,7 @@ from torch.optim.optimizer import Optimizer, required
 from msamp import _backend
 from msamp.common.dtype import Floating
 from msamp.common.tensor import ScalingTensor, ScalingMeta
-from msamp.nn import model_state
+from msamp.nn import model_state, ScalingParameter
 
 
 class LBOptimizer(Optimizer):
@@ -28,7 +28,16 @@ class LBOptimizer(Optimizer):
         return rtn
 
     def all_reduce_grads(self, model):
-        """Gradient averaging across data-parallel ranks; a no-op on one GPU."""
+        """Average the ScalingTensor gradients of `model`'s parameters over the data-parallel ranks
+        (optimizer.py:45-51); skipped when the FP8 DDP wrapper reduces them itself."""
+        if model_state.use_fp8_ddp:
+            return
+        grads = [p.grad for p in model.parameters() if isinstance(p, ScalingParameter) and p.grad is not None]
+        self._all_reduce_avg(grads)
+
+    @staticmethod
+    def _all_reduce_avg(grads):
+        """Nothing to do with one rank (tensor_dist.py:118-120); more ranks are outside this single-GPU build."""
         if torch.distributed.is_available() and torch.distributed.is_initialized() \
                 and torch.distributed.get_world_size() > 1:
             raise NotImplementedError('FP8 gradient all-reduce is outside this single-GPU build')
