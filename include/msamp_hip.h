@@ -147,6 +147,23 @@ int msamp_scale_cast(const void* x, int in_dtype, size_t n, const float* scale, 
 int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int32_t* counters, int n, int window, float fp_max,
                        int margin, msamp_stream_t stream);
 
+/* The same for several groups of metas in one launch -- the optimizer updates the `input` and the `ograd`
+ * group (different formats, possibly different windows) once per step (optimizer.py:75-82 loops over them).
+ * `groups` is a HOST array of n_groups <= MSAMP_MAX_SCALE_GROUPS descriptors whose pointers are device
+ * pointers with the meaning they have above. */
+#define MSAMP_MAX_SCALE_GROUPS 4
+typedef struct msamp_scale_group {
+    float* scales;
+    float* amaxs;
+    uint8_t* bad;         /* nullable */
+    int32_t* counters;    /* nullable */
+    int32_t n;
+    int32_t window;
+    float fp_max;
+    int32_t reserved;
+} msamp_scale_group;
+int msamp_scale_update_groups(const msamp_scale_group* groups, int n_groups, int margin, msamp_stream_t stream);
+
 /* tex.te_gemm as Gemm.fp8_gemm calls it (gemm.py:121-144; transa=True, transb=False):
  * D[N][M] = (B[N][K] . A[M][K]^T) * *a_scale_inv * *b_scale_inv (+ bias[M]) (+ D if accumulate).
  * A, B: FP8 bytes, row-major, K contiguous, K % 16 == 0, 16-byte aligned.  d_dtype: F32/F16/BF16.

@@ -827,15 +827,15 @@ __global__ void scaling_factor_kernel(const float* amax, const float* scale_in, 
 __device__ __forceinline__ float nanmax(float a, float b) { return (a != a) ? a : ((b != b) ? b : fmaxf(a, b)); }
 
 // One wavefront per meta (window <= 64): lane j holds amaxs[i][j], so the row is read and written
-// with one load and one store per lane instead of a chain of dependent accesses.
-__global__ __launch_bounds__(256) void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad,
-                                                            int32_t* counters, int n, int window, float fp_max,
-                                                            int margin) {
+// with one load and one store per lane instead of a chain of dependent accesses; the scale and the
+// counter are fetched with the row, not after the reduction.
+__device__ __forceinline__ void scale_update_row(float* scales, float* amaxs, uint8_t* bad, int32_t* counters, int i,
+                                                 int window, float fp_max, int margin) {
     const int lane = threadIdx.x & 63;
-    const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (i >= n) return;
     float* row = amaxs + static_cast<size_t>(i) * window;
     float v = lane < window ? row[lane] : 0.0f;
+    const float old_scale = scales[i];
+    const int32_t old_count = counters != nullptr ? counters[i] : 0;
     const float a0_raw = __shfl(v, 0);
     const bool is_bad = !(fabsf(a0_raw) < __uint_as_float(0x7f800000u));
     const float a0 = is_bad ? 0.0f : a0_raw;
@@ -848,10 +848,29 @@ __global__ __launch_bounds__(256) void scale_update_kernel(float* scales, float*
     const float left = __shfl_up(v, 1);
     if (lane < window) row[lane] = lane == 0 ? 0.0f : left;
     if (lane == 0) {
-        scales[i] = scale_rule(mx, scales[i], fp_max, margin);
+        scales[i] = scale_rule(mx, old_scale, fp_max, margin);
         if (bad != nullptr) bad[i] = is_bad ? 1 : 0;
-        if (counters != nullptr) counters[i] = is_bad ? 0 : counters[i] + 1;
+        if (counters != nullptr) counters[i] = is_bad ? 0 : old_count + 1;
     }
+}
+
+__global__ __launch_bounds__(256) void scale_update_kernel(float* scales, float* amaxs, uint8_t* bad,
+                                                            int32_t* counters, int n, int window, float fp_max,
+                                                            int margin) {
+    const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (i >= n) return;
+    scale_update_row(scales, amaxs, bad, counters, i, window, fp_max, margin);
+}
+
+// several groups of metas (one format and window each) in one launch: blockIdx.y picks the group
+struct ScaleGroups {
+    msamp_scale_group g[MSAMP_MAX_SCALE_GROUPS];
+};
+__global__ __launch_bounds__(256) void scale_update_groups_kernel(ScaleGroups groups, int margin) {
+    const msamp_scale_group& g = groups.g[blockIdx.y];
+    const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (i >= g.n) return;
+    scale_update_row(g.scales, g.amaxs, g.bad, g.counters, i, g.window, g.fp_max, margin);
 }
 
 // any window: one lane per meta
@@ -1424,6 +1443,39 @@ int msamp_scale_update(float* scales, float* amaxs, uint8_t* bad, int32_t* count
                            scales, amaxs, bad, counters, n, window, fp_max, margin);
     }
     MSAMP_CHECK_LAUNCH("scale_update_kernel");
+    return MSAMP_OK;
+}
+
+int msamp_scale_update_groups(const msamp_scale_group* groups, int n_groups, int margin, msamp_stream_t stream) {
+    MSAMP_REQUIRE(n_groups >= 0 && n_groups <= MSAMP_MAX_SCALE_GROUPS, MSAMP_ERR_SHAPE,
+                  "msamp_scale_update_groups: n_groups=%d (at most %d)", n_groups, MSAMP_MAX_SCALE_GROUPS);
+    if (n_groups == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(groups, MSAMP_ERR_NULL, "msamp_scale_update_groups: null pointer");
+    ScaleGroups packed = {};
+    int n_max = 0, used = 0;
+    bool narrow = true;
+    for (int k = 0; k < n_groups; ++k) {
+        const msamp_scale_group& g = groups[k];
+        MSAMP_REQUIRE(g.n >= 0 && g.window >= 1, MSAMP_ERR_SHAPE, "msamp_scale_update_groups: group %d: n=%d window=%d", k,
+                      g.n, g.window);
+        if (g.n == 0) continue;
+        MSAMP_REQUIRE(g.scales && g.amaxs, MSAMP_ERR_NULL, "msamp_scale_update_groups: group %d: null pointer", k);
+        narrow = narrow && g.window <= 64;
+        n_max = g.n > n_max ? g.n : n_max;
+        packed.g[used++] = g;
+    }
+    if (used == 0) return MSAMP_OK;
+    if (!narrow) {    // a window wider than a wavefront: group by group through the single-group entry point
+        for (int k = 0; k < used; ++k) {
+            const msamp_scale_group& g = packed.g[k];
+            const int rc = msamp_scale_update(g.scales, g.amaxs, g.bad, g.counters, g.n, g.window, g.fp_max, margin, stream);
+            if (rc != MSAMP_OK) return rc;
+        }
+        return MSAMP_OK;
+    }
+    hipLaunchKernelGGL(scale_update_groups_kernel, dim3((n_max + 3) / 4, used), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       packed, margin);
+    MSAMP_CHECK_LAUNCH("scale_update_groups_kernel");
     return MSAMP_OK;
 }
 

@@ -46,6 +46,7 @@ _SIGNATURES = {
     'msamp_cast_transpose_gated': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp], _i),
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
@@ -155,6 +156,33 @@ def scale_update(scales, amaxs, fp_max, margin, counters=None, want_mask=True):
         'msamp_scale_update'
     )
     return bad
+
+
+MAX_SCALE_GROUPS = 4
+
+
+class _ScaleGroup(ctypes.Structure):
+    """msamp_scale_group."""
+    _fields_ = [('scales', ctypes.c_void_p), ('amaxs', ctypes.c_void_p), ('bad', ctypes.c_void_p),
+                ('counters', ctypes.c_void_p), ('n', ctypes.c_int32), ('window', ctypes.c_int32),
+                ('fp_max', ctypes.c_float), ('reserved', ctypes.c_int32)]
+
+
+def scale_update_groups(groups, margin):
+    """scale_update for several (scales, amaxs, fp_max, counters) groups in one launch (counters may be None)."""
+    lib = load()
+    for start in range(0, len(groups), MAX_SCALE_GROUPS):
+        part = groups[start:start + MAX_SCALE_GROUPS]
+        table = (_ScaleGroup * len(part))()
+        for row, (scales, amaxs, fp_max, counters) in zip(table, part):
+            _gpu(scales, 'scales')
+            _gpu(amaxs, 'amaxs')
+            if counters is not None:
+                _gpu(counters, 'counters')
+            row.scales, row.amaxs, row.bad, row.counters = _ptr(scales), _ptr(amaxs), None, _ptr(counters)
+            row.n, row.window = amaxs.shape
+            row.fp_max = fp_max
+        _check(lib.msamp_scale_update_groups(table, len(part), margin, _stream()), 'msamp_scale_update_groups')
 
 
 # ---- casts --------------------------------------------------------------------------------------

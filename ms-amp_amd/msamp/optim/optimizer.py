@@ -61,12 +61,19 @@ class LBOptimizer(Optimizer):
             if not ScalingMeta.in_time_scaling:
                 names.append('wgrad')
         margin = 0
+        if all(metas[name]['amax_counters'].is_cuda for name in names):
+            # counters live on the GPU and are updated by the same kernel (no device-to-host copy), and all
+            # groups go in one launch
+            _backend.scale_update_groups(
+                [(metas[n]['scales'], metas[n]['amaxs'], Floating.qfp_max[metas[n]['qtype']], metas[n]['amax_counters'])
+                 for n in names], margin
+            )
+            return
         for name in names:
             meta = metas[name]
             fp_max = Floating.qfp_max[meta['qtype']]
             counters = meta['amax_counters']
             if counters.is_cuda:
-                # counters live on the GPU and are updated by the same kernel: no device-to-host copy
                 _backend.scale_update(meta['scales'], meta['amaxs'], fp_max, margin, counters=counters, want_mask=False)
             else:
                 bad = _backend.scale_update(meta['scales'], meta['amaxs'], fp_max, margin).cpu().bool()

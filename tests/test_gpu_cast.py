@@ -234,6 +234,31 @@ def test_window_update_keeps_device_counters(be):
     assert scales.tolist() == [128.0, 128.0, 4.0]
 
 
+def test_grouped_window_update_matches_group_by_group(be):
+    """Two groups of different format, size and window in one launch against one launch per group; a window wider
+    than a wavefront takes the group-by-group route inside the library."""
+    g = torch.Generator().manual_seed(3)
+    for windows in ((16, 16), (16, 1), (3, 70)):
+        groups = []
+        for n, window, fp_max in ((5, windows[0], 448.0), (9, windows[1], 57344.0)):
+            scales = torch.rand(n, generator=g) + 0.5
+            amaxs = torch.rand(n, window, generator=g) * 100
+            amaxs[1, 0] = float('inf')
+            amaxs[n - 1, 0] = float('nan')
+            counters = torch.randint(0, 20, (n, ), generator=g, dtype=torch.int32)
+            groups.append((scales, amaxs, fp_max, counters))
+        one = [(s.clone().cuda(), a.clone().cuda(), f, c.clone().cuda()) for s, a, f, c in groups]
+        be.scale_update_groups(one, 0)
+        for (s, a, f, c), (s1, a1, _, c1) in zip(groups, one):
+            s2, a2, c2 = s.clone().cuda(), a.clone().cuda(), c.clone().cuda()
+            be.scale_update(s2, a2, f, 0, counters=c2, want_mask=False)
+            assert same_float(s1, s2) and same_float(a1, a2) and torch.equal(c1, c2)
+    be.scale_update_groups([], 0)
+    # more groups than one launch takes: the wrapper splits them, the library itself refuses
+    be.scale_update_groups([(s.clone().cuda(), a.clone().cuda(), f, None) for s, a, f, _ in groups] * 3, 0)
+    assert be.load().msamp_scale_update_groups(None, be.MAX_SCALE_GROUPS + 1, 0, None) == -2
+
+
 def test_delayed_cast_accumulates_amax_and_skips_nan(be):
     g = torch.Generator().manual_seed(5)
     x = torch.randn(100000, generator=g).to(torch.bfloat16)

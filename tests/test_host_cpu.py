@@ -215,6 +215,16 @@ def test_adamw_descriptor_layout_matches_header():
     assert int(re.search(r'#define MSAMP_WORKSPACE_BYTES (\d+)', header).group(1)) == _backend.WORKSPACE_BYTES
 
 
+def test_scale_group_layout_matches_header():
+    import ctypes
+    header = open(os.path.join(ROOT, 'include', 'msamp_hip.h')).read()
+    body = header[header.index('typedef struct msamp_scale_group {'):header.index('} msamp_scale_group;')]
+    fields = re.findall(r'(\w+);', body)
+    assert fields == [name for name, _ in _backend._ScaleGroup._fields_]
+    assert ctypes.sizeof(_backend._ScaleGroup) == 4 * 8 + 4 * 4
+    assert int(re.search(r'#define MSAMP_MAX_SCALE_GROUPS (\d+)', header).group(1)) == _backend.MAX_SCALE_GROUPS
+
+
 def test_one_pass_kernels_stay_off_under_a_process_group(monkeypatch):
     """Kernels whose workgroups wait for each other are only asked for when no other rank exists."""
     import torch.distributed as dist
