@@ -239,7 +239,8 @@ __device__ __noinline__ void store_quad_slow(OT* D, int row, int col, int NR, in
 //  * Two 64 KiB LDS stages.  A slice is computed in two 64-byte sub-steps; the fragments of the next
 //    sub-step are read while the 16 MFMAs of the current one execute (two register buffers).
 //  * One workgroup barrier per slice, between the sub-steps: by then every wave holds the whole slice
-//    in registers, so the stage is refilled right away (X half now, Y half during the next sub-step 0).
+//    in registers, so the stage is refilled right away with the slice after next (all 16 loads during
+//    the second sub-step, which leaves them a whole sub-step to land).
 //  * LDS reads and tile loads are interleaved with the MFMAs one at a time, so that neither the LDS nor
 //    the vector-memory queue backs up and stalls the MFMA stream.
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -363,12 +364,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     const int nk = K / kBK;
     int fa[64], fb[64];    // fragments [X0..X3, Y0..Y3] x 8 registers, two buffers
 
-    // One sub-step: 16 MFMAs on `cur`, 16 fragment-half reads into `nxt`, 8 tile loads.
+    // One sub-step: 16 MFMAs on `cur`, the fragment reads of the next sub-step into `nxt` and, if asked for, the
+    // 16 tile loads of slice ld_kt, one per MFMA.
     // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row l%32, four
     // consecutive D columns per register quad -- the layout the epilogue wants.
-    // EARLY: the loads go out two per MFMA during the first four MFMAs (they are needed soonest).
     auto sub_step = [&](const int* cur, int* nxt, int rd_stage, int rd_ks, bool do_read, int ld_kt, int ld_stage,
-                        int ld_first, bool do_load, int early) {
+                        bool do_load) {
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
 #pragma unroll
@@ -385,18 +386,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
 #pragma unroll
                     for (int p = n * kPieces / 16; p < (n + 1) * kPieces / 16; ++p) read_piece(nxt, rd_stage, rd_ks, p);
                 }
-                if (do_load) {
-                    if (early == 2) {
-                        dma(ld_kt, ld_stage, n);    // the whole slice, one load per MFMA
-                    } else if (early == 1) {
-                        if (n < 4) {
-                            dma(ld_kt, ld_stage, ld_first + 2 * n);
-                            dma(ld_kt, ld_stage, ld_first + 2 * n + 1);
-                        }
-                    } else if (n & 1) {
-                        dma(ld_kt, ld_stage, ld_first + (n >> 1));
-                    }
-                }
+                if (do_load) dma(ld_kt, ld_stage, n);
             }
         }
         static_for<16>([&](auto nc) {
@@ -406,10 +396,6 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         });
     };
 
-#ifndef MSAMP_GEMM_SCHED
-#define MSAMP_GEMM_SCHED 1
-#endif
-#if MSAMP_GEMM_SCHED == 1
     // prologue: slices 0 and 1; wait for slice 0; read its first fragments
 #pragma unroll
     for (int w = 0; w < 16; ++w) dma(0, 0, w);
@@ -430,10 +416,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     for (; kt + 3 < nk; kt += 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            sub_step(fa, fb, u, 1, true, 0, 0, 0, false, 0);
+            sub_step(fa, fb, u, 1, true, 0, 0, false);
             wait_vmcnt<0>();
             __syncthreads();
-            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, 0, true, 2);
+            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, true);
         }
     }
     for (; kt < nk; kt += 2) {
@@ -441,55 +427,13 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         for (int u = 0; u < 2; ++u) {
             const int k1 = kt + u;
             if (k1 < nk) {
-                sub_step(fa, fb, u, 1, true, 0, 0, 0, false, 0);
+                sub_step(fa, fb, u, 1, true, 0, 0, false);
                 wait_vmcnt<0>();
                 __syncthreads();
-                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, 0, k1 + 2 < nk, 2);
+                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, k1 + 2 < nk);
             }
         }
     }
-#else
-    // prologue: slice 0 and the X half of slice 1; wait for slice 0; read its first fragments
-#pragma unroll
-    for (int w = 0; w < 16; ++w) dma(0, 0, w);
-    if (nk > 1) {
-#pragma unroll
-        for (int w = 0; w < 8; ++w) dma(1, 1, w);
-        wait_vmcnt<8>();
-    } else {
-        wait_vmcnt<0>();
-    }
-    __syncthreads();
-#pragma unroll
-    for (int p = 0; p < kPieces; ++p) read_piece(fa, 0, 0, p);
-
-    // slice kt lives in stage kt & 1.  Sub-step 0: MFMAs on its first half, read its second half, send the
-    // Y half of slice kt+1 on its way (its X half went out during the previous sub-step 1).  Barrier: slice
-    // kt+1 has landed for every wave and nobody needs the LDS copy of slice kt any more.  Sub-step 1: MFMAs
-    // on the second half, read the first half of slice kt+1, start refilling this stage with slice kt+2.
-    int kt = 0;
-    for (; kt + 3 < nk; kt += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            sub_step(fa, fb, u, 1, true, kt + u + 1, u ^ 1, 8, true, 1);
-            wait_vmcnt<0>();
-            __syncthreads();
-            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, 0, true, 0);
-        }
-    }
-    for (; kt < nk; kt += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int k1 = kt + u;
-            if (k1 < nk) {
-                sub_step(fa, fb, u, 1, true, k1 + 1, u ^ 1, 8, k1 + 1 < nk, 1);
-                wait_vmcnt<0>();
-                __syncthreads();
-                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, 0, k1 + 2 < nk, 0);
-            }
-        }
-    }
-#endif
     // No barrier here: the last LDS reads of every wave were issued (and awaited) before the barrier of the last
     // slice, and no load is in flight, so each wave may start on its patch as soon as its own MFMAs are done.
 
