@@ -164,6 +164,37 @@ typedef struct msamp_scale_group {
 } msamp_scale_group;
 int msamp_scale_update_groups(const msamp_scale_group* groups, int n_groups, int margin, msamp_stream_t stream);
 
+/* ---- a bucket of gradients into one flat FP8 buffer -------------------------------------------------
+ * The compute steps of the FP8 gradient reducer (nn/distributed.py:143-184) for all tensors of a bucket at
+ * once; the two collectives between and after them are the caller's.  `items` is a DEVICE array of
+ * descriptors (acc is scratch: zero it once, the library leaves it zero), `block_map` a DEVICE array of
+ * n_blocks {item index, chunk index} int32 pairs, chunks of MSAMP_BUCKET_CHUNK elements, every chunk of every
+ * item listed once.  in_dtype: F32/F16/BF16 for all items. */
+#define MSAMP_BUCKET_CHUNK 16384
+typedef struct msamp_bucket_item {
+    const void* src;     /* the gradient, in_dtype                                             */
+    uint8_t* dst;        /* where its FP8 codes go inside the flat buffer                       */
+    float* amax;         /* meta.amax[0]                                                        */
+    float* scale;        /* meta.scale: read as the rule's fallback, then rewritten             */
+    float* scale_inv;    /* meta.scale_inv: rewritten                                           */
+    uint64_t numel;
+    uint32_t acc;        /* scratch                                                             */
+    uint32_t reserved;
+} msamp_bucket_item;
+
+/* amax[0] = max|src| per item, NaN propagating (distributed.py:156: g.abs().max()); with
+ * MSAMP_FLAG_NAN_TO_INF a NaN or +Inf result becomes +Inf (distributed.py:159: the MAX all-reduce that
+ * follows ignores NaN). */
+int msamp_bucket_amax(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype,
+                      int flags, msamp_stream_t stream);
+
+/* scale = rule(amax[0], fallback scale, fp_max, margin) * pre_scale (distributed.py:163-170, pre_scale =
+ * 1/sqrt(world size)), dst = FP8 codes of src * scale (distributed.py:179-185), scale_inv = (1/scale) /
+ * scale_inv_div (distributed.py:186 followed by :192, the division of the finished tensor by the world size;
+ * pass 1 for none).  amax[0] is read as the caller left it (reduced over the ranks or not). */
+int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype,
+                      int fp8_type, float pre_scale, float scale_inv_div, int margin, msamp_stream_t stream);
+
 /* tex.te_gemm as Gemm.fp8_gemm calls it (gemm.py:121-144; transa=True, transb=False):
  * D[N][M] = (B[N][K] . A[M][K]^T) * *a_scale_inv * *b_scale_inv (+ bias[M]) (+ D if accumulate).
  * A, B: FP8 bytes, row-major, K contiguous, K % 16 == 0, 16-byte aligned.  d_dtype: F32/F16/BF16.

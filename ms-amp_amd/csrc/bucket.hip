@@ -1,0 +1,165 @@
+// Quantizing a bucket of high-precision gradients into one flat FP8 buffer, many tensors per launch: the
+// compute steps of the FP8 gradient reducer (msamp/nn/distributed.py:143-184) either side of its amax
+// all-reduce.  One workgroup handles one 16384-element chunk of one tensor; a device table describes the
+// tensors and a block map assigns the chunks, as in the fused AdamW step.
+#include "common.cuh"
+
+namespace msamp {
+
+constexpr int kBucketThreads = 256;
+
+// max |x| of one chunk, as the bit pattern of the float (a NaN pattern compares above every number, so it wins)
+template <typename IT>
+__global__ __launch_bounds__(kBucketThreads) void bucket_amax_kernel(msamp_bucket_item* __restrict__ items,
+                                                                     const int32_t* __restrict__ block_map) {
+    constexpr int EPT = In16<IT>::EPT;
+    constexpr int kVecs = MSAMP_BUCKET_CHUNK / (kBucketThreads * EPT);    // 16 (fp32) or 8 (16-bit)
+    __shared__ uint32_t red[kBucketThreads / kWave];
+    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
+    msamp_bucket_item& d = items[t];
+    const IT* x = static_cast<const IT*>(d.src);
+    const size_t n = d.numel, base = static_cast<size_t>(chunk) * MSAMP_BUCKET_CHUNK;
+    uint32_t m = 0;
+    if (base + MSAMP_BUCKET_CHUNK <= n && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+        float v[kVecs][EPT];
+#pragma unroll
+        for (int u = 0; u < kVecs; ++u) In16<IT>::load(x + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT, v[u]);
+#pragma unroll
+        for (int u = 0; u < kVecs; ++u)
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) {
+                const uint32_t a = __float_as_uint(v[u][j]) & 0x7fffffffu;
+                m = a > m ? a : m;
+            }
+    } else {
+        for (size_t i = base + threadIdx.x; i < n && i < base + MSAMP_BUCKET_CHUNK; i += kBucketThreads) {
+            const uint32_t a = __float_as_uint(Elem<IT>::load(x + i)) & 0x7fffffffu;
+            m = a > m ? a : m;
+        }
+    }
+    m = block_max_u32(m, red);
+    if (threadIdx.x == 0 && m) atomicMax(&d.acc, m);
+}
+
+// amax[0] of every tensor from the accumulated pattern (NaN and +Inf become +Inf when asked: the all-reduce that
+// follows in the reducer ignores NaN); the accumulator goes back to zero
+__global__ void bucket_amax_finish_kernel(msamp_bucket_item* items, int n_items, int flags) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_items) return;
+    msamp_bucket_item& d = items[t];
+    float a = __uint_as_float(d.acc);
+    d.acc = 0u;
+    if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(a < __uint_as_float(0x7f800000u))) a = __uint_as_float(0x7f800000u);
+    *d.amax = a;
+}
+
+// scale = rule(amax[0], fallback = the scale in force) * pre_scale, scale_inv = (1 / scale) / inv_div (the reducer
+// divides the finished ScalingTensor by the world size, which is a division of scale_inv: two roundings, kept)
+__global__ void bucket_scale_kernel(msamp_bucket_item* items, int n_items, float fp_max, int margin, float pre_scale,
+                                    float inv_div) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_items) return;
+    msamp_bucket_item& d = items[t];
+    const float sf = scale_rule(*d.amax, *d.scale, fp_max, margin) * pre_scale;
+    *d.scale = sf;
+    const float inv = 1.0f / sf;
+    *d.scale_inv = inv / inv_div;
+}
+
+template <typename IT, int FMT>
+__global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp_bucket_item* __restrict__ items,
+                                                                     const int32_t* __restrict__ block_map) {
+    constexpr int EPT = In16<IT>::EPT;
+    constexpr int kVecs = MSAMP_BUCKET_CHUNK / (kBucketThreads * EPT);
+    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
+    const msamp_bucket_item& d = items[t];
+    const IT* x = static_cast<const IT*>(d.src);
+    uint8_t* out = d.dst;
+    const float s = *d.scale;
+    const size_t n = d.numel, base = static_cast<size_t>(chunk) * MSAMP_BUCKET_CHUNK;
+    // a tensor's place in the flat buffer follows from the sizes before it: vector stores only where it allows
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & (EPT - 1)) == 0;
+    if (base + MSAMP_BUCKET_CHUNK <= n && vec) {
+        float v[kVecs][EPT];
+#pragma unroll
+        for (int u = 0; u < kVecs; ++u) In16<IT>::load(x + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT, v[u]);
+#pragma unroll
+        for (int u = 0; u < kVecs; ++u) {
+            uint32_t w[EPT / 4];
+#pragma unroll
+            for (int j = 0; j < EPT / 4; ++j)
+                w[j] = quant4<FMT>(v[u][4 * j] * s, v[u][4 * j + 1] * s, v[u][4 * j + 2] * s, v[u][4 * j + 3] * s);
+            uint8_t* o = out + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT;
+            if constexpr (EPT == 4) {
+                *reinterpret_cast<uint32_t*>(o) = w[0];
+            } else {
+                *reinterpret_cast<uint2*>(o) = make_uint2(w[0], w[1]);
+            }
+        }
+    } else {
+        for (size_t i = base + threadIdx.x; i < n && i < base + MSAMP_BUCKET_CHUNK; i += kBucketThreads)
+            out[i] = static_cast<uint8_t>(quant1<FMT>(Elem<IT>::load(x + i) * s));
+    }
+}
+
+static int check_bucket_args(const char* who, const msamp_bucket_item* items, int n_items, const int32_t* block_map,
+                             int n_blocks, int in_dtype) {
+    MSAMP_REQUIRE(n_items >= 0 && n_blocks >= 0, MSAMP_ERR_SHAPE, "%s: n_items=%d n_blocks=%d", who, n_items, n_blocks);
+    MSAMP_REQUIRE(is_hp(in_dtype), MSAMP_ERR_DTYPE, "%s: in_dtype %d", who, in_dtype);
+    MSAMP_REQUIRE(n_items == 0 || items != nullptr, MSAMP_ERR_NULL, "%s: null descriptor table", who);
+    MSAMP_REQUIRE(n_blocks == 0 || block_map != nullptr, MSAMP_ERR_NULL, "%s: null block map", who);
+    return MSAMP_OK;
+}
+
+}    // namespace msamp
+
+using namespace msamp;
+
+extern "C" {
+
+int msamp_bucket_amax(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype, int flags,
+                      msamp_stream_t stream) {
+    const int rc = check_bucket_args("msamp_bucket_amax", items, n_items, block_map, n_blocks, in_dtype);
+    if (rc != MSAMP_OK || n_items == 0) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (n_blocks > 0) {
+        if (in_dtype == MSAMP_DT_F32)
+            hipLaunchKernelGGL(bucket_amax_kernel<float>, dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map);
+        else if (in_dtype == MSAMP_DT_F16)
+            hipLaunchKernelGGL(bucket_amax_kernel<f16_t>, dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map);
+        else
+            hipLaunchKernelGGL(bucket_amax_kernel<bf16_t>, dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map);
+        MSAMP_CHECK_LAUNCH("bucket_amax_kernel");
+    }
+    hipLaunchKernelGGL(bucket_amax_finish_kernel, dim3((n_items + 63) / 64), dim3(64), 0, st, items, n_items, flags);
+    MSAMP_CHECK_LAUNCH("bucket_amax_finish_kernel");
+    return MSAMP_OK;
+}
+
+int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype,
+                      int fp8_type, float pre_scale, float scale_inv_div, int margin, msamp_stream_t stream) {
+    const int rc = check_bucket_args("msamp_bucket_cast", items, n_items, block_map, n_blocks, in_dtype);
+    if (rc != MSAMP_OK) return rc;
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_bucket_cast: fp8_type %d", fp8_type);
+    if (n_items == 0) return MSAMP_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(bucket_scale_kernel, dim3((n_items + 63) / 64), dim3(64), 0, st, items, n_items, fp8_max(fp8_type),
+                       margin, pre_scale, scale_inv_div);
+    MSAMP_CHECK_LAUNCH("bucket_scale_kernel");
+    if (n_blocks == 0) return MSAMP_OK;
+#define BUCKET_CAST(IT)                                                                                                  \
+    do {                                                                                                               \
+        if (fp8_type == MSAMP_DT_E4M3)                                                                                 \
+            hipLaunchKernelGGL((bucket_cast_kernel<IT, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+        else                                                                                                           \
+            hipLaunchKernelGGL((bucket_cast_kernel<IT, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+    } while (0)
+    if (in_dtype == MSAMP_DT_F32) BUCKET_CAST(float);
+    else if (in_dtype == MSAMP_DT_F16) BUCKET_CAST(f16_t);
+    else BUCKET_CAST(bf16_t);
+#undef BUCKET_CAST
+    MSAMP_CHECK_LAUNCH("bucket_cast_kernel");
+    return MSAMP_OK;
+}
+
+}    // extern "C"

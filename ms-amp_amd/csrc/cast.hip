@@ -11,39 +11,6 @@ namespace msamp {
 constexpr int kCastThreads = 256;
 constexpr int kCastUnroll = 4;
 
-template <typename IT>
-struct In16;    // one 16-byte load = EPT elements as float
-template <>
-struct In16<float> {
-    static constexpr int EPT = 4;
-    static __device__ __forceinline__ void decode(const uint4& t, float* v) {
-        v[0] = __uint_as_float(t.x), v[1] = __uint_as_float(t.y), v[2] = __uint_as_float(t.z), v[3] = __uint_as_float(t.w);
-    }
-    static __device__ __forceinline__ void load(const float* p, float* v) { decode(*reinterpret_cast<const uint4*>(p), v); }
-};
-template <>
-struct In16<bf16_t> {
-    static constexpr int EPT = 8;
-    static __device__ __forceinline__ void load(const bf16_t* p, float* v) { decode(*reinterpret_cast<const uint4*>(p), v); }
-    static __device__ __forceinline__ void decode(const uint4& t, float* v) {
-        v[0] = __uint_as_float(t.x << 16), v[1] = __uint_as_float(t.x & 0xffff0000u);
-        v[2] = __uint_as_float(t.y << 16), v[3] = __uint_as_float(t.y & 0xffff0000u);
-        v[4] = __uint_as_float(t.z << 16), v[5] = __uint_as_float(t.z & 0xffff0000u);
-        v[6] = __uint_as_float(t.w << 16), v[7] = __uint_as_float(t.w & 0xffff0000u);
-    }
-};
-template <>
-struct In16<f16_t> {
-    static constexpr int EPT = 8;
-    static __device__ __forceinline__ void load(const f16_t* p, float* v) { decode(*reinterpret_cast<const uint4*>(p), v); }
-    static __device__ __forceinline__ void decode(const uint4& t, float* v) {
-        v[0] = f16_bits_to_float(t.x & 0xffffu), v[1] = f16_bits_to_float(t.x >> 16);
-        v[2] = f16_bits_to_float(t.y & 0xffffu), v[3] = f16_bits_to_float(t.y >> 16);
-        v[4] = f16_bits_to_float(t.z & 0xffffu), v[5] = f16_bits_to_float(t.z >> 16);
-        v[6] = f16_bits_to_float(t.w & 0xffffu), v[7] = f16_bits_to_float(t.w >> 16);
-    }
-};
-
 // issue an atomic max on a non-negative float cell only when it can change the cell
 __device__ __forceinline__ void amax_publish(float* amax, float v) {
     int vb = __float_as_int(v);

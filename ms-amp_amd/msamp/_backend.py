@@ -47,6 +47,8 @@ _SIGNATURES = {
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
+    'msamp_bucket_amax': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
+    'msamp_bucket_cast': ([_vp, _i, _vp, _i, _i, _i, _f, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
@@ -376,6 +378,45 @@ def fp8_gemm(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, out, accumulate=False, 
         ), 'msamp_fp8_gemm'
     )
     return out
+
+
+# ---- gradient buckets -----------------------------------------------------------------------------
+BUCKET_CHUNK = 16384
+BUCKET_ITEM_WORDS = 7    # int64 words per msamp_bucket_item (56 bytes)
+
+
+def bucket_tables(srcs, dsts, amaxs, scales, scale_invs):
+    """Device descriptor table and block map for quantizing `srcs` into `dsts` (views of one flat buffer)."""
+    import numpy as np
+    rows = [(s.data_ptr(), d.data_ptr(), a.data_ptr(), sc.data_ptr(), si.data_ptr(), s.numel(), 0)
+            for s, d, a, sc, si in zip(srcs, dsts, amaxs, scales, scale_invs)]
+    device = srcs[0].device
+    items = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), BUCKET_ITEM_WORDS)).to(device)
+    chunks = [(s.numel() + BUCKET_CHUNK - 1) // BUCKET_CHUNK for s in srcs]
+    item_idx = np.repeat(np.arange(len(srcs), dtype=np.int32), chunks)
+    chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in chunks]) if sum(chunks) else np.zeros(0, np.int32)
+    block_map = torch.from_numpy(np.stack([item_idx, chunk_idx], axis=1).copy()).to(device)
+    return items, block_map
+
+
+def bucket_amax(items, block_map, in_dt, nan_to_inf=True):
+    """amax[0] of every item of the table."""
+    lib = load()
+    _gpu(items, 'descriptor table')
+    _check(
+        lib.msamp_bucket_amax(_ptr(items), items.shape[0], _ptr(block_map), block_map.shape[0], in_dt,
+                              FLAG_NAN_TO_INF if nan_to_inf else 0, _stream()), 'msamp_bucket_amax'
+    )
+
+
+def bucket_cast(items, block_map, in_dt, fp8_dt, pre_scale, scale_inv_div=1.0, margin=0):
+    """scale = rule(amax[0]) * pre_scale, scale_inv = (1/scale) / scale_inv_div, FP8 codes of every item into its place."""
+    lib = load()
+    _gpu(items, 'descriptor table')
+    _check(
+        lib.msamp_bucket_cast(_ptr(items), items.shape[0], _ptr(block_map), block_map.shape[0], in_dt, fp8_dt, pre_scale,
+                              scale_inv_div, margin, _stream()), 'msamp_bucket_cast'
+    )
 
 
 # ---- AdamW --------------------------------------------------------------------------------------

@@ -19,6 +19,11 @@ Pinning status of each function (what fixes its output besides its own formula):
 * ``arithmetic.add_to_fp8``: the identity the reference's test demands
   (tests/operators/test_arithmetic.py:25-42: equal to dequantize, add, in-time cast) and a
   hand-worked case.
+* ``bucket.quantize_bucket``: a composition of the pinned pieces above (amax, scale rule,
+  encode) in the order of msamp/nn/distributed.py:143-184, plus what the composition must
+  satisfy: an exact pre-scale for world sizes that are powers of four, the gradient back
+  to half a code step after dequantizing and multiplying by the world size, and a sum of
+  ``world`` identical buckets that stays inside the format.
 * ``gemm.fp8_gemm``: definition (fp32 matmul of dequantized operands) and the exact
   case of tests/operators/test_gemm.py:45-56.
 * ``adamw.*``: textbook AdamW against ``torch.optim.AdamW`` to the reference's own
