@@ -195,6 +195,21 @@ int msamp_bucket_amax(msamp_bucket_item* items, int n_items, const int32_t* bloc
 int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype,
                       int fp8_type, float pre_scale, float scale_inv_div, int margin, msamp_stream_t stream);
 
+/* Norms of FP8 tensors without dequantizing them to memory: what clip_grad_norm_ computes per gradient
+ * (nn/clip_grad.py:29-41: `g.to(float32)` then `abs().max()` or `torch.norm(g, p)`), for many tensors per launch.
+ * out[i] = |scale_inv| * (sum |q|^p)^(1/p) for norm_kind 1 or 2, |scale_inv| * max|q| for norm_kind 0 (the
+ * infinity norm), accumulated in double and rounded to float once; NaN codes give NaN.  `items`: DEVICE array
+ * (acc is scratch: zero it once); block_map as for the bucket entry points, chunks of MSAMP_BUCKET_CHUNK codes. */
+typedef struct msamp_norm_item {
+    const uint8_t* q;
+    const float* scale_inv;
+    float* out;
+    uint64_t numel;
+    double acc;          /* scratch */
+} msamp_norm_item;
+int msamp_fp8_norms(msamp_norm_item* items, int n_items, const int32_t* block_map, int n_blocks, int fp8_type,
+                    int norm_kind, msamp_stream_t stream);
+
 /* tex.te_gemm as Gemm.fp8_gemm calls it (gemm.py:121-144; transa=True, transb=False):
  * D[N][M] = (B[N][K] . A[M][K]^T) * *a_scale_inv * *b_scale_inv (+ bias[M]) (+ D if accumulate).
  * A, B: FP8 bytes, row-major, K contiguous, K % 16 == 0, 16-byte aligned.  d_dtype: F32/F16/BF16.

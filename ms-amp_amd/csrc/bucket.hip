@@ -102,6 +102,89 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp
     }
 }
 
+// ---- norms of FP8 gradients (clip_grad_norm_) ----------------------------------------------------------------
+// sum |q|^p (p = 1, 2) or max |q| over the codes of each tensor, accumulated in double: the dequantization factor
+// is constant per tensor and is applied once at the end, so a tensor is read at one byte per element and never
+// expanded to float32 in memory.
+template <int FMT, int KIND>    // KIND: 1, 2, or 0 for the maximum
+__global__ __launch_bounds__(kBucketThreads) void fp8_norm_kernel(msamp_norm_item* __restrict__ items,
+                                                                   const int32_t* __restrict__ block_map) {
+    __shared__ double red[kBucketThreads / kWave];
+    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
+    msamp_norm_item& d = items[t];
+    const uint8_t* q = d.q;
+    const size_t n = d.numel, base = static_cast<size_t>(chunk) * MSAMP_BUCKET_CHUNK;
+    double acc = 0.0;
+    auto take = [&](float v) {
+        const double a = fabs(static_cast<double>(v));
+        if constexpr (KIND == 0) {
+            acc = (a != a || acc != acc) ? (a != a ? a : acc) : (a > acc ? a : acc);    // NaN stays
+        } else if constexpr (KIND == 1) {
+            acc += a;
+        } else {
+            acc = fma(a, a, acc);
+        }
+    };
+    if (base + MSAMP_BUCKET_CHUNK <= n && (reinterpret_cast<uintptr_t>(q) & 15) == 0) {
+        constexpr int kVecs = MSAMP_BUCKET_CHUNK / (kBucketThreads * 16);    // 4
+        uint4 w[kVecs];
+#pragma unroll
+        for (int u = 0; u < kVecs; ++u)
+            w[u] = *reinterpret_cast<const uint4*>(q + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * 16);
+#pragma unroll
+        for (int u = 0; u < kVecs; ++u) {
+            const uint32_t words[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float a, b, c, e;
+                dequant4<FMT>(words[j], a, b, c, e);
+                take(a), take(b), take(c), take(e);
+            }
+        }
+    } else {
+        for (size_t i = base + threadIdx.x; i < n && i < base + MSAMP_BUCKET_CHUNK; i += kBucketThreads) take(dequant1<FMT>(q[i]));
+    }
+    // workgroup total (maximum): lanes, then wavefronts
+#pragma unroll
+    for (int o = 32; o; o >>= 1) {
+        const double other = __shfl_xor(acc, o);
+        if constexpr (KIND == 0) {
+            acc = (other != other || acc != acc) ? (other != other ? other : acc) : (other > acc ? other : acc);
+        } else {
+            acc += other;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double total = red[0];
+        for (int w = 1; w < kBucketThreads / kWave; ++w) {
+            if constexpr (KIND == 0) {
+                total = (red[w] != red[w] || total != total) ? (red[w] != red[w] ? red[w] : total) : (red[w] > total ? red[w] : total);
+            } else {
+                total += red[w];
+            }
+        }
+        if constexpr (KIND == 0) {
+            // bit patterns of non-negative doubles order like the values, NaN patterns above all of them
+            atomicMax(reinterpret_cast<unsigned long long*>(&d.acc), static_cast<unsigned long long>(__double_as_longlong(total)));
+        } else {
+            atomicAdd(&d.acc, total);
+        }
+    }
+}
+
+// out[i] = |scale_inv| * acc^(1/p) (the maximum itself for KIND 0), rounded to float once; the accumulator goes back to zero
+__global__ void fp8_norm_finish_kernel(msamp_norm_item* items, int n_items, int kind) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_items) return;
+    msamp_norm_item& d = items[t];
+    const double acc = d.acc;
+    d.acc = 0.0;
+    const double root = kind == 2 ? sqrt(acc) : acc;
+    *d.out = static_cast<float>(fabs(static_cast<double>(*d.scale_inv)) * root);
+}
+
 static int check_bucket_args(const char* who, const msamp_bucket_item* items, int n_items, const int32_t* block_map,
                              int n_blocks, int in_dtype) {
     MSAMP_REQUIRE(n_items >= 0 && n_blocks >= 0, MSAMP_ERR_SHAPE, "%s: n_items=%d n_blocks=%d", who, n_items, n_blocks);
@@ -159,6 +242,34 @@ int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* bloc
     else BUCKET_CAST(bf16_t);
 #undef BUCKET_CAST
     MSAMP_CHECK_LAUNCH("bucket_cast_kernel");
+    return MSAMP_OK;
+}
+
+int msamp_fp8_norms(msamp_norm_item* items, int n_items, const int32_t* block_map, int n_blocks, int fp8_type, int norm_kind,
+                    msamp_stream_t stream) {
+    MSAMP_REQUIRE(n_items >= 0 && n_blocks >= 0, MSAMP_ERR_SHAPE, "msamp_fp8_norms: n_items=%d n_blocks=%d", n_items, n_blocks);
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_fp8_norms: fp8_type %d", fp8_type);
+    MSAMP_REQUIRE(norm_kind >= 0 && norm_kind <= 2, MSAMP_ERR_SHAPE, "msamp_fp8_norms: norm_kind %d (1, 2, or 0 for the maximum)",
+                  norm_kind);
+    if (n_items == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(items != nullptr && (n_blocks == 0 || block_map != nullptr), MSAMP_ERR_NULL, "msamp_fp8_norms: null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (n_blocks > 0) {
+#define NORM_LAUNCH(FMT)                                                                                                \
+    do {                                                                                                              \
+        if (norm_kind == 0)                                                                                           \
+            hipLaunchKernelGGL((fp8_norm_kernel<FMT, 0>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+        else if (norm_kind == 1)                                                                                      \
+            hipLaunchKernelGGL((fp8_norm_kernel<FMT, 1>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+        else                                                                                                          \
+            hipLaunchKernelGGL((fp8_norm_kernel<FMT, 2>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+    } while (0)
+        if (fp8_type == MSAMP_DT_E4M3) NORM_LAUNCH(MSAMP_DT_E4M3); else NORM_LAUNCH(MSAMP_DT_E5M2);
+#undef NORM_LAUNCH
+        MSAMP_CHECK_LAUNCH("fp8_norm_kernel");
+    }
+    hipLaunchKernelGGL(fp8_norm_finish_kernel, dim3((n_items + 63) / 64), dim3(64), 0, st, items, n_items, norm_kind);
+    MSAMP_CHECK_LAUNCH("fp8_norm_finish_kernel");
     return MSAMP_OK;
 }
 

@@ -47,6 +47,7 @@ _SIGNATURES = {
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
+    'msamp_fp8_norms': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
     'msamp_bucket_amax': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
     'msamp_bucket_cast': ([_vp, _i, _vp, _i, _i, _i, _f, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
@@ -417,6 +418,33 @@ def bucket_cast(items, block_map, in_dt, fp8_dt, pre_scale, scale_inv_div=1.0, m
         lib.msamp_bucket_cast(_ptr(items), items.shape[0], _ptr(block_map), block_map.shape[0], in_dt, fp8_dt, pre_scale,
                               scale_inv_div, margin, _stream()), 'msamp_bucket_cast'
     )
+
+
+NORM_ITEM_WORDS = 5    # int64 words per msamp_norm_item (40 bytes)
+
+
+def fp8_norms(values, scale_invs, fp8_dt, norm_type):
+    """Per-tensor p-norms (p = 1, 2 or inf) of FP8 payloads times their scale_inv, as one float32 vector."""
+    import numpy as np
+    kind = {1.0: 1, 2.0: 2, float('inf'): 0}[float(norm_type)]
+    lib = load()
+    device = values[0].device
+    out = torch.empty(len(values), dtype=torch.float32, device=device)
+    rows = [(v.data_ptr(), si.data_ptr(), out.data_ptr() + 4 * i, v.numel(), 0) for i, (v, si) in enumerate(zip(values, scale_invs))]
+    for v in values:
+        _gpu(v, 'fp8 tensor')
+        if not v.is_contiguous():
+            raise ValueError('fp8 tensors must be contiguous')
+    items = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), NORM_ITEM_WORDS)).to(device)
+    chunks = [(v.numel() + BUCKET_CHUNK - 1) // BUCKET_CHUNK for v in values]
+    item_idx = np.repeat(np.arange(len(values), dtype=np.int32), chunks)
+    chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in chunks]) if sum(chunks) else np.zeros(0, np.int32)
+    block_map = torch.from_numpy(np.stack([item_idx, chunk_idx], axis=1).copy()).to(device)
+    _check(
+        lib.msamp_fp8_norms(_ptr(items), len(values), _ptr(block_map), block_map.shape[0], fp8_dt, kind, _stream()),
+        'msamp_fp8_norms'
+    )
+    return out
 
 
 # ---- AdamW --------------------------------------------------------------------------------------

@@ -102,3 +102,65 @@ def test_bucket_sum_of_ranks_is_the_average():
     assert (codes * world).abs().max().item() <= 448.0 * math.sqrt(world)
     avg = t.float().cpu() * world
     assert ((avg - g).abs() <= g.abs() * 2.0 ** -4 + g.abs().max() * 2.0 ** -9).all()
+
+
+@pytest.mark.parametrize('fp8_dt,fmt', [(5, fp8.E4M3), (6, fp8.E5M2)])
+@pytest.mark.parametrize('norm_type', [1.0, 2.0, float('inf')])
+def test_fp8_norms_against_float64(fp8_dt, fmt, norm_type):
+    """Per-tensor norms straight from the codes against a float64 evaluation of the dequantized values (to one
+    float32 rounding), and against what the reference computes (float32 torch.norm of the dequantized tensor)."""
+    from msamp import _backend
+    g = torch.Generator().manual_seed(int(norm_type if norm_type < 10 else 7) + fp8_dt)
+    sizes = [1, 7, 16384, 16384 * 3 + 11, 100000, 4096 * 1024]
+    values, sis = [], []
+    for n in sizes:
+        top = 0x7B if fmt == fp8.E4M3 else 0x7A
+        q = torch.randint(0, top, (n + 1, ), generator=g, dtype=torch.uint8) | (torch.randint(0, 2, (n + 1, ), generator=g, dtype=torch.uint8) << 7)
+        values.append(q[1:] if n % 2 else q[:n])    # odd sizes start one byte off a 16-byte boundary
+        sis.append(torch.tensor(-2.0 ** float(torch.randint(-12, 3, (1, ), generator=g))))
+    got = _backend.fp8_norms([v.cuda() for v in values], [s.cuda() for s in sis], fp8_dt, norm_type).cpu()
+    for k, (v, s) in enumerate(zip(values, sis)):
+        x = fp8.decode(v, fmt).double() * s.double()
+        want = x.abs().max() if norm_type == float('inf') else x.abs().pow(norm_type).sum().pow(1.0 / norm_type)
+        assert got[k].item() == pytest.approx(want.item(), rel=2e-7), (k, norm_type)
+        ref32 = x.float().abs().max() if norm_type == float('inf') else torch.norm(x.float(), norm_type)
+        if v.numel() <= 100000:    # beyond that the CPU's sequential float32 sum is itself off by more than 1e-4
+            assert got[k].item() == pytest.approx(ref32.item(), rel=1e-4)
+
+
+def test_fp8_norms_nan_empty_and_repeat():
+    """A NaN code makes that tensor's norm NaN (as torch.norm would) and only that one; an empty tensor has norm 0;
+    calling twice gives the same numbers (the scratch accumulators are left clean)."""
+    from msamp import _backend
+    a = torch.full((40000, ), 0x38, dtype=torch.uint8)    # 1.0 in E4M3
+    b = a.clone()
+    b[12345] = 0x7F
+    vals = [a.cuda(), b.cuda(), torch.zeros(0, dtype=torch.uint8, device='cuda')]
+    si = [torch.tensor(0.5, device='cuda')] * 3
+    for norm_type, want in ((2.0, 100.0), (1.0, 20000.0), (float('inf'), 0.5)):
+        for _ in range(2):
+            got = _backend.fp8_norms(vals, si, 5, norm_type).cpu()
+            assert got[0].item() == want and math.isnan(got[1].item()) and got[2].item() == 0.0
+
+
+def test_clip_grad_norm_uses_the_codes():
+    """clip_grad_norm_ over FP8 ScalingTensor gradients and a plain bias gradient: the total equals the norm of the
+    dequantized gradients, and clipping multiplies every gradient by the same coefficient (scale_inv only for FP8)."""
+    import msamp
+    from msamp.common.dtype import Dtypes
+    from msamp.nn import LinearReplacer
+    torch.manual_seed(3)
+    model = LinearReplacer.replace(torch.nn.Sequential(torch.nn.Linear(64, 48), torch.nn.Linear(48, 16)).cuda(), Dtypes.kfloat16)
+    model(torch.randn(32, 64, device='cuda')).sum().backward()
+    params = list(model.parameters())
+    for norm_type in (2.0, 1.0, float('inf')):
+        flat = torch.cat([p.grad.float().flatten() for p in params]).double()
+        want = flat.abs().max() if norm_type == float('inf') else flat.abs().pow(norm_type).sum().pow(1 / norm_type)
+        codes = [p.grad.value.clone() for p in params if hasattr(p.grad, 'value')]
+        before = [p.grad.float().clone() for p in params]
+        total = msamp.clip_grad_norm_(params, want.item() / 4, norm_type=norm_type)
+        assert total.item() == pytest.approx(want.item(), rel=1e-5)
+        coef = (want.item() / 4) / (total.item() + 1e-6)
+        for p, old in zip(params, before):
+            assert torch.allclose(p.grad.float(), old * coef, rtol=1e-5, atol=0)
+        assert all(torch.equal(c, p.grad.value) for c, p in zip(codes, [p for p in params if hasattr(p.grad, 'value')]))
