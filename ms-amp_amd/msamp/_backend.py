@@ -112,8 +112,9 @@ def _dt(t):
 
 
 def workspace(device):
-    """Per-device scratch words shared by the two-pass kernels (calls are stream ordered)."""
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    """Scratch words of the two-pass kernels: one buffer per device and stream, since calls that share a buffer
+    must be ordered on one stream (the current stream is the one every entry point is given)."""
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device(), _stream())
     ws = _workspaces.get(key)
     if ws is None:
         ws = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=device)

@@ -192,6 +192,32 @@ def test_in_time_cast_on_a_second_stream(be):
     assert torch.equal(q1, q2) and same_float(am1, am2) and same_float(s1, s2) and same_float(si1, si2)
 
 
+def test_two_pass_casts_on_two_streams_at_once(be):
+    """Two streams each run two-pass in-time casts of different tensors with nothing ordering them: each stream has
+    its own scratch words, so neither sees the other's partial maxima."""
+    g = torch.Generator().manual_seed(4)
+    xa = (torch.randn(6_000_000, generator=g) * 3).cuda()
+    xb = (torch.randn(6_000_000, generator=g) * 0.01).cuda()
+    want = []
+    for x in (xa, xb):
+        s, si, am = make_meta()
+        want.append((be.cast_to_fp8_intime(x, s, am[0:1], si, 5, two_pass=True), s, am))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    got_a, got_b = [], []
+    for _ in range(8):
+        s, si, am = make_meta()
+        got_a.append((be.cast_to_fp8_intime(xa, s, am[0:1], si, 5, two_pass=True), s, am))
+        with torch.cuda.stream(side):
+            s, si, am = make_meta()
+            got_b.append((be.cast_to_fp8_intime(xb, s, am[0:1], si, 5, two_pass=True), s, am))
+    torch.cuda.synchronize()
+    for got, ref in ((got_a, want[0]), (got_b, want[1])):
+        for q, s, am in got:
+            assert torch.equal(q, ref[0]) and same_float(s, ref[1]) and same_float(am, ref[2])
+
+
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize('counter', [0, 3, 4, 100])
 def test_gated_casts_follow_the_device_counter(be, dtype, counter):
