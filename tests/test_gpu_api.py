@@ -384,3 +384,57 @@ def test_grad_scaler_unscale_with_scaling_tensor_grads():
     g.meta.amax[0] = float('inf')
     torch._amp_foreach_non_finite_check_and_unscale_([g], found, torch.tensor(1.0, device='cuda'))
     assert found.item() == 1
+
+
+def test_empty_inputs_are_accepted_everywhere():
+    """Zero elements through every entry point: nothing is written but the meta, which comes out as for a tensor of
+    zeros (amax 0, the scale in force kept, scale_inv = 1 / scale).  The reference raises here (`max()` of an empty
+    tensor); a library must not fault."""
+    from msamp import _backend as be
+    from tests.gpu_util import make_meta
+    dev = 'cuda'
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        x = torch.zeros(0, dtype=dtype, device=dev)
+        for fp8_dt in (5, 6):
+            s, si, am = make_meta(scale=4.0)
+            am[0] = 3.0
+            assert be.cast_to_fp8(x, s, am[0:1], si, fp8_dt).numel() == 0
+            assert am[0].item() == 3.0 and s.item() == 4.0 and si.item() == 0.25
+            for two_pass in (False, True):
+                s, si, am = make_meta(scale=4.0)
+                am[0] = 3.0
+                assert be.cast_to_fp8_intime(x, s, am[0:1], si, fp8_dt, two_pass=two_pass).numel() == 0
+                assert am[0].item() == 0.0 and s.item() == 4.0 and si.item() == 0.25
+            for counter in (0, 99):
+                s, si, am = make_meta(scale=4.0)
+                cnt = torch.full((), counter, dtype=torch.int32, device=dev)
+                assert be.cast_to_fp8_gated(x, s, am[0:1], si, fp8_dt, cnt, 16).numel() == 0
+                assert s.item() == 4.0 and si.item() == 0.25
+            for shape in ((0, 64), (64, 0), (0, 0)):
+                s, si, am = make_meta(scale=4.0)
+                q, qt = be.cast_transpose(x.view(shape), s, am[0:1], si, fp8_dt)
+                assert q.shape == shape and qt.shape == shape[::-1]
+                q, qt = be.cast_transpose(x.view(shape), s, am[0:1], si, fp8_dt, in_time=True)
+                assert q.shape == shape and s.item() == 4.0
+        cell = torch.full((1, ), 7.0, device=dev)
+        be.amax(x, cell)
+        assert cell.item() == 0.0
+        assert be.scale_cast(x, torch.ones((), device=dev), torch.float16).numel() == 0
+    q0 = torch.zeros(0, dtype=torch.uint8, device=dev)
+    assert be.cast_from_fp8(q0, torch.ones((), device=dev), 5, torch.float32).numel() == 0
+    assert be.fp8_transpose(q0.view(0, 16)).shape == (16, 0)
+    s, si, am = make_meta(scale=4.0)
+    be.add_to_fp8(q0, 5, s, si, am[0:1], torch.zeros(0, device=dev))
+    be.scale_update(torch.zeros(0, device=dev), torch.zeros(0, 16, device=dev), 448.0, 0, want_mask=False)
+    # GEMM: no rows or no columns -> nothing to do; no reduction length is an error, as is a ragged one
+    one = torch.ones((), device=dev)
+    a = torch.zeros(0, 32, dtype=torch.uint8, device=dev)
+    b = torch.zeros(8, 32, dtype=torch.uint8, device=dev)
+    be.fp8_gemm(a, 5, one, b, 5, one, torch.empty(8, 0, device=dev))
+    be.fp8_gemm(b, 5, one, a, 5, one, torch.empty(0, 8, device=dev))
+    with pytest.raises(Exception):
+        be.fp8_gemm(torch.zeros(8, 0, dtype=torch.uint8, device=dev), 5, one, torch.zeros(8, 0, dtype=torch.uint8, device=dev), 5, one,
+                    torch.empty(8, 8, device=dev))
+    # fused AdamW: no tensors at all
+    be.adamw_fused(torch.zeros(0, be.ADAMW_DESC_WORDS, dtype=torch.int64, device=dev), 0,
+                   torch.zeros(0, 2, dtype=torch.int32, device=dev), 0, 5, 6, 1e-3, 0.9, 0.95, 1e-8, 0.1, 1, True, False, False, True)
