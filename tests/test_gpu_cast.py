@@ -192,6 +192,33 @@ def test_in_time_cast_on_a_second_stream(be):
     assert torch.equal(q1, q2) and same_float(am1, am2) and same_float(s1, s2) and same_float(si1, si2)
 
 
+def test_casts_beyond_2_31_elements(be):
+    """64-bit indexing: 2^31 + 8 bf16 elements through the in-time cast (two passes at this size), the delayed cast
+    and the dequantization; the maximum sits in the last element, slices at both ends and across the 2^31 mark are
+    compared with the oracle."""
+    n = (1 << 31) + 8
+    x = torch.empty(n, dtype=torch.bfloat16, device='cuda')
+    g = torch.Generator(device='cuda').manual_seed(31)
+    step = 1 << 28
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        x[lo:hi] = torch.randn(hi - lo, generator=g, device='cuda').bfloat16()
+    x[n - 1] = 77.0
+    s, si, am = make_meta()
+    q = be.cast_to_fp8_intime(x, s, am[0:1], si, 5)
+    assert am[0].item() == 77.0 and s.item() == 4.0 and si.item() == 0.25
+    s2, si2, am2 = make_meta(scale=4.0)
+    q2 = be.cast_to_fp8(x, s2, am2[0:1], si2, 5)
+    assert am2[0].item() == 77.0
+    back = be.cast_from_fp8(q, si, 5, torch.bfloat16)
+    for lo, hi in ((0, 4096), ((1 << 31) - 2048, (1 << 31) + 8), (n - 4099, n)):
+        om = oracle_meta(scale=4.0)
+        want = ocast.cast_to_fp8(x[lo:hi].cpu(), om, FMT[5], in_time=False)
+        assert torch.equal(q[lo:hi].cpu(), want) and torch.equal(q2[lo:hi].cpu(), want)
+        assert torch.equal(back[lo:hi].cpu(), ocast.cast_from_fp8(want, torch.tensor(0.25), FMT[5], torch.bfloat16))
+    assert torch.equal(q[1 << 30:(1 << 30) + (1 << 20)], q2[1 << 30:(1 << 30) + (1 << 20)])
+
+
 def test_two_pass_casts_on_two_streams_at_once(be):
     """Two streams each run two-pass in-time casts of different tensors with nothing ordering them: each stream has
     its own scratch words, so neither sees the other's partial maxima."""
