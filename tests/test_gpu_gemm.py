@@ -251,3 +251,17 @@ def test_llama_layer_shapes_sampled(be, tokens, d_out, d_in):
     want = ogemm.fp8_gemm(cpu(x, cin, 1).t().contiguous(), torch.tensor(xs), fp8.E4M3, cpu(dy, cols, 1).t().contiguous(),
                           torch.tensor(dys), fp8.E5M2)
     assert rel_fro(dw[cols.cuda()][:, cin.cuda()], want) < TOL_F32
+
+
+def test_operand_beyond_4_gib(be):
+    """An operand of 70 016 x 65 536 bytes (4.6 GB): its 32-bit byte offsets would wrap, so the library has to route
+    it to the kernel with 64-bit addressing.  Rows below and above the 4 GiB mark against the oracle."""
+    m, n, k = 256, 70016, 65536
+    a = _gpu_codes((m, k), 5, 21)
+    b = _gpu_codes((n, k), 5, 22)
+    one = lambda v: torch.tensor(v, device='cuda')
+    out = torch.empty(n, m, dtype=torch.float32, device='cuda')
+    be.fp8_gemm(a, 5, one(2.0**-8), b, 5, one(2.0**-8), out)
+    rows = torch.tensor([0, 65535, 65536, 65537, n - 1])
+    want = ogemm.fp8_gemm(a.cpu(), torch.tensor(2.0**-8), fp8.E4M3, b[rows.cuda()].cpu(), torch.tensor(2.0**-8), fp8.E4M3)
+    assert rel_fro(out[rows.cuda()], want) < TOL_F32
