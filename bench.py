@@ -163,6 +163,27 @@ def bench_cast(iters=20):
     return out
 
 
+def bench_grad_side(iters=10):
+    """The reducer's compute steps on one bucket of 32 bf16 gradients of [4096,1024] (amax, scales, quantize
+    into the flat E4M3 buffer: 2 B read twice + 1 B written per element), and the per-tensor 2-norms of 64
+    such FP8 gradients (1 B read per element)."""
+    import torch
+    from msamp import _backend
+    from msamp.nn import GradientBucket
+    n = 4096 * 1024
+    grads = [(torch.randn(n, device='cuda') * 1e-3).bfloat16() for _ in range(32)]
+    bucket = GradientBucket([n] * len(grads))
+    out = {}
+    ms = _time_gpu(lambda: bucket.quantize(grads, world_size=8), iters)
+    out['bucket_quantize_32x4M_bf16'] = {'ms': ms, 'GBps': n * len(grads) * 5 / ms / 1e6}
+    del grads, bucket
+    qs = [torch.randint(0, 120, (n,), dtype=torch.uint8, device='cuda') for _ in range(64)]
+    sis = [torch.ones((), device='cuda') for _ in qs]
+    ms = _time_gpu(lambda: _backend.fp8_norms(qs, sis, _backend.DT_E4M3, 2.0), iters)
+    out['fp8_l2_norms_64x4M_e4m3'] = {'ms': ms, 'GBps': n * len(qs) / ms / 1e6}
+    return out
+
+
 def bench_adam(iters=5, total_params=1_000_000_000):
     """Fused FP8 AdamW over 1.0e9 parameters held as [4096,1024] tensors (last one truncated):
     E4M3 weights, E5M2 grads, E4M3 exp_avg, scaled-fp16 exp_avg_sq; step t=2."""
@@ -326,6 +347,8 @@ def main():
         cast = bench_cast()
         adam = bench_adam()
         torch.cuda.empty_cache()
+        grad_side = bench_grad_side()
+        torch.cuda.empty_cache()
         result['cast_amax_GBps'] = cast['c1_intime_fp32_e4m3']['GBps']
         result['fp8_adam_Gparams_per_s'] = adam['Gparams_per_s']
         result['kernels'] = {
@@ -335,6 +358,8 @@ def main():
                             'GBps': round(adam['GBps_algorithmic'], 1),
                             'frac_hbm': round(adam['GBps_algorithmic'] / HBM_PEAK_GBS, 4), 'params': adam['params'],
                             'tensors': adam['tensors']},
+            'grad_side': {k: {'ms': round(v['ms'], 4), 'GBps': round(v['GBps'], 1),
+                              'frac_hbm': round(v['GBps'] / HBM_PEAK_GBS, 4)} for k, v in grad_side.items()},
         }
     if not args.skip_cpu:
         result['cpu_baseline'] = cpu_baseline()

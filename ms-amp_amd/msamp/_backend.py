@@ -387,6 +387,27 @@ BUCKET_CHUNK = 16384
 BUCKET_ITEM_WORDS = 7    # int64 words per msamp_bucket_item (56 bytes)
 
 
+_CHUNK_MAPS = {}
+
+
+def chunk_map(numels, device):
+    """[(item, chunk)] rows, one per workgroup of BUCKET_CHUNK elements, as an int32 device tensor.  The map
+    depends on the sizes only, so the last few are kept per device."""
+    import numpy as np
+    key = (str(device), tuple(int(n) for n in numels))
+    hit = _CHUNK_MAPS.get(key)
+    if hit is not None:
+        return hit
+    chunks = [(n + BUCKET_CHUNK - 1) // BUCKET_CHUNK for n in key[1]]
+    item_idx = np.repeat(np.arange(len(chunks), dtype=np.int32), chunks)
+    chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in chunks]) if sum(chunks) else np.zeros(0, np.int32)
+    block_map = torch.from_numpy(np.stack([item_idx, chunk_idx], axis=1).copy()).to(device)
+    if len(_CHUNK_MAPS) >= 32:
+        _CHUNK_MAPS.pop(next(iter(_CHUNK_MAPS)))
+    _CHUNK_MAPS[key] = block_map
+    return block_map
+
+
 def bucket_tables(srcs, dsts, amaxs, scales, scale_invs):
     """Device descriptor table and block map for quantizing `srcs` into `dsts` (views of one flat buffer)."""
     import numpy as np
@@ -394,11 +415,7 @@ def bucket_tables(srcs, dsts, amaxs, scales, scale_invs):
             for s, d, a, sc, si in zip(srcs, dsts, amaxs, scales, scale_invs)]
     device = srcs[0].device
     items = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), BUCKET_ITEM_WORDS)).to(device)
-    chunks = [(s.numel() + BUCKET_CHUNK - 1) // BUCKET_CHUNK for s in srcs]
-    item_idx = np.repeat(np.arange(len(srcs), dtype=np.int32), chunks)
-    chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in chunks]) if sum(chunks) else np.zeros(0, np.int32)
-    block_map = torch.from_numpy(np.stack([item_idx, chunk_idx], axis=1).copy()).to(device)
-    return items, block_map
+    return items, chunk_map([s.numel() for s in srcs], device)
 
 
 def bucket_amax(items, block_map, in_dt, nan_to_inf=True):
@@ -437,10 +454,7 @@ def fp8_norms(values, scale_invs, fp8_dt, norm_type):
         if not v.is_contiguous():
             raise ValueError('fp8 tensors must be contiguous')
     items = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), NORM_ITEM_WORDS)).to(device)
-    chunks = [(v.numel() + BUCKET_CHUNK - 1) // BUCKET_CHUNK for v in values]
-    item_idx = np.repeat(np.arange(len(values), dtype=np.int32), chunks)
-    chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in chunks]) if sum(chunks) else np.zeros(0, np.int32)
-    block_map = torch.from_numpy(np.stack([item_idx, chunk_idx], axis=1).copy()).to(device)
+    block_map = chunk_map([v.numel() for v in values], device)
     _check(
         lib.msamp_fp8_norms(_ptr(items), len(values), _ptr(block_map), block_map.shape[0], fp8_dt, kind, _stream()),
         'msamp_fp8_norms'

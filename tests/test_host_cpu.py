@@ -235,3 +235,15 @@ def test_one_pass_kernels_stay_off_under_a_process_group(monkeypatch):
     assert _backend._shared_device() is True
     monkeypatch.setattr(dist, 'get_world_size', lambda group=None: 1)
     assert _backend._shared_device() is False
+
+
+def test_chunk_map_rows_and_cache():
+    """One (item, chunk) row per BUCKET_CHUNK elements, ragged tails and empty items included; the same sizes
+    return the same tensor."""
+    from msamp import _backend
+    c = _backend.BUCKET_CHUNK
+    m = _backend.chunk_map([2 * c + 1, 0, c], 'cpu')
+    assert m.dtype == torch.int32
+    assert m.tolist() == [[0, 0], [0, 1], [0, 2], [2, 0]]
+    assert _backend.chunk_map([2 * c + 1, 0, c], 'cpu') is m
+    assert _backend.chunk_map([], 'cpu').shape[0] == 0
