@@ -140,7 +140,18 @@ def bench_cast(iters=20):
     q = _backend.cast_to_fp8_intime(x, s, am[0:1], si, _backend.DT_E4M3)
     ms = _time_gpu(lambda: _backend.cast_from_fp8(q, si, _backend.DT_E4M3, torch.float32), iters)
     out['c1_dequant_e4m3_fp32'] = {'ms': ms, 'GBps': x.numel() * 5 / ms / 1e6}
-    del x, q
+    # the same cast with nothing in the caches: eight distinct 64 MiB inputs in turn (512 MiB, twice the 256 MiB
+    # memory-side cache), which is how a training step meets its activations
+    xs = [x] + [torch.randn_like(x) for _ in range(7)]
+    turn = {'i': 0}
+
+    def cold_cast():
+        turn['i'] = (turn['i'] + 1) % len(xs)
+        _backend.cast_to_fp8_intime(xs[turn['i']], s, am[0:1], si, _backend.DT_E4M3)
+
+    ms = _time_gpu(cold_cast, 2 * len(xs), warm=len(xs))
+    out['c1_intime_fp32_e4m3_cold'] = {'ms': ms, 'GBps': x.numel() * 5 / ms / 1e6}
+    del x, q, xs
     a = torch.randn(8192, 4096, device='cuda').bfloat16()
     ms = _time_gpu(lambda: _backend.cast_to_fp8(a, s, am[0:1], si, _backend.DT_E4M3), iters)
     out['c2_delayed_bf16_e4m3'] = {'ms': ms, 'GBps': a.numel() * 3 / ms / 1e6}
