@@ -157,7 +157,6 @@ __global__ __launch_bounds__(THREADS) void cast_to_fp8_kernel(const IT* __restri
 // ---------------------------------------------------------------------------------------------
 // First pass of the in-time casts: NaN-propagating max|x| per workgroup, written to the workspace
 // (no atomics, no fences: the kernel boundary orders it before the second pass).
-__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 
 // With fin.amax set, the workgroup that finishes last (a ticket counter in the workspace tells) also
 // reduces the partial maxima and applies the scale rule, which saves the finalize launch.
@@ -293,9 +292,6 @@ __global__ __launch_bounds__(kCastThreads) void amax_finalize_kernel(const uint3
 constexpr int kResThreads = 512;
 constexpr int kResVecs = 16;
 constexpr int kResBlocksPerCu = 2;
-constexpr int kWsSlotBytes = 8192;
-constexpr int kMaxSlots = 512;
-static_assert(kWsSlotBytes + (kMaxSlots + 2) * 8 <= MSAMP_WORKSPACE_BYTES, "slots exceed the workspace");
 
 template <typename IT>
 __device__ __forceinline__ uint32_t abs_bits_hi(uint32_t raw) {    // raw element bits -> ordered key

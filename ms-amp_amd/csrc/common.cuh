@@ -196,6 +196,14 @@ __device__ __forceinline__ float dequant1(uint32_t byte) {
     return a;
 }
 
+// ---- meeting place of the kernels whose workgroups wait for each other --------------------------------
+// `kMaxSlots` eight-byte {token, max} slots start at byte kWsSlotBytes of the workspace; two post words follow.
+constexpr int kWsSlotBytes = 8192;
+constexpr int kMaxSlots = 512;
+static_assert(kWsSlotBytes + (kMaxSlots + 2) * 8 <= MSAMP_WORKSPACE_BYTES, "slots exceed the workspace");
+
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+
 // ---- reductions ------------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
 #pragma unroll

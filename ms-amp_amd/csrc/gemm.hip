@@ -265,13 +265,48 @@ __device__ __forceinline__ void wait_vmcnt() {
 //    row count to be a multiple of 256.
 typedef int v2i __attribute__((ext_vector_type(2)));
 
-template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
+//  * QF (an FP8 format, or 0): the output is not stored in OT but cast on to FP8 with in-time scaling in the same
+//    launch, the way cast_to_fp8 of the stored output would: D is rounded to OT in registers, max |D| is taken over
+//    the whole matrix, the scale follows from it, and the codes of D * scale are what reaches memory -- bit for
+//    bit what the two steps give, without D's trip through memory.  Every workgroup holds its tile in registers
+//    while the maxima meet (slots in the workspace, as in the one-pass in-time cast), so the launch must have all
+//    its workgroups on the chip at once: the host only takes this path for at most one tile per CU.
+struct QuantArgs {
+    uint8_t* q;          // [NR][NC] FP8 codes
+    float* scale;        // in: the fallback of the scale rule; out: the scale used
+    float* amax;         // out: max |D|
+    float* scale_inv;    // out: 1 / scale
+    uint64_t* slots;     // kMaxSlots meeting slots and two post words
+    float fp_max;
+    int margin;
+    int flags;
+    uint32_t token;
+    uint32_t spin_limit;
+};
+
+// a * b rounded to OT (as the plain epilogue stores it) and widened again
+template <typename OT>
+__device__ __forceinline__ void round_pair(float a, float b, float& ra, float& rb) {
+    if constexpr (sizeof(OT) == 4) {
+        ra = a, rb = b;
+    } else if constexpr (__is_same(OT, bf16_t)) {
+        const uint32_t p = pack_bf16(a, b);
+        ra = __uint_as_float(p << 16), rb = __uint_as_float(p & 0xffff0000u);
+    } else {
+        const f32x2 v = {a, b};
+        const f16x2 h = __builtin_convertvector(v, f16x2);
+        ra = static_cast<float>(h[0]), rb = static_cast<float>(h[1]);
+    }
+}
+
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
                                                                      const uint8_t* __restrict__ Y, OT* __restrict__ D,
                                                                      int NR, int NC, int K,
                                                                      const float* __restrict__ x_scale_inv,
                                                                      const float* __restrict__ y_scale_inv, int accumulate,
-                                                                     const void* __restrict__ bias, int bias_dt) {
+                                                                     const void* __restrict__ bias, int bias_dt,
+                                                                     QuantArgs qa) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     int tr, tc;
     tile_of_block((NR + kDmaTile - 1) / kDmaTile, (NC + kDmaTile - 1) / kDmaTile, tr, tc);
@@ -437,6 +472,126 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // No barrier here: the last LDS reads of every wave were issued (and awaited) before the barrier of the last
     // slice, and no load is in flight, so each wave may start on its patch as soon as its own MFMAs are done.
 
+    if constexpr (QF != 0) {
+        // ---- fused in-time cast (whole tiles only, no bias, no accumulation: the host sees to that)
+        __shared__ uint32_t q_red[kGemmThreads / kWave];
+        __shared__ uint32_t q_scale, q_amax;
+        const float alpha = alpha_early;
+        // max |acc| as an ordered bit pattern: NaN above Inf above everything finite, so a NaN reaches the amax
+        // as it does through abs().max()
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) m = umax(m, __float_as_uint(acc[i][j][r]) & 0x7fffffffu);
+        m = block_max_u32(m, q_red);    // valid in lane 0 of wave 0
+        const int tid = threadIdx.x;
+        if (tid == 0) {
+            // Scaling by |alpha| and rounding to OT never reorder magnitudes, so the maximum of the rounded outputs
+            // is the rounded, scaled maximum.
+            float am, unused;
+            round_pair<OT>(__uint_as_float(m) * fabsf(alpha), 0.0f, am, unused);
+            m = __float_as_uint(am) & 0x7fffffffu;
+            __hip_atomic_store(qa.slots + blockIdx.x, (static_cast<uint64_t>(qa.token) << 32) | m, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // Workgroup 0 collects the slots (its first wave), derives amax and scale and posts
+        // both, tagged with the token, in the two words behind the slots; the other workgroups poll only those.
+        // Every wait is bounded: if it runs out, amax and scale become NaN, which no caller can overlook.
+        uint64_t* post = qa.slots + kMaxSlots;
+        if (blockIdx.x == 0) {
+            if (tid < kWave) {
+                uint32_t spins = 0, mm;
+                bool all_in;
+                do {
+                    uint64_t sv[kMaxSlots / kWave];
+#pragma unroll
+                    for (int j = 0; j < kMaxSlots / kWave; ++j)
+                        sv[j] = __hip_atomic_load(qa.slots + tid + j * kWave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    bool ok = true;
+                    mm = 0;
+#pragma unroll
+                    for (int j = 0; j < kMaxSlots / kWave; ++j) {
+                        const bool live = static_cast<uint32_t>(tid + j * kWave) < gridDim.x;
+                        ok = ok && (!live || static_cast<uint32_t>(sv[j] >> 32) == qa.token);
+                        mm = umax(mm, live ? static_cast<uint32_t>(sv[j]) : 0u);
+                    }
+                    all_in = __all(ok);
+                } while (!all_in && ++spins < qa.spin_limit);
+                mm = wave_max_u32(mm);
+                if (tid == 0) {
+                    float am = __uint_as_float(mm);
+                    if (!all_in) am = __uint_as_float(0x7fc00000u);
+                    else if ((qa.flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
+                    const float sc = scale_rule(am, *qa.scale, qa.fp_max, qa.margin);
+                    const uint64_t tag = static_cast<uint64_t>(qa.token) << 32;
+                    __hip_atomic_store(post, tag | __float_as_uint(am), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(post + 1, tag | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    q_scale = __float_as_uint(sc);
+                    q_amax = __float_as_uint(am);
+                    *qa.amax = am;
+                    *qa.scale = sc;
+                    *qa.scale_inv = 1.0f / sc;
+                }
+            }
+        } else {
+            if (tid == 0) {
+                uint32_t spins = 0;
+                uint64_t pa, ps;
+                bool posted;
+                do {
+                    pa = __hip_atomic_load(post, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ps = __hip_atomic_load(post + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    posted = static_cast<uint32_t>(pa >> 32) == qa.token && static_cast<uint32_t>(ps >> 32) == qa.token;
+                } while (!posted && ++spins < qa.spin_limit);
+                q_amax = posted ? static_cast<uint32_t>(pa) : 0x7fc00000u;
+                q_scale = posted ? static_cast<uint32_t>(ps) : 0x7fc00000u;
+            }
+        }
+        __syncthreads();    // also: every wave is through with the stages, which the patches below reuse
+        const float sc = __uint_as_float(q_scale);
+        // with a positive finite amax and the scale derived from it nothing leaves the format and nothing is NaN:
+        // the clamp and the NaN patch of the general conversion can go
+        const bool in_range = __uint_as_float(q_amax) * sc <= qa.fp_max && __uint_as_float(q_amax) > 0.0f;
+        constexpr int kQPitch = 128 + 16;    // bytes per patch row: 128 codes and padding that staggers the banks
+        uint8_t* qpatch = smem + wave * (32 * kQPitch);
+        auto emit = [&](auto checked) {
+            constexpr bool kChecked = decltype(checked)::value;
+            static_for<4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        // the outputs as OT would hold them, then scaled
+                        float r0, r1, r2, r3;
+                        round_pair<OT>(acc[i][j][4 * q] * alpha, acc[i][j][4 * q + 1] * alpha, r0, r1);
+                        round_pair<OT>(acc[i][j][4 * q + 2] * alpha, acc[i][j][4 * q + 3] * alpha, r2, r3);
+                        uint32_t w;
+                        if constexpr (kChecked) w = quant4<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
+                        else w = quant4_in_range<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
+                        *reinterpret_cast<uint32_t*>(qpatch + l32 * kQPitch + j * 32 + q * 8 + lh * 4) = w;
+                    }
+                });
+                // the patch is private to this wave and the LDS serves one wave's requests in order: no waits here
+                auto rd = [&](int u) {
+                    return *reinterpret_cast<const uint4*>(qpatch + (u * 8 + (lane >> 3)) * kQPitch + (lane & 7) * 16);
+                };
+                const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3);
+                auto st = [&](int u, const uint4& v) {
+                    const int grow = row0 + wr * 128 + i * 32 + u * 8 + (lane >> 3);
+                    const int gcol = col0 + wc * 128 + (lane & 7) * 16;
+                    *reinterpret_cast<uint4*>(qa.q + static_cast<size_t>(grow) * NC + gcol) = v;
+                };
+                st(0, val0), st(1, val1), st(2, val2), st(3, val3);
+            });
+        };
+        if (in_range) emit(std::false_type{}); else emit(std::true_type{});
+        return;
+    }
+
     // ---- epilogue: per 32-row block, accumulators -> this wave's LDS patch -> 16-byte row stores
     constexpr int kEsz = static_cast<int>(sizeof(OT));
     constexpr int kPitch = 128 * kEsz + 16;    // bytes per patch row (padding staggers the banks)
@@ -518,8 +673,27 @@ static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, 
     }
     const int tiles = ((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
     hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys,
-                       accumulate, bias, bias_dt);
+                       accumulate, bias, bias_dt, QuantArgs{});
     MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel");
+    return MSAMP_OK;
+}
+
+// the same kernel with the in-time cast to FP8 fused in (see QF above); the caller has checked the shape
+template <int XF, int YF, typename OT, bool XT, bool YT, int QF>
+static int launch_gemm_dma_quant(const uint8_t* X, const uint8_t* Y, int NR, int NC, int K, const float* xs, const float* ys,
+                                 const QuantArgs& qa, hipStream_t st) {
+    constexpr int smem = 2 * kDmaStage;
+    static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, QF>;
+    if (!configured.load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel, fused cast)");
+        configured.store(true, std::memory_order_release);
+    }
+    const int tiles = (NR / kDmaTile) * (NC / kDmaTile);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(nullptr), NR, NC, K, xs, ys, 0,
+                       static_cast<const void*>(nullptr), 0, qa);
+    MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel (fused cast)");
     return MSAMP_OK;
 }
 
@@ -606,9 +780,65 @@ static int pick_types_kmajor(const uint8_t* X, int x_type, const uint8_t* Y, int
     return pick_out_kmajor<MSAMP_DT_E5M2, MSAMP_DT_E5M2, XT, YT>(X, Y, D, d_dtype, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
 }
 
+template <int XF, int YF, bool T>
+static int pick_out_quant(const uint8_t* X, const uint8_t* Y, int d_dtype, int NR, int NC, int K, const float* xs, const float* ys,
+                          const QuantArgs& qa, hipStream_t st) {
+    switch (d_dtype) {
+        case MSAMP_DT_F32:
+            return launch_gemm_dma_quant<XF, YF, float, T, T, MSAMP_DT_E4M3>(X, Y, NR, NC, K, xs, ys, qa, st);
+        case MSAMP_DT_F16:
+            return launch_gemm_dma_quant<XF, YF, f16_t, T, T, MSAMP_DT_E4M3>(X, Y, NR, NC, K, xs, ys, qa, st);
+        default:
+            return launch_gemm_dma_quant<XF, YF, bf16_t, T, T, MSAMP_DT_E4M3>(X, Y, NR, NC, K, xs, ys, qa, st);
+    }
+}
+
+template <bool T>
+static int pick_types_quant(const uint8_t* X, int x_type, const uint8_t* Y, int y_type, int d_dtype, int NR, int NC, int K,
+                            const float* xs, const float* ys, const QuantArgs& qa, hipStream_t st) {
+    if (x_type == MSAMP_DT_E4M3 && y_type == MSAMP_DT_E4M3)
+        return pick_out_quant<MSAMP_DT_E4M3, MSAMP_DT_E4M3, T>(X, Y, d_dtype, NR, NC, K, xs, ys, qa, st);
+    if (x_type == MSAMP_DT_E4M3)
+        return pick_out_quant<MSAMP_DT_E4M3, MSAMP_DT_E5M2, T>(X, Y, d_dtype, NR, NC, K, xs, ys, qa, st);
+    if (y_type == MSAMP_DT_E4M3)
+        return pick_out_quant<MSAMP_DT_E5M2, MSAMP_DT_E4M3, T>(X, Y, d_dtype, NR, NC, K, xs, ys, qa, st);
+    return pick_out_quant<MSAMP_DT_E5M2, MSAMP_DT_E5M2, T>(X, Y, d_dtype, NR, NC, K, xs, ys, qa, st);
+}
+
 }    // namespace msamp
 
 using namespace msamp;
+
+extern "C" int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
+                                   int b_type, const float* b_scale_inv, int b_kmajor, int d_dtype, uint8_t* q, int q_type,
+                                   float* scale, float* amax, float* scale_inv, int m, int n, int k, int margin, int flags,
+                                   void* workspace, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(a_type) && is_fp8(b_type) && is_fp8(q_type), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_cast: types %d, %d -> %d",
+                  a_type, b_type, q_type);
+    MSAMP_REQUIRE(is_hp(d_dtype), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_cast: intermediate dtype %d", d_dtype);
+    MSAMP_REQUIRE(m > 0 && n > 0 && k > 0, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_cast: m=%d n=%d k=%d", m, n, k);
+    MSAMP_REQUIRE(a && b && q && a_scale_inv && b_scale_inv && scale && amax && scale_inv, MSAMP_ERR_NULL,
+                  "msamp_fp8_gemm_cast: null pointer");
+    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(q, 16), MSAMP_ERR_SHAPE,
+                  "msamp_fp8_gemm_cast: operands and output must be 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool both = a_kmajor && b_kmajor, neither = !a_kmajor && !b_kmajor;
+    const long tiles = static_cast<long>(n / kDmaTile) * (m / kDmaTile);
+    const bool fits32 = static_cast<unsigned long long>(n) * k < (1ull << 32) && static_cast<unsigned long long>(m) * k < (1ull << 32);
+    if (q_type != MSAMP_DT_E4M3 || !(both || neither) || m % kDmaTile || n % kDmaTile || k % kBK || !fits32 ||
+        tiles > cu_count() || tiles > kMaxSlots || workspace == nullptr || (flags & MSAMP_FLAG_TWO_PASS) ||
+        !waiting_kernels_allowed(st))
+        return MSAMP_NOT_FUSED;
+    QuantArgs qa;
+    qa.q = q, qa.scale = scale, qa.amax = amax, qa.scale_inv = scale_inv;
+    qa.slots = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + kWsSlotBytes);
+    qa.fp_max = fp8_max(q_type), qa.margin = margin, qa.flags = flags;
+    qa.token = next_tokens(1);
+    qa.spin_limit = 1u << 20;    // a fraction of a second of polling
+    // X = b (rows of D), Y = a (columns of D)
+    if (both) return pick_types_quant<true>(b, b_type, a, a_type, d_dtype, n, m, k, b_scale_inv, a_scale_inv, qa, st);
+    return pick_types_quant<false>(b, b_type, a, a_type, d_dtype, n, m, k, b_scale_inv, a_scale_inv, qa, st);
+}
 
 extern "C" int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
                                      int b_type, const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int m, int n,

@@ -46,6 +46,7 @@ _SIGNATURES = {
     'msamp_cast_transpose_gated': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp], _i),
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_fp8_gemm_cast': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp], _i),
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
     'msamp_fp8_norms': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
     'msamp_bucket_amax': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
@@ -379,6 +380,33 @@ def fp8_gemm(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, out, accumulate=False, 
             1 if accumulate else 0, _ptr(bias), _dt(bias) if bias is not None else DT_F32, _stream()
         ), 'msamp_fp8_gemm'
     )
+    return out
+
+
+NOT_FUSED = 1
+
+
+def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, scale, amax_cell, scale_inv, margin=0,
+                  nan_to_inf=False, a_kmajor=False, b_kmajor=False):
+    """The product of fp8_gemm, rounded to hp_dtype and cast on to FP8 with in-time scaling (amax_cell[0], scale and
+    scale_inv are updated) in one launch.  Returns the uint8 payload [N, M], or None when the fused form does not apply
+    to this problem or stream (nothing has been touched then): take fp8_gemm and cast_to_fp8_intime instead."""
+    lib = load()
+    _gpu(a, 'mat_a')
+    _gpu(b, 'mat_b')
+    k, m = a.shape if a_kmajor else a.shape[::-1]
+    kb, n = b.shape if b_kmajor else b.shape[::-1]
+    if kb != k:
+        raise ValueError(f'shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}')
+    out = torch.empty(n, m, dtype=torch.uint8, device=a.device)
+    rc = lib.msamp_fp8_gemm_cast(
+        _ptr(a), a_dt, _ptr(a_scale_inv), 1 if a_kmajor else 0, _ptr(b), b_dt, _ptr(b_scale_inv), 1 if b_kmajor else 0,
+        _TORCH_TO_DT[hp_dtype], _ptr(out), q_dt, _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), m, n, k, margin,
+        (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _shared_device() else 0), _ptr(workspace(a.device)), _stream()
+    )
+    if rc == NOT_FUSED:
+        return None
+    _check(rc, 'msamp_fp8_gemm_cast')
     return out
 
 

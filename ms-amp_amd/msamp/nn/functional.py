@@ -57,19 +57,24 @@ class _FP8GemmFunction(torch.autograd.Function):
                 mat_a, mat_b, layout = ctx.input_fp8, ograd_fp8, dict(a_kmajor=True, b_kmajor=True)
             else:
                 mat_a, mat_b, layout = ctx.input_fp8.fp8_transpose(), ograd_fp8_t, {}
-            if ctx.weight.grad is None:
-                wgrad = Gemm.fp8_gemm(mat_a, mat_b, ctx.output_qtype, use_split_accumulator=True, **layout)
-            else:
-                # gradient accumulation: add into the dequantized previous gradient
-                old_wgrad = ctx.weight.grad.to(ctx.output_dtype)
-                wgrad = Gemm.fp8_gemm(
-                    mat_a, mat_b, ctx.output_qtype, accumulate=True, out=old_wgrad, use_split_accumulator=True, **layout
-                )
-                del old_wgrad
-            if model_state.use_fp8_ddp:
-                wgrad.meta = metas['wgrad']
-            else:
-                wgrad = wgrad.cast(Dtypes.kfloat8_e4m3, meta=metas['wgrad'], sync=True)
+            wgrad = None
+            if ctx.weight.grad is None and not model_state.use_fp8_ddp:
+                # GEMM and cast in one launch where the kernel takes the problem (same bits as the two steps below)
+                wgrad = Gemm.fp8_gemm_cast(mat_a, mat_b, ctx.output_qtype, metas['wgrad'], sync=True, **layout)
+            if wgrad is None:
+                if ctx.weight.grad is None:
+                    wgrad = Gemm.fp8_gemm(mat_a, mat_b, ctx.output_qtype, use_split_accumulator=True, **layout)
+                else:
+                    # gradient accumulation: add into the dequantized previous gradient
+                    old_wgrad = ctx.weight.grad.to(ctx.output_dtype)
+                    wgrad = Gemm.fp8_gemm(
+                        mat_a, mat_b, ctx.output_qtype, accumulate=True, out=old_wgrad, use_split_accumulator=True, **layout
+                    )
+                    del old_wgrad
+                if model_state.use_fp8_ddp:
+                    wgrad.meta = metas['wgrad']
+                else:
+                    wgrad = wgrad.cast(Dtypes.kfloat8_e4m3, meta=metas['wgrad'], sync=True)
             ctx.weight.backward_grad_update(wgrad)
 
         return input_grad, None, None, None

@@ -24,6 +24,25 @@ class Gemm:
 
     @classmethod
     @torch.no_grad()
+    def fp8_gemm_cast(cls, mat_a, mat_b, out_qtype, meta, sync=False, a_kmajor=False, b_kmajor=False):
+        """fp8_gemm(mat_a, mat_b, out_qtype).cast(meta.qtype, meta=meta, sync=sync) for a meta with in-time scaling,
+        as one kernel launch (not in the reference, which takes the two steps: nn/functional.py:100-123).  Returns the
+        FP8 ScalingTensor, or None if the fused kernel does not take this problem -- the caller then takes the two
+        steps itself; the result is the same bit for bit."""
+        assert isinstance(mat_a, ScalingTensor) and isinstance(mat_b, ScalingTensor)
+        assert mat_a.is_cuda and mat_a.is_contiguous() and mat_b.is_cuda and mat_b.is_contiguous()
+        assert Dtypes.is_fp8_qtype(mat_a.qtype) and Dtypes.is_fp8_qtype(mat_b.qtype) and Dtypes.is_fp8_qtype(meta.qtype)
+        if meta.scaling_mode() != 'in_time' or (a_kmajor != b_kmajor):
+            return None
+        payload = _backend.fp8_gemm_cast(
+            mat_a.value, int(mat_a.qtype), mat_a.meta.scale_inv, mat_b.value, int(mat_b.qtype), mat_b.meta.scale_inv,
+            Dtypes.get_dtype_from_qtype(out_qtype), int(meta.qtype), meta.scale, meta.amax[0:1], meta.scale_inv,
+            nan_to_inf=sync, a_kmajor=a_kmajor, b_kmajor=b_kmajor
+        )
+        return None if payload is None else ScalingTensor(payload, meta)
+
+    @classmethod
+    @torch.no_grad()
     def fp8_gemm(
         cls, mat_a, mat_b, out_qtype, bias=None, accumulate=False, out=None, use_split_accumulator=False, a_kmajor=False,
         b_kmajor=False

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from oracle import fp8, gemm as ogemm
-from tests.gpu_util import FMT, rel_fro
+from tests.gpu_util import FMT, rel_fro, same_float
 
 pytestmark = pytest.mark.gpu
 
@@ -265,3 +265,116 @@ def test_operand_beyond_4_gib(be):
     rows = torch.tensor([0, 65535, 65536, 65537, n - 1])
     want = ogemm.fp8_gemm(a.cpu(), torch.tensor(2.0**-8), fp8.E4M3, b[rows.cuda()].cpu(), torch.tensor(2.0**-8), fp8.E4M3)
     assert rel_fro(out[rows.cuda()], want) < TOL_F32
+
+
+def _two_steps(be, a, a_dt, sa, b, b_dt, sb, hp, nan_to_inf, kmajor, old_scale=1.0):
+    """The unfused path: GEMM into an hp buffer, then the in-time cast of that buffer."""
+    k, m = a.shape if kmajor else a.shape[::-1]
+    n = b.shape[1] if kmajor else b.shape[0]
+    d = be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, torch.empty(n, m, dtype=hp, device='cuda'), a_kmajor=kmajor, b_kmajor=kmajor)
+    s, si, am = torch.full((), old_scale, device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+    q = be.cast_to_fp8_intime(d, s, am, si, 5, nan_to_inf=nan_to_inf)
+    return q, s, si, am
+
+
+@pytest.mark.parametrize('a_dt,b_dt', [(5, 6), (5, 5), (6, 6)])
+@pytest.mark.parametrize('m,n,k', [(256, 256, 128), (1024, 512, 384), (4096, 4096, 512), (2048, 8192, 256)])
+@pytest.mark.parametrize('hp', [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize('kmajor', [True, False])
+def test_gemm_with_fused_cast_matches_the_two_steps(be, a_dt, b_dt, m, n, k, hp, kmajor):
+    """GEMM + in-time cast in one launch: payload, amax, scale and scale_inv must equal, bit for bit, what the GEMM
+    into an hp buffer followed by the in-time cast of that buffer gives (the weight-gradient path of FP8Linear)."""
+    a = _rand_fp8((m, k), a_dt, 3 * m + k).cuda()
+    b = _rand_fp8((n, k), b_dt, 5 * n + k, spread=0.5).cuda()
+    if kmajor:
+        a, b = a.t().contiguous(), b.t().contiguous()
+    sa, sb = torch.tensor(0.125, device='cuda'), torch.tensor(0.5, device='cuda')
+    want_q, want_s, want_si, want_am = _two_steps(be, a, a_dt, sa, b, b_dt, sb, hp, True, kmajor)
+    s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+    got = be.fp8_gemm_cast(a, a_dt, sa, b, b_dt, sb, hp, 5, s, am, si, nan_to_inf=True, a_kmajor=kmajor, b_kmajor=kmajor)
+    assert got is not None, 'the fused kernel should take this problem'
+    assert torch.equal(got, want_q)
+    assert same_float(am, want_am) and same_float(s, want_s) and same_float(si, want_si)
+    assert float(want_am) > 0
+
+
+@pytest.mark.parametrize('nan_to_inf', [True, False])
+@pytest.mark.parametrize('poison', ['nan', 'inf', 'zero'])
+def test_gemm_with_fused_cast_special_values(be, nan_to_inf, poison):
+    """A NaN or Inf in the product (E5M2 operands carry them) reaches amax as through the two steps, the scale falls
+    back to the old one; an all-zero product leaves amax 0 and the old scale."""
+    m, n, k = 512, 256, 128
+    a = _rand_fp8((m, k), 6, 1).cuda()
+    b = _rand_fp8((n, k), 6, 2).cuda()
+    if poison == 'nan':
+        a[7, 5] = 0x7f
+    elif poison == 'inf':
+        a[7, 5] = 0x7c
+    else:
+        a.zero_()
+    one = torch.ones((), device='cuda')
+    want_q, want_s, want_si, want_am = _two_steps(be, a, 6, one, b, 6, one, torch.bfloat16, nan_to_inf, False, old_scale=4.0)
+    s, si, am = torch.full((), 4.0, device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+    got = be.fp8_gemm_cast(a, 6, one, b, 6, one, torch.bfloat16, 5, s, am, si, nan_to_inf=nan_to_inf)
+    assert got is not None
+    assert torch.equal(got, want_q)
+    assert same_float(am, want_am) and same_float(s, want_s) and same_float(si, want_si)
+
+
+def test_gemm_with_fused_cast_declines_what_it_cannot_take(be):
+    """Ragged shapes, mixed layouts, more tiles than compute units, a capturing stream: None, and nothing written."""
+    one = torch.ones((), device='cuda')
+
+    def call(m, n, k, **kw):
+        a = _rand_fp8((m, k), 5, 1).cuda()
+        b = _rand_fp8((n, k), 5, 2).cuda()
+        s, si, am = torch.full((), 2.0, device='cuda'), torch.full((), 3.0, device='cuda'), torch.full((1,), 5.0, device='cuda')
+        got = be.fp8_gemm_cast(a, 5, one, b, 5, one, torch.bfloat16, kw.pop('q_dt', 5), s, am, si, **kw)
+        return got, float(s), float(si), float(am)
+
+    assert call(300, 256, 128) == (None, 2.0, 3.0, 5.0)
+    assert call(256, 256, 144) == (None, 2.0, 3.0, 5.0)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    side = 256 * (int(cus ** 0.5) + 1)
+    assert call(side, side, 128) == (None, 2.0, 3.0, 5.0)
+    assert call(256, 256, 128, q_dt=6) == (None, 2.0, 3.0, 5.0)
+    got, *_ = call(256, 256, 128)
+    assert got is not None
+
+
+def test_fp8linear_weight_gradient_uses_the_fused_kernel_and_matches():
+    """FP8Linear backward: the weight gradient from the fused launch equals the one from the two steps."""
+    import msamp
+    from msamp import _backend
+    from msamp.nn import LinearReplacer
+    from msamp.common.dtype import Dtypes
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(512, 256, bias=False).cuda().bfloat16()
+    model = LinearReplacer.replace(lin, Dtypes.kfloat16)
+    x = torch.randn(1024, 512, device='cuda', dtype=torch.bfloat16)
+    dy = torch.randn(1024, 256, device='cuda', dtype=torch.bfloat16)
+
+    def grad(fused):
+        saved = _backend.fp8_gemm_cast
+        calls = []
+        if fused:
+            def spy(*a, **kw):
+                out = saved(*a, **kw)
+                calls.append(out is not None)
+                return out
+            _backend.fp8_gemm_cast = spy
+        else:
+            _backend.fp8_gemm_cast = lambda *a, **kw: None
+        try:
+            for p in model.parameters():
+                p.grad = None
+            model(x).backward(dy)
+        finally:
+            _backend.fp8_gemm_cast = saved
+        g = model.weight.grad
+        return g.value.clone(), g.meta.scale.clone(), g.meta.scale_inv.clone(), g.meta.amax.clone(), calls
+
+    q1, s1, si1, am1, calls = grad(True)
+    assert calls == [True]
+    q0, s0, si0, am0, _ = grad(False)
+    assert torch.equal(q1, q0) and same_float(s1, s0) and same_float(si1, si0) and same_float(am1, am0)
