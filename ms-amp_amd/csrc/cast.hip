@@ -874,7 +874,15 @@ static int launch_cast(const IT* x, size_t n, const float* scale, float* amax, f
 #define LAUNCH(FMT, AM, INT) \
     hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, AM, INT>), dim3(grid), dim3(kCastThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, INT == kInTime ? 1 : 0, INT != kGivenScale ? *it : none)
     if (it != nullptr && it->known_amax != nullptr) {
-        if (fp8_type == MSAMP_DT_E4M3) LAUNCH(MSAMP_DT_E4M3, false, kRescale); else LAUNCH(MSAMP_DT_E5M2, false, kRescale);
+        // few, large, long-lived workgroups (two of 512 lanes per CU, grid-stride), like the cast that publishes an amax
+        constexpr int kBigThreads = 512;
+        int g2 = grid_for(n, static_cast<size_t>(kBigThreads) * EPT * kCastUnroll);
+        const int cap = cu_count() * 2;
+        g2 = g2 < cap ? g2 : cap;
+#define LAUNCH_RESCALE(FMT) \
+    hipLaunchKernelGGL((cast_to_fp8_kernel<IT, FMT, false, kRescale, kBigThreads>), dim3(g2), dim3(kBigThreads), 0, st, x, out, n, scale, amax, scale_inv, vec_ok, 0, *it)
+        if (fp8_type == MSAMP_DT_E4M3) LAUNCH_RESCALE(MSAMP_DT_E4M3); else LAUNCH_RESCALE(MSAMP_DT_E5M2);
+#undef LAUNCH_RESCALE
     } else if (it != nullptr) {
         // second pass of an in-time cast: fewer, longer-lived workgroups (each one re-derives the scale),
         // walking the tensor back to front to meet what the first pass left in the caches
