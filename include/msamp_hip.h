@@ -236,8 +236,9 @@ int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv
  * buffer.  flags and workspace as for msamp_cast_to_fp8_intime.
  * Returns MSAMP_NOT_FUSED (1), having done nothing, when the fused form does not apply and the caller has to take
  * the two steps: it needs m and n multiples of 256, k a multiple of 128, at most one 256 x 256 output tile per
- * compute unit (its workgroups wait for each other), q_type E4M3, both operands K-major or neither, a stream on which
- * such kernels are allowed (not capturing, the device's first), and no MSAMP_FLAG_TWO_PASS. */
+ * compute unit (its workgroups wait for each other), q_type E4M3, both operands K-major or neither (and with neither,
+ * enough tiles that msamp_fp8_gemm would use the same kernel), a stream on which such kernels are allowed (not
+ * capturing, the device's first), and no MSAMP_FLAG_TWO_PASS. */
 #define MSAMP_NOT_FUSED 1
 int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b, int b_type,
                         const float* b_scale_inv, int b_kmajor, int d_dtype, uint8_t* q, int q_type, float* scale,

@@ -826,9 +826,12 @@ extern "C" int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_
     const long tiles = static_cast<long>(n / kDmaTile) * (m / kDmaTile);
     const bool fits32 = static_cast<unsigned long long>(n) * k < (1ull << 32) && static_cast<unsigned long long>(m) * k < (1ull << 32);
     if (q_type != MSAMP_DT_E4M3 || !(both || neither) || m % kDmaTile || n % kDmaTile || k % kBK || !fits32 ||
-        tiles > cu_count() || tiles > kMaxSlots || workspace == nullptr || (flags & MSAMP_FLAG_TWO_PASS) ||
-        !waiting_kernels_allowed(st))
+        tiles > cu_count() || tiles > kMaxSlots || workspace == nullptr || (flags & MSAMP_FLAG_TWO_PASS))
         return MSAMP_NOT_FUSED;
+    // Row-major operands with few tiles: msamp_fp8_gemm would take its generic kernel there, which adds the K slices up
+    // in another order; decline, so that this entry and the two steps always agree to the bit.
+    if (neither && tiles * 2 < cu_count()) return MSAMP_NOT_FUSED;
+    if (!waiting_kernels_allowed(st)) return MSAMP_NOT_FUSED;
     QuantArgs qa;
     qa.q = q, qa.scale = scale, qa.amax = amax, qa.scale_inv = scale_inv;
     qa.slots = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + kWsSlotBytes);

@@ -292,6 +292,12 @@ def test_gemm_with_fused_cast_matches_the_two_steps(be, a_dt, b_dt, m, n, k, hp,
     want_q, want_s, want_si, want_am = _two_steps(be, a, a_dt, sa, b, b_dt, sb, hp, True, kmajor)
     s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
     got = be.fp8_gemm_cast(a, a_dt, sa, b, b_dt, sb, hp, 5, s, am, si, nan_to_inf=True, a_kmajor=kmajor, b_kmajor=kmajor)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    if not kmajor and (m // 256) * (n // 256) * 2 < cus:
+        # row-major operands with few tiles go to the generic kernel in fp8_gemm (another summation order), so the
+        # fused entry declines rather than differ from the two steps in a last bit here and there
+        assert got is None and float(s) == 1.0 and float(am) == 0.0
+        return
     assert got is not None, 'the fused kernel should take this problem'
     assert torch.equal(got, want_q)
     assert same_float(am, want_am) and same_float(s, want_s) and same_float(si, want_si)
@@ -304,8 +310,8 @@ def test_gemm_with_fused_cast_special_values(be, nan_to_inf, poison):
     """A NaN or Inf in the product (E5M2 operands carry them) reaches amax as through the two steps, the scale falls
     back to the old one; an all-zero product leaves amax 0 and the old scale."""
     m, n, k = 512, 256, 128
-    a = _rand_fp8((m, k), 6, 1).cuda()
-    b = _rand_fp8((n, k), 6, 2).cuda()
+    a = _rand_fp8((k, m), 6, 1).cuda()    # both operands K-major, as the backward pass has them
+    b = _rand_fp8((k, n), 6, 2).cuda()
     if poison == 'nan':
         a[7, 5] = 0x7f
     elif poison == 'inf':
@@ -313,9 +319,9 @@ def test_gemm_with_fused_cast_special_values(be, nan_to_inf, poison):
     else:
         a.zero_()
     one = torch.ones((), device='cuda')
-    want_q, want_s, want_si, want_am = _two_steps(be, a, 6, one, b, 6, one, torch.bfloat16, nan_to_inf, False, old_scale=4.0)
+    want_q, want_s, want_si, want_am = _two_steps(be, a, 6, one, b, 6, one, torch.bfloat16, nan_to_inf, True, old_scale=4.0)
     s, si, am = torch.full((), 4.0, device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
-    got = be.fp8_gemm_cast(a, 6, one, b, 6, one, torch.bfloat16, 5, s, am, si, nan_to_inf=nan_to_inf)
+    got = be.fp8_gemm_cast(a, 6, one, b, 6, one, torch.bfloat16, 5, s, am, si, nan_to_inf=nan_to_inf, a_kmajor=True, b_kmajor=True)
     assert got is not None
     assert torch.equal(got, want_q)
     assert same_float(am, want_am) and same_float(s, want_s) and same_float(si, want_si)
@@ -326,8 +332,8 @@ def test_gemm_with_fused_cast_declines_what_it_cannot_take(be):
     one = torch.ones((), device='cuda')
 
     def call(m, n, k, **kw):
-        a = _rand_fp8((m, k), 5, 1).cuda()
-        b = _rand_fp8((n, k), 5, 2).cuda()
+        a = _rand_fp8((k, m) if kw.get('a_kmajor') else (m, k), 5, 1).cuda()
+        b = _rand_fp8((k, n) if kw.get('b_kmajor') else (n, k), 5, 2).cuda()
         s, si, am = torch.full((), 2.0, device='cuda'), torch.full((), 3.0, device='cuda'), torch.full((1,), 5.0, device='cuda')
         got = be.fp8_gemm_cast(a, 5, one, b, 5, one, torch.bfloat16, kw.pop('q_dt', 5), s, am, si, **kw)
         return got, float(s), float(si), float(am)
@@ -338,7 +344,9 @@ def test_gemm_with_fused_cast_declines_what_it_cannot_take(be):
     side = 256 * (int(cus ** 0.5) + 1)
     assert call(side, side, 128) == (None, 2.0, 3.0, 5.0)
     assert call(256, 256, 128, q_dt=6) == (None, 2.0, 3.0, 5.0)
-    got, *_ = call(256, 256, 128)
+    assert call(256, 256, 128) == (None, 2.0, 3.0, 5.0)    # row-major, too few tiles for the direct-to-LDS kernel
+    assert call(256, 256, 128, a_kmajor=True) == (None, 2.0, 3.0, 5.0)    # mixed layouts
+    got, *_ = call(256, 256, 128, a_kmajor=True, b_kmajor=True)
     assert got is not None
 
 
