@@ -221,8 +221,10 @@ int msamp_fp8_gemm(const uint8_t* a, int a_type, const float* a_scale_inv, const
 /* The same product with operands handed over K-major: a_kmajor != 0 means `a` points at A^T, i.e. [K][M]
  * with M contiguous, likewise b_kmajor for [K][N].  The backward GEMMs of a linear layer
  * (nn/functional.py:84-111 of the reference) then read W, x and dy as they are, and the explicit FP8
- * transposes (transformer_engine_wrapper.py:165-176) are not needed.  Results are bit-identical to
- * msamp_fp8_gemm on transposed copies.  Supported: a K-major alone, or both; k % 128 == 0 and the row
+ * transposes (transformer_engine_wrapper.py:165-176) are not needed.  Results equal msamp_fp8_gemm on
+ * transposed copies: to the bit wherever that call runs the same direct-to-LDS kernel (from half as many 256 x 256
+ * output tiles as there are compute units); below that its generic kernel adds the K slices up in another order,
+ * which can move a last bit in a few outputs per million.  Supported: a K-major alone, or both; k % 128 == 0 and the row
  * count of every K-major operand (m, and n if b_kmajor) a multiple of 256; otherwise MSAMP_ERR_SHAPE. */
 int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
                           int b_type, const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int m, int n, int k,

@@ -129,19 +129,31 @@ def test_kmajor_operands_match_transposed_copies(be, a_dt, b_dt, m, n, k, out_dt
     b = _rand_fp8((n, k), b_dt, 13 * n + k, spread=0.5).cuda()
     a_t, b_t = a.t().contiguous(), b.t().contiguous()
     sa, sb = torch.tensor(0.25, device='cuda'), torch.tensor(2.0, device='cuda')
+    # The row-major call runs the same kernel as the K-major one from CUs/2 tiles on: equal to the bit.  Below that it
+    # takes the generic kernel, which adds the K slices up in another order: a last bit may move in a few outputs per
+    # million, no more.
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    same_kernel = ((m + 255) // 256) * ((n + 255) // 256) * 2 >= cus and k % 128 == 0
+
+    def same(got, want):
+        if same_kernel:
+            return torch.equal(got, want)
+        return (got != want).float().mean().item() < 1e-4 and rel_fro(got, want) < 1e-5
+
     want = be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'))
     got = be.fp8_gemm(a_t, a_dt, sa, b, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'), a_kmajor=True)
-    assert torch.equal(got, want)
+    assert same(got, want)
     assert be.gemm_kmajor_supported(m, n, k, True, True) == (n % 256 == 0)
     if n % 256 == 0:
-        got = be.fp8_gemm(a_t, a_dt, sa, b_t, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'), a_kmajor=True,
-                          b_kmajor=True)
-        assert torch.equal(got, want)
+        got_both = be.fp8_gemm(a_t, a_dt, sa, b_t, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'), a_kmajor=True,
+                               b_kmajor=True)
+        assert torch.equal(got_both, got)    # one kernel, two layouts: always to the bit
+        assert same(got_both, want)
         bias = torch.randn(m, device='cuda').to(out_dtype)
         base = torch.randn(n, m, device='cuda').to(out_dtype)
         want2 = be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, base.clone(), accumulate=True, bias=bias)
         got2 = be.fp8_gemm(a_t, a_dt, sa, b_t, b_dt, sb, base.clone(), accumulate=True, bias=bias, a_kmajor=True, b_kmajor=True)
-        assert torch.equal(got2, want2)
+        assert same(got2, want2)
 
 
 def test_kmajor_rejects_unsupported_shapes(be):
