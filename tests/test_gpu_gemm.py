@@ -398,3 +398,28 @@ def test_fp8linear_weight_gradient_uses_the_fused_kernel_and_matches():
     assert calls == [True]
     q0, s0, si0, am0, _ = grad(False)
     assert torch.equal(q1, q0) and same_float(s1, s0) and same_float(si1, si0) and same_float(am1, am0)
+
+
+def test_gemm_with_fused_cast_many_random_cases(be):
+    """A sweep over seeds, scales, layouts and output types at the shapes the fused kernel takes (K-major: any whole
+    tiles; row-major: from half as many tiles as compute units): every case equal to the two steps, to the bit."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    side = 256 * max(1, int((cus // 2) ** 0.5 + 0.999))    # side x side has at least cus / 2 tiles
+    cases = 0
+    for it in range(12):
+        for (m, n, k), kmajor in (((1024, 768, 384), True), ((256, 256, 1024), True), ((side, side, 256), False),
+                                  ((side, side, 384), True)):
+            hp = (torch.bfloat16, torch.float32, torch.float16)[it % 3]
+            a_dt, b_dt = ((5, 6), (6, 5), (5, 5), (6, 6))[it % 4]
+            a = _gpu_codes((k, m) if kmajor else (m, k), a_dt, 100 * it + m)
+            b = _gpu_codes((k, n) if kmajor else (n, k), b_dt, 200 * it + n)
+            sa = torch.tensor(2.0 ** -(it % 7), device='cuda')
+            sb = torch.tensor(2.0 ** -(it % 5 + 3), device='cuda')
+            want_q, want_s, want_si, want_am = _two_steps(be, a, a_dt, sa, b, b_dt, sb, hp, True, kmajor)
+            s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+            got = be.fp8_gemm_cast(a, a_dt, sa, b, b_dt, sb, hp, 5, s, am, si, nan_to_inf=True, a_kmajor=kmajor, b_kmajor=kmajor)
+            assert got is not None, (it, m, n, k, kmajor)
+            assert torch.equal(got, want_q), (it, m, n, k, kmajor, hp)
+            assert same_float(am, want_am) and same_float(s, want_s) and same_float(si, want_si), (it, m, n, k, kmajor, hp)
+            cases += 1
+    assert cases == 48
