@@ -35,7 +35,7 @@ class _FP8GemmFunction(torch.autograd.Function):
         need_dgrad, need_wgrad = ctx.input_fp8.requires_grad, ctx.weight.requires_grad
         # The reference materializes dy^T, W^T and x^T (fused cast-transpose + two FP8 transposes) because its
         # GEMM reads K-contiguous operands only.  This kernel also reads [K, rows] operands in place, so when
-        # the shapes allow, dy is only cast and W, x, dy go to the GEMMs as they are (the same products).
+        # the shapes allow, dy is only cast and W, x, dy go to the GEMMs as they are (same results).
         in_place = (not need_dgrad or Gemm.kmajor_supported(d_in, tokens, d_out, True, False)) and \
             (not need_wgrad or Gemm.kmajor_supported(d_in, d_out, tokens, True, True))
         if in_place:

