@@ -282,8 +282,7 @@ def test_training_step_replays_from_a_graph():
 
 def test_backward_without_transposed_copies_matches_the_explicit_path(monkeypatch):
     """At shapes the kernel reads K-major operands for, the backward pass skips dy^T, W^T and x^T; gradients and
-    metas must equal, bit for bit, what the path with the three explicit transposes gives (which at this size runs
-    the generic GEMM kernel: both kernels add up the same blocks of K in the same order)."""
+    metas must equal, bit for bit, what the path with the three explicit transposes gives."""
     from msamp.operators.gemm import Gemm
     tokens, d_in, d_out = 512, 256, 768
     torch.manual_seed(9)

@@ -129,8 +129,6 @@ def test_kmajor_operands_match_transposed_copies(be, a_dt, b_dt, m, n, k, out_dt
     b = _rand_fp8((n, k), b_dt, 13 * n + k, spread=0.5).cuda()
     a_t, b_t = a.t().contiguous(), b.t().contiguous()
     sa, sb = torch.tensor(0.25, device='cuda'), torch.tensor(2.0, device='cuda')
-    # The row-major call takes the generic kernel for the small shapes here and the direct-to-LDS kernel for the large
-    # one; the K-major calls always take the latter.  Both add up the same 64-byte blocks of K in the same order.
     same = torch.equal
 
     want = be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'))
@@ -408,3 +406,17 @@ def test_gemm_with_fused_cast_many_random_cases(be):
             assert same_float(am, want_am) and same_float(s, want_s) and same_float(si, want_si), (it, m, n, k, kmajor, hp)
             cases += 1
     assert cases == 48
+
+
+@pytest.mark.parametrize('m,n,k', [(256, 256, 256), (300, 200, 384), (1024, 768, 1024), (2048, 2048, 4096)])
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16])
+def test_generic_and_direct_to_lds_kernels_agree_to_the_bit(be, m, n, k, out_dtype):
+    """K a multiple of 128 goes to the direct-to-LDS kernel; the same operands with 16 zero bytes appended to every row
+    (K + 16) go to the generic kernel.  The zeros add nothing, and both kernels add up the 64-byte blocks of K in
+    ascending order, so the outputs must be equal bit for bit (which makes results independent of the dispatch)."""
+    a, b = _gpu_codes((m, k), 5, 3 * m + k), _gpu_codes((n, k), 6, 7 * n + k)
+    sa, sb = torch.tensor(0.5, device='cuda'), torch.tensor(0.25, device='cuda')
+    want = be.fp8_gemm(a, 5, sa, b, 6, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'))
+    a2, b2 = torch.nn.functional.pad(a, (0, 16)).contiguous(), torch.nn.functional.pad(b, (0, 16)).contiguous()
+    got = be.fp8_gemm(a2, 5, sa, b2, 6, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'))
+    assert torch.equal(got, want)
