@@ -420,3 +420,29 @@ def test_generic_and_direct_to_lds_kernels_agree_to_the_bit(be, m, n, k, out_dty
     a2, b2 = torch.nn.functional.pad(a, (0, 16)).contiguous(), torch.nn.functional.pad(b, (0, 16)).contiguous()
     got = be.fp8_gemm(a2, 5, sa, b2, 6, sb, torch.empty(n, m, dtype=out_dtype, device='cuda'))
     assert torch.equal(got, want)
+
+
+def test_random_small_ragged_problems_with_bias_and_accumulation(be):
+    """Random shapes up to 700 x 700 with K both a multiple of 128 (direct-to-LDS kernel, whose 256 x 256 tiles are
+    mostly padding here) and not (generic kernel), every output type, with and without bias and accumulation."""
+    import random
+    rng = random.Random(4)
+    for it in range(32):
+        m, n = rng.randint(1, 700), rng.randint(1, 700)
+        k = rng.choice([128, 256, 384, 1024, 16, 48, 144, 1040])
+        a_dt, b_dt = rng.choice([(5, 5), (5, 6), (6, 5), (6, 6)])
+        a = _rand_fp8((m, k), a_dt, 10 * it + 1)
+        b = _rand_fp8((n, k), b_dt, 10 * it + 2, spread=0.5)
+        a_si, b_si = 2.0 ** rng.randint(-6, 3), 2.0 ** rng.randint(-6, 3)
+        ref = ogemm.fp8_gemm(a, torch.tensor(a_si), FMT[a_dt], b, torch.tensor(b_si), FMT[b_dt])
+        od = rng.choice([torch.float32, torch.bfloat16, torch.float16])
+        mode = rng.choice(['plain', 'bias', 'acc', 'both'])
+        bias = torch.randn(m).to(od) if mode in ('bias', 'both') else None
+        base = torch.randn(n, m).to(od) if mode in ('acc', 'both') else None
+        if bias is not None:
+            ref = ref + bias.float()
+        if base is not None:
+            ref = ref + base.float()
+        got = _run(be, a, a_dt, a_si, b, b_dt, b_si, out_dtype=od, accumulate=base is not None, bias=bias,
+                   out=None if base is None else base.clone().cuda())
+        assert rel_fro(got.float(), ref) < (TOL_F32 if od == torch.float32 else TOL_16), (it, m, n, k, od, mode)
