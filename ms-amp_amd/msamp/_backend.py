@@ -398,6 +398,8 @@ def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, sc
     kb, n = b.shape if b_kmajor else b.shape[::-1]
     if kb != k:
         raise ValueError(f'shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}')
+    if hp_dtype not in _TORCH_TO_DT:
+        raise TypeError(f'unsupported intermediate dtype {hp_dtype}')
     out = torch.empty(n, m, dtype=torch.uint8, device=a.device)
     rc = lib.msamp_fp8_gemm_cast(
         _ptr(a), a_dt, _ptr(a_scale_inv), 1 if a_kmajor else 0, _ptr(b), b_dt, _ptr(b_scale_inv), 1 if b_kmajor else 0,
