@@ -1,12 +1,18 @@
 """Benchmark of the FP8 hot path on one MI355X.
 
-A step is one forward + backward of a single FP8Linear at x[8192,4096] (bf16), W[4096,4096] (bf16
-payload), dy[8192,4096] (bf16) in steady-state delayed scaling (amax history 16): input cast to E4M3,
-weight cast, y = x W^T, cast of dy to E5M2, dx = dy W and dW = dy^T x (the kernel reads W, x and dy
-K-major in place, so no transposed copies are made), the in-time E4M3 cast of dW and the amax-window
-update.  `value` is the three GEMMs'
-2*M*N*K flops divided by the whole step time (inputs resident in HBM).  Beside it: the GEMM kernel's
-own roofline (HIP events around the GEMM launches of every fourth step inside the timed region), the cast+amax and fused
+Headline workload (config 4 of the baseline): every FP8Linear GEMM of one Llama-7B-shaped transformer layer,
+forward and backward, at 16384 tokens -- QKV [12288,4096], O [4096,4096], gate and up [11008,4096], down
+[4096,11008] -- through the msamp API in steady-state delayed scaling (amax history 16): per layer the input
+cast to E4M3, the weight cast, y = x W^T, the cast of dy to E5M2, dx = dy W and dW = dy^T x (W, x and dy are
+read K-major in place, no transposed copies), the in-time E4M3 cast of dW; once per step the amax-window
+update.  A step is one such pass over the five layers; `value` is the fifteen GEMMs' 2*M*N*K flops divided by
+the whole step time, inputs resident in HBM.
+
+`roofline` is the GEMM kernel alone: the flops of the GEMM launches bracketed by HIP events inside the timed
+region (every fourth step), divided by their summed duration, against the dense-FP8 MFMA peak.
+
+Beside it: the same step at config 2 (one FP8Linear 8192 x 4096 x 4096), a per-shape GEMM sweep over the
+Llama-7B (config 4) and Llama-70B (config 5) projections x {forward, dgrad, wgrad}, the cast+amax and fused
 FP8-AdamW kernels against the HBM roofline, and the CPU oracle timed on the host cores.
 
 Prints one JSON line.  Synthetic data, random weights.
@@ -24,102 +30,21 @@ for _p in (ROOT, os.path.join(ROOT, 'ms-amp_amd')):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0
-GEMM_EVENT_STRIDE = 4
 FP8_PEAK_TFLOPS = 5000.0
+GEMM_EVENT_STRIDE = 4
+SCALING_WARMUP_STEPS = 17    # one more than the amax window: afterwards the casts use delayed scaling
+
+# (name, out_features, in_features) of the projections of one layer
+LLAMA_7B = {'tokens': 16384, 'proj': (('qkv', 12288, 4096), ('o', 4096, 4096), ('gate', 11008, 4096),
+                                       ('up', 11008, 4096), ('down', 4096, 11008))}
+LLAMA_70B = {'tokens': 16384, 'proj': (('qkv', 10240, 8192), ('o', 8192, 8192), ('gate', 28672, 8192),
+                                        ('up', 28672, 8192), ('down', 8192, 28672))}
+CONFIG_2 = {'tokens': 8192, 'proj': (('linear', 4096, 4096), )}
 
 
 def _events():
     import torch
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-
-
-def bench_fp8linear(steps, warmup):
-    import torch
-    import msamp    # noqa: F401
-    from msamp import _backend
-    from msamp.common.dtype import Dtypes
-    from msamp.nn import LinearReplacer, model_state
-    from msamp.optim import LBAdamW
-    import msamp.operators.gemm.gemm as gemm_mod
-
-    tokens, d_in, d_out = 8192, 4096, 4096
-    g = torch.Generator(device='cuda').manual_seed(0)
-    x = torch.randn(tokens, d_in, device='cuda', generator=g).bfloat16().requires_grad_(True)
-    dy = (torch.randn(tokens, d_out, device='cuda', generator=g) * 1e-3).bfloat16()
-    lin = torch.nn.Linear(d_in, d_out, bias=False).cuda()
-    with torch.no_grad():
-        lin.weight.copy_(torch.randn(d_out, d_in, device='cuda', generator=g) * 0.02)
-    model_state.clear()
-    model = LinearReplacer.replace(lin.bfloat16(), Dtypes.kbfloat16)
-    opt = LBAdamW(model.parameters())    # only its scaling-factor update runs here
-
-    gemm_events = []
-    real_gemm = _backend.fp8_gemm
-    real_gemm_cast = _backend.fp8_gemm_cast
-
-    class _Timed:
-        enabled = False
-
-        @staticmethod
-        def fp8_gemm(*args, **kwargs):
-            if not _Timed.enabled:
-                return real_gemm(*args, **kwargs)
-            s, e = _events()
-            s.record()
-            out = real_gemm(*args, **kwargs)
-            e.record()
-            gemm_events.append((s, e))
-            return out
-
-        @staticmethod
-        def fp8_gemm_cast(*args, **kwargs):
-            # the weight-gradient GEMM with its cast to E4M3 fused in: one launch, timed as the GEMM it is
-            if not _Timed.enabled:
-                return real_gemm_cast(*args, **kwargs)
-            s, e = _events()
-            s.record()
-            out = real_gemm_cast(*args, **kwargs)
-            e.record()
-            if out is not None:
-                gemm_events.append((s, e))
-            return out
-
-        def __getattr__(self, name):
-            return getattr(_backend, name)
-
-    gemm_mod._backend = _Timed()
-
-    def step():
-        y = model(x)
-        y.backward(dy)
-        opt._update_scaling_factors()
-        model.weight.grad = None
-        x.grad = None
-
-    for _ in range(max(warmup, 17)):    # >= 17 steps: past the 16-step warm-up, casts are single-pass
-        step()
-    assert not model.scaling_metas['input'].is_in_time_scaling()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        # an event pair costs the stream a few microseconds: bracket the GEMMs of every fourth step only
-        _Timed.enabled = i % GEMM_EVENT_STRIDE == 0
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    _Timed.enabled = False
-    gemm_mod._backend = _backend
-
-    flops_per_gemm = 2.0 * tokens * d_in * d_out
-    ms_per_step = dt / steps * 1e3
-    gemm_ms = sum(s.elapsed_time(e) for s, e in gemm_events) / len(gemm_events)
-    return {
-        'ms_per_step': ms_per_step,
-        'step_tflops': 3 * flops_per_gemm / (ms_per_step * 1e-3) / 1e12,
-        'gemm_ms': gemm_ms,
-        'gemm_tflops': flops_per_gemm / (gemm_ms * 1e-3) / 1e12,
-        'gemm_launches': len(gemm_events),
-    }
 
 
 def _time_gpu(fn, iters, warm=3):
@@ -138,15 +63,206 @@ def _time_gpu(fn, iters, warm=3):
     return s.elapsed_time(e) / iters
 
 
-def bench_cast(iters=20):
-    """cast+amax throughput: C1 (fp32 [4096,4096], in-time, E4M3), steady-state delayed cast of bf16
-    [8192,4096], and the in-time cast of one Llama-70B MLP weight (bf16 [28672,8192])."""
+# ---- synthetic inputs (bench-local: the GPU legs import nothing from tests/ or oracle/) ---------------------------
+def c1_input(seed=0, n_rows=4096, n_cols=4096):
+    """Config 1: fp32 N(0,1) with 0.1 % of the entries (uniformly chosen) multiplied by 100.  On the CPU."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(n_rows, n_cols, generator=g)
+    idx = torch.randperm(x.numel(), generator=g)[:x.numel() // 1000]
+    x.view(-1)[idx] *= 100
+    return x
+
+
+def new_meta(window=1):
+    """Device-side (scale, scale_inv, amax) as the C ABI wants them."""
+    import torch
+    return torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(window, device='cuda')
+
+
+def fp8_randn(shape, std, fp8_dt, seed):
+    """N(0, std) drawn on the GPU in bf16 and cast to FP8 in-time; returns (payload, scale_inv)."""
     import torch
     from msamp import _backend
-    from tests.gpu_util import c1_input, make_meta
+    g = torch.Generator(device='cuda').manual_seed(seed)
+    x = torch.randn(shape, device='cuda', dtype=torch.bfloat16, generator=g)
+    if std != 1.0:
+        x *= std
+    s, si, am = new_meta()
+    q = _backend.cast_to_fp8_intime(x, s, am, si, fp8_dt)
+    return q, si
+
+
+# ---- FP8Linear steps through the msamp API -------------------------------------------------------------------
+def bench_layer(cfg, steps, warmup):
+    """Forward + backward of every projection of `cfg` as FP8Linear modules, then the amax-window update."""
+    import torch
+    import msamp    # noqa: F401
+    from msamp import _backend
+    from msamp.common.dtype import Dtypes
+    from msamp.nn import LinearReplacer, model_state
+    from msamp.optim import LBAdamW
+    import msamp.operators.gemm.gemm as gemm_mod
+
+    tokens = cfg['tokens']
+    g = torch.Generator(device='cuda').manual_seed(0)
+    layers = torch.nn.ModuleList()
+    inputs, ograds = {}, []
+    flops = 0.0
+    for _, d_out, d_in in cfg['proj']:
+        lin = torch.nn.Linear(d_in, d_out, bias=False, device='cuda', dtype=torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.copy_(torch.randn(d_out, d_in, device='cuda', generator=g) * 0.02)
+        layers.append(lin)
+        if d_in not in inputs:
+            inputs[d_in] = torch.randn(tokens, d_in, device='cuda', generator=g).bfloat16().requires_grad_(True)
+        ograds.append((torch.randn(tokens, d_out, device='cuda', generator=g) * 1e-3).bfloat16())
+        flops += 3 * 2.0 * tokens * d_in * d_out
+    model_state.clear()
+    model = LinearReplacer.replace(layers, Dtypes.kbfloat16)
+    opt = LBAdamW(model.parameters())    # only its scaling-factor update runs here
+
+    gemm_events = []
+    real_gemm, real_gemm_cast = _backend.fp8_gemm, _backend.fp8_gemm_cast
+
+    class _Timed:
+        enabled = False
+
+        @staticmethod
+        def _flops(a, out, a_kmajor):
+            return 2.0 * out.numel() * (a.shape[0] if a_kmajor else a.shape[1])
+
+        @staticmethod
+        def fp8_gemm(a, a_dt, a_si, b, b_dt, b_si, out, accumulate=False, bias=None, a_kmajor=False, b_kmajor=False):
+            if not _Timed.enabled:
+                return real_gemm(a, a_dt, a_si, b, b_dt, b_si, out, accumulate, bias, a_kmajor=a_kmajor, b_kmajor=b_kmajor)
+            s, e = _events()
+            s.record()
+            real_gemm(a, a_dt, a_si, b, b_dt, b_si, out, accumulate, bias, a_kmajor=a_kmajor, b_kmajor=b_kmajor)
+            e.record()
+            gemm_events.append((s, e, _Timed._flops(a, out, a_kmajor)))
+            return out
+
+        @staticmethod
+        def fp8_gemm_cast(a, *args, **kwargs):
+            # the weight-gradient GEMM with its cast to E4M3 fused in: one launch, timed as the GEMM it is
+            if not _Timed.enabled:
+                return real_gemm_cast(a, *args, **kwargs)
+            s, e = _events()
+            s.record()
+            out = real_gemm_cast(a, *args, **kwargs)
+            e.record()
+            if out is not None:
+                gemm_events.append((s, e, _Timed._flops(a, out, kwargs.get('a_kmajor', False))))
+            return out
+
+        def __getattr__(self, name):
+            return getattr(_backend, name)
+
+    gemm_mod._backend = _Timed()
+
+    def step():
+        for lin, dy in zip(model, ograds):
+            x = inputs[lin.in_features]
+            lin(x).backward(dy)
+            lin.weight.grad = None
+            x.grad = None
+        opt._update_scaling_factors()
+
+    try:
+        for _ in range(SCALING_WARMUP_STEPS):    # untimed set-up: fill the amax windows
+            step()
+        assert not model[0].scaling_metas['input'].is_in_time_scaling()
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            # an event pair costs the stream a few microseconds: bracket the GEMMs of every fourth step only
+            _Timed.enabled = i % GEMM_EVENT_STRIDE == 0
+            step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    finally:
+        _Timed.enabled = False
+        gemm_mod._backend = _backend
+        model_state.clear()
+
+    ms_per_step = dt / steps * 1e3
+    gemm_ms_total = sum(s.elapsed_time(e) for s, e, _ in gemm_events)
+    gemm_flops_total = sum(f for _, _, f in gemm_events)
+    return {
+        'ms_per_step': ms_per_step,
+        'step_tflops': flops / (ms_per_step * 1e-3) / 1e12,
+        'gemm_tflops': gemm_flops_total / (gemm_ms_total * 1e-3) / 1e12,
+        'gemm_avg_launch_ms': gemm_ms_total / len(gemm_events),
+        'gemm_avg_launch_flops': gemm_flops_total / len(gemm_events),
+        'gemm_launches': len(gemm_events),
+        'gemms_per_step': 3 * len(cfg['proj']),
+    }
+
+
+# ---- GEMM sweep: one row per projection and pass, straight through the C ABI -------------------------------------
+def bench_gemm_sweep(cfg, iters=10, accumulate_row=None):
+    """Forward (E4M3 x E4M3), dgrad (W K-major, dy E5M2) and wgrad (x and dy K-major) of every projection, bf16
+    out, operands drawn as the configs describe them and cast to FP8 by the library."""
+    import torch
+    from msamp import _backend
+    E4, E5 = _backend.DT_E4M3, _backend.DT_E5M2
+    tokens = cfg['tokens']
+    rows, seen = [], {}
+    acts = {}
+    for name, d_out, d_in in cfg['proj']:
+        if (d_out, d_in) in seen:    # gate and up: same problem, measured once, counted twice in the aggregate
+            for r in seen[(d_out, d_in)]:
+                rows.append(dict(r, proj=name))
+            continue
+        if d_in not in acts:
+            acts[d_in] = fp8_randn((tokens, d_in), 1.0, E4, seed=d_in)
+        x, x_si = acts[d_in]
+        w, w_si = fp8_randn((d_out, d_in), 0.02, E4, seed=d_out + 1)
+        dy, dy_si = fp8_randn((tokens, d_out), 1e-3, E5, seed=d_out + 2)
+        y = torch.empty(tokens, d_out, dtype=torch.bfloat16, device='cuda')
+        dx = torch.empty(tokens, d_in, dtype=torch.bfloat16, device='cuda')
+        dw = torch.empty(d_out, d_in, dtype=torch.bfloat16, device='cuda')
+        passes = [
+            ('fwd', lambda: _backend.fp8_gemm(w, E4, w_si, x, E4, x_si, y), (d_out, tokens, d_in)),
+            ('dgrad', lambda: _backend.fp8_gemm(w, E4, w_si, dy, E5, dy_si, dx, a_kmajor=True), (d_in, tokens, d_out)),
+            ('wgrad', lambda: _backend.fp8_gemm(x, E4, x_si, dy, E5, dy_si, dw, a_kmajor=True, b_kmajor=True),
+             (d_in, d_out, tokens)),
+        ]
+        if accumulate_row == name:
+            passes.append(('wgrad_accumulate',
+                           lambda: _backend.fp8_gemm(x, E4, x_si, dy, E5, dy_si, dw, accumulate=True, a_kmajor=True, b_kmajor=True),
+                           (d_in, d_out, tokens)))
+        mine = []
+        for pname, fn, (m, n, k) in passes:
+            ms = _time_gpu(fn, iters)
+            fl = 2.0 * m * n * k
+            tf = fl / (ms * 1e-3) / 1e12
+            mine.append({'proj': name, 'pass': pname, 'm': m, 'n': n, 'k': k, 'ms': round(ms, 4), 'tflops': round(tf, 1),
+                         'frac_mfma': round(tf / FP8_PEAK_TFLOPS, 4)})
+        seen[(d_out, d_in)] = mine
+        rows.extend(mine)
+        del w, dy, y, dx, dw
+    core = [r for r in rows if r['pass'] in ('fwd', 'dgrad', 'wgrad')]
+    fl = sum(2.0 * r['m'] * r['n'] * r['k'] for r in core)
+    ms = sum(r['ms'] for r in core)
+    agg = fl / (ms * 1e-3) / 1e12
+    return {'rows': rows, 'aggregate': {'flops': fl, 'ms': round(ms, 3), 'tflops': round(agg, 1),
+                                        'frac_mfma': round(agg / FP8_PEAK_TFLOPS, 4), 'gemms': len(core)}}
+
+
+# ---- cast group ----------------------------------------------------------------------------------------------
+def bench_cast(iters=20):
+    """cast+amax throughput: C1 (fp32 [4096,4096], in-time, E4M3 / E5M2, dequantize), steady-state delayed cast of
+    bf16 [8192,4096], and the in-time cast of one Llama-70B MLP weight (bf16 [28672,8192], N(0,0.01) with 0.01 %
+    outliers x 50) and of the whole layer's 855 638 016 weight elements."""
+    import torch
+    from msamp import _backend
     out = {}
     x = c1_input(0).cuda()
-    s, si, am = make_meta()
+    s, si, am = new_meta()
     ms = _time_gpu(lambda: _backend.cast_to_fp8_intime(x, s, am[0:1], si, _backend.DT_E4M3), iters)
     out['c1_intime_fp32_e4m3'] = {'ms': ms, 'GBps': x.numel() * 5 / ms / 1e6}
     ms = _time_gpu(lambda: _backend.cast_to_fp8_intime(x, s, am[0:1], si, _backend.DT_E5M2), iters)
@@ -175,10 +291,28 @@ def bench_cast(iters=20):
     ms = _time_gpu(lambda: _backend.fp8_transpose(qa), iters)
     out['c2_fp8_transpose'] = {'ms': ms, 'GBps': a.numel() * 2 / ms / 1e6}
     del a, qa
-    w = (torch.randn(28672, 8192, device='cuda') * 0.01).bfloat16()
+
+    def c5_weight(d_out, d_in, seed):
+        g = torch.Generator(device='cuda').manual_seed(seed)
+        w = torch.randn(d_out, d_in, device='cuda', generator=g) * 0.01
+        idx = torch.randint(0, w.numel(), (w.numel() // 10000, ), device='cuda', generator=g)
+        w.view(-1)[idx] *= 50
+        return w.bfloat16()
+
+    weights = [c5_weight(d_out, d_in, 100 + i) for i, (_, d_out, d_in) in enumerate(LLAMA_70B['proj'])]
+    metas = [new_meta() for _ in weights]
+    w = weights[2]    # gate: [28672, 8192], 234 881 024 elements
     ms = _time_gpu(lambda: _backend.cast_to_fp8_intime(w, s, am[0:1], si, _backend.DT_E4M3), max(iters // 2, 5))
     out['c5_intime_bf16_e4m3_235M'] = {'ms': ms, 'GBps': w.numel() * 3 / ms / 1e6}
-    del w
+
+    def layer_cast():
+        for wt, (ws, wsi, wam) in zip(weights, metas):
+            _backend.cast_to_fp8_intime(wt, ws, wam[0:1], wsi, _backend.DT_E4M3)
+
+    n_layer = sum(wt.numel() for wt in weights)
+    ms = _time_gpu(layer_cast, 5, warm=2)
+    out['c5_intime_bf16_e4m3_layer_856M'] = {'ms': ms, 'GBps': n_layer * 3 / ms / 1e6}
+    del w, weights
     # what a plain copy reaches on this box (the practical ceiling of the streaming kernels above): 256 MiB of
     # fp32 through the library's scale_cast at scale 1, read once, written once
     src = torch.ones(64 * 1024 * 1024, device='cuda')
@@ -200,7 +334,7 @@ def bench_grad_side(iters=10):
     bucket = GradientBucket([n] * len(grads))
     out = {}
     ms = _time_gpu(lambda: bucket.quantize(grads, world_size=8), iters)
-    out['bucket_quantize_32x4M_bf16'] = {'ms': ms, 'GBps': n * len(grads) * 5 / ms / 1e6}
+    out['bucket_quantize_32x4M_bf16'] = {'ms': ms, 'GBps': n * len(grads) * 3 / ms / 1e6}
     del grads, bucket
     qs = [torch.randint(0, 120, (n,), dtype=torch.uint8, device='cuda') for _ in range(64)]
     sis = [torch.ones((), device='cuda') for _ in qs]
@@ -225,13 +359,13 @@ def bench_adam(iters=5, total_params=1_000_000_000):
         g = (torch.randn(n, device='cuda') * 1e-3)
         d = {}
         for name, src, dt in (('w', w, _backend.DT_E4M3), ('g', g, _backend.DT_E5M2)):
-            s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+            s, si, am = new_meta()
             d[name] = (_backend.cast_to_fp8_intime(src, s, am, si, dt), s, si, am)
         m = (torch.randn(n, device='cuda') * 1e-4).abs_()
-        s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+        s, si, am = new_meta()
         d['m'] = (_backend.cast_to_fp8_intime(m, s, am, si, _backend.DT_E4M3), s, si, am)
         v = (torch.randn(n, device='cuda') * 1e-4).abs_()
-        s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+        s, si, am = new_meta()
         _backend.amax(v, am)
         s.copy_(_backend.compute_scaling_factor(am, s.reshape(1), 65504.0, 0)[0])
         si.copy_(1.0 / s)
@@ -259,12 +393,13 @@ def bench_adam(iters=5, total_params=1_000_000_000):
             'tensors': len(sizes), 'params': total_params}
 
 
+# ---- CPU baseline: the oracle on the host cores --------------------------------------------------------------
 def cpu_baseline():
-    """The oracle (PyTorch CPU restatement of the reference math) on a bounded sample, all host cores."""
+    """The oracle (PyTorch CPU restatement of the reference math) on a bounded sample, all host cores: the
+    config-1 cast at full size, the config-3 AdamW step on 16 of its [4096,1024] tensors, the config-5 cast of one
+    [28672,8192] weight, and the GEMM definition (fp32 matmul of dequantized operands) on a slice of config 2."""
     import torch
     from oracle import adamw as oadam, cast as ocast, fp8
-    from tests.gpu_util import c1_input
-    from tests.test_gpu_adam import _inputs
     # the box sets OMP_NUM_THREADS to its CPU share; never spread over more threads than that
     cores = min(os.cpu_count() or 1, int(os.environ.get('OMP_NUM_THREADS', '16') or 16))
     torch.set_num_threads(cores)
@@ -282,8 +417,26 @@ def cpu_baseline():
     x = c1_input(0)
     t = med(lambda: ocast.cast_to_fp8(x, ocast.new_meta(), fp8.E4M3, in_time=True))
     cast_gbps = x.numel() * 5 / t / 1e9
+    del x
+
     n = 4096 * 1024
-    tens = [_inputs(n, i, fp8.E4M3, fp8.E5M2) for i in range(2)]
+    n_tensors = 16
+
+    def adam_inputs(seed):
+        g = torch.Generator().manual_seed(seed)
+
+        def quant(v, fmt):
+            meta = ocast.new_meta()
+            return ocast.cast_to_fp8(v, meta, fmt, in_time=True), meta
+
+        w, wm = quant(0.02 * torch.randn(n, generator=g), fp8.E4M3)
+        gq, gm = quant(1e-3 * torch.randn(n, generator=g), fp8.E5M2)
+        m, mm = quant((1e-4 * torch.randn(n, generator=g)).abs(), fp8.E4M3)
+        vm = ocast.new_meta()
+        v = ocast.cast_to_fp16((1e-4 * torch.randn(n, generator=g)).abs(), vm, in_time=True)
+        return dict(w=w, wm=wm, g=gq, gm=gm, m=m, mm=mm, v=v, vm=vm)
+
+    tens = [adam_inputs(i) for i in range(n_tensors)]
 
     def adam():
         for d in tens:
@@ -291,18 +444,31 @@ def cpu_baseline():
                               lr=3e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=2)
 
     ta = med(adam, runs=3, warm=1)
-    adam_gps = len(tens) * n / ta / 1e9
-    # GEMM definition (fp32 matmul of dequantized operands) on 1024 of the 8192 token rows
+    adam_gps = n_tensors * n / ta / 1e9
+    del tens
+
+    g = torch.Generator().manual_seed(5)
+    w5 = torch.randn(28672, 8192, generator=g) * 0.01
+    idx = torch.randint(0, w5.numel(), (w5.numel() // 10000, ), generator=g)
+    w5.view(-1)[idx] *= 50
+    w5 = w5.bfloat16()
+    t5 = med(lambda: ocast.cast_to_fp8(w5, ocast.new_meta(), fp8.E4M3, in_time=True), runs=3, warm=1)
+    c5_gbps = w5.numel() * 3 / t5 / 1e9
+    del w5
+
+    # GEMM definition (fp32 matmul of dequantized operands) on 1024 of the 8192 token rows of config 2
     a = fp8.decode(fp8.encode(torch.randn(4096, 4096) * 0.02 * 64, fp8.E4M3), fp8.E4M3)
     b = fp8.decode(fp8.encode(torch.randn(1024, 4096), fp8.E4M3), fp8.E4M3)
     tg = med(lambda: b @ a.t(), runs=5, warm=1)
     gemm_tflops = 2.0 * 1024 * 4096 * 4096 / tg / 1e12
     return {
         'value': gemm_tflops, 'unit': 'TFLOP/s', 'cores': cores, 'threads': torch.get_num_threads(), 'kind': 'port',
-        'sample': 'fp32 matmul of dequantized operands, 1024 of 8192 token rows of the forward GEMM; '
-                  'cast: full config-1 tensor fp32[4096,4096] in-time E4M3; adam: 2 of 239 tensors [4096,1024]',
-        'cast_amax': {'value': cast_gbps, 'unit': 'GB/s (5 B/elt)'},
-        'fp8_adam': {'value': adam_gps, 'unit': 'Gparams/s'},
+        'sample': 'gemm: fp32 matmul of dequantized operands, 1024 of the 8192 token rows of the config-2 forward GEMM; '
+                  'cast: full config-1 tensor fp32[4096,4096] in-time E4M3 (median of 5) and one config-5 weight '
+                  'bf16[28672,8192] (median of 3); adam: 16 of the 239 config-3 tensors [4096,1024] (median of 3)',
+        'cast_amax': {'value': cast_gbps, 'unit': 'GB/s (5 B/elt, config 1)'},
+        'cast_amax_c5': {'value': c5_gbps, 'unit': 'GB/s (3 B/elt, config 5 weight)'},
+        'fp8_adam': {'value': adam_gps, 'unit': 'Gparams/s', 'tensors': n_tensors},
     }
 
 
@@ -318,23 +484,30 @@ def pmc_calibration_copy():
 
 
 def measured_gemm_traffic():
-    """HBM bytes per GEMM launch as last measured with rocprofv3 --pmc (profiles/fp8_gemm_hbm_traffic.json),
-    or None when no measurement is on file."""
-    path = os.path.join(ROOT, 'profiles', 'fp8_gemm_hbm_traffic.json')
+    """(HBM bytes per GEMM launch of the headline step, where the figure comes from): the last rocprofv3 --pmc
+    measurement on file under profiles/ -- a static figure, not taken in this run -- or (None, None)."""
+    name = 'fp8_gemm_hbm_traffic.json'
     try:
-        with open(path) as f:
-            return json.load(f)['traffic_bytes_per_launch']
+        with open(os.path.join(ROOT, 'profiles', name)) as f:
+            return json.load(f)['traffic_bytes_per_launch'], 'profiles/%s (static: measured with rocprofv3 --pmc, not in this run)' % name
     except (OSError, KeyError, ValueError):
-        return None
+        return None, None
+
+
+def _round_kernels(d):
+    return {k: {'ms': round(v['ms'], 4), 'GBps': round(v['GBps'], 1), 'frac_hbm': round(v['GBps'] / HBM_PEAK_GBS, 4)}
+            for k, v in d.items()}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--skip-cpu', action='store_true', help='leave out the CPU-oracle baseline')
-    ap.add_argument('--skip-extra', action='store_true', help='leave out the cast and Adam kernel sections')
+    ap.add_argument('--skip-extra', action='store_true', help='leave out the sweep, cast and Adam kernel sections')
+    ap.add_argument('--only', choices=('gemm_c4', 'gemm_c5', 'cast', 'adam'), default=None,
+                    help='run one kernel section alone (after the calibration copy), for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)', file=sys.stderr)
@@ -346,30 +519,61 @@ def main():
     torch.cuda.set_device(0)
 
     pmc_calibration_copy()
-    lin = bench_fp8linear(args.steps, args.warmup)
+    if args.only:
+        if args.only == 'gemm_c4':
+            out = bench_gemm_sweep(LLAMA_7B, iters=3, accumulate_row='gate')
+        elif args.only == 'gemm_c5':
+            out = bench_gemm_sweep(LLAMA_70B, iters=3)
+        elif args.only == 'cast':
+            out = _round_kernels(bench_cast())
+        else:
+            out = bench_adam()
+        print(json.dumps({'only': args.only, 'result': out}))
+        return
+
+    lin = bench_layer(LLAMA_7B, args.steps, args.warmup)
+    traffic, traffic_source = measured_gemm_traffic()
     result = {
         'metric': 'FP8 GEMM TFLOPS, cast+amax GB/s, FP8-Adam Gparams/s on 1 MI355X',
         'value': lin['step_tflops'],
-        'unit': 'TFLOP/s (3 GEMMs of one FP8Linear fwd+bwd / whole step incl. casts and window update)',
+        'unit': 'TFLOP/s (15 GEMMs of one Llama-7B layer of FP8Linear fwd+bwd / whole step incl. casts and window update)',
         'n_gpus': 1,
         'steps': args.steps,
-        'warmup': max(args.warmup, 17),
+        'warmup': args.warmup,
         'ms_per_step': lin['ms_per_step'],
         'higher_is_better': True,
         'scaling': 'weak',
         'vs_baseline': None,
         'dtype': 'fp8 (e4m3 x e4m3 / e4m3 x e5m2), fp32 accumulate',
         'data': 'synthetic',
-        'config': {'workload': 'single FP8Linear fwd+bwd, x bf16[8192,4096], W bf16[4096,4096], dy bf16[8192,4096], '
-                               'delayed scaling (history 16), outputs bf16, dW -> E4M3'},
+        'config': {'workload': 'config 4: Llama-7B layer, every FP8Linear GEMM fwd+bwd at 16384 tokens (QKV [12288,4096], '
+                               'O [4096,4096], gate/up [11008,4096], down [4096,11008]); x, dy bf16, W bf16 payload, delayed '
+                               'scaling (history 16) after %d untimed scaling warm-up steps, outputs bf16, dW -> E4M3'
+                               % SCALING_WARMUP_STEPS},
         'roofline': {
-            'kernel': 'fp8_gemm_dma_kernel', 'bound': 'mfma', 'achieved': lin['gemm_tflops'], 'peak': FP8_PEAK_TFLOPS,
-            'unit': 'TFLOP/s', 'frac': lin['gemm_tflops'] / FP8_PEAK_TFLOPS, 'traffic': measured_gemm_traffic(),
-            'avg_launch_ms': lin['gemm_ms'], 'launches': lin['gemm_launches'],
+            'kernel': 'fp8_gemm_dma_kernel (flop-weighted over the 15 GEMM launches of the config-4 step)',
+            'bound': 'mfma', 'achieved': lin['gemm_tflops'], 'peak': FP8_PEAK_TFLOPS, 'unit': 'TFLOP/s',
+            'frac': lin['gemm_tflops'] / FP8_PEAK_TFLOPS, 'traffic': traffic, 'traffic_source': traffic_source,
+            'avg_launch_ms': lin['gemm_avg_launch_ms'], 'avg_launch_flops': lin['gemm_avg_launch_flops'],
+            'launches': lin['gemm_launches'],
         },
     }
     if not args.skip_extra:
+        torch.cuda.empty_cache()
+        c2 = bench_layer(CONFIG_2, max(args.steps, 200), args.warmup)
+        result['c2_step'] = {
+            'workload': 'config 2: single FP8Linear fwd+bwd, x bf16[8192,4096], W bf16[4096,4096], dy bf16[8192,4096]',
+            'ms_per_step': round(c2['ms_per_step'], 4), 'step_tflops': round(c2['step_tflops'], 1),
+            'gemm_tflops': round(c2['gemm_tflops'], 1), 'gemm_frac_mfma': round(c2['gemm_tflops'] / FP8_PEAK_TFLOPS, 4),
+            'gemm_avg_launch_ms': round(c2['gemm_avg_launch_ms'], 4), 'gemm_launches': c2['gemm_launches'],
+        }
+        torch.cuda.empty_cache()
+        result['gemm_sweep'] = {'c4_llama7b': bench_gemm_sweep(LLAMA_7B, accumulate_row='gate')}
+        torch.cuda.empty_cache()
+        result['gemm_sweep']['c5_llama70b'] = bench_gemm_sweep(LLAMA_70B, iters=5)
+        torch.cuda.empty_cache()
         cast = bench_cast()
+        torch.cuda.empty_cache()
         adam = bench_adam()
         torch.cuda.empty_cache()
         grad_side = bench_grad_side()
@@ -377,14 +581,12 @@ def main():
         result['cast_amax_GBps'] = cast['c1_intime_fp32_e4m3']['GBps']
         result['fp8_adam_Gparams_per_s'] = adam['Gparams_per_s']
         result['kernels'] = {
-            'cast': {k: {'ms': round(v['ms'], 4), 'GBps': round(v['GBps'], 1), 'frac_hbm': round(v['GBps'] / HBM_PEAK_GBS, 4)}
-                     for k, v in cast.items()},
+            'cast': _round_kernels(cast),
             'fused_adamw': {'ms': round(adam['ms'], 3), 'Gparams_per_s': round(adam['Gparams_per_s'], 1),
                             'GBps': round(adam['GBps_algorithmic'], 1),
                             'frac_hbm': round(adam['GBps_algorithmic'] / HBM_PEAK_GBS, 4), 'params': adam['params'],
                             'tensors': adam['tensors']},
-            'grad_side': {k: {'ms': round(v['ms'], 4), 'GBps': round(v['GBps'], 1),
-                              'frac_hbm': round(v['GBps'] / HBM_PEAK_GBS, 4)} for k, v in grad_side.items()},
+            'grad_side': _round_kernels(grad_side),
         }
     if not args.skip_cpu:
         result['cpu_baseline'] = cpu_baseline()
