@@ -88,6 +88,17 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
                              uint8_t* out, int fp8_type, int margin, int flags, void* workspace,
                              msamp_stream_t stream);
 
+/* msamp_cast_to_fp8_intime without the workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): it has no counterpart in
+ * the reference.  The MSAMP_WORKSPACE_BYTES of scratch live in a static device array inside the library (each GPU
+ * the library runs on holds its own copy until the process ends); the call allocates and frees nothing.  Same
+ * kernels and same results as msamp_cast_to_fp8_intime.  n above MSAMP_STATIC_MAX_ELEMS is rejected with
+ * MSAMP_ERR_SHAPE.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race on it -- order them on one stream. */
+#define MSAMP_STATIC_MAX_ELEMS ((size_t)1 << 32)
+int msamp_cast_to_fp8_intime_static(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
+                                    uint8_t* out, int fp8_type, int margin, int flags, msamp_stream_t stream);
+
 /* ScalingTensor.cast from a scaled 16/32-bit payload to FP8 (msamp/common/tensor/tensor.py:223-265):
  * x holds value * old_scale and *amax = max|value| is known, so no reduction is needed:
  * s = rule(amax[0], 1, fp_max(fp8_type), margin); out[i] = fp8_sat_rne(float(x[i]) * (s * *old_scale_inv));

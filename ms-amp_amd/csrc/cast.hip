@@ -1198,6 +1198,34 @@ static int launch_add_to_fp8(uint8_t* q, int fp8_type, const IT* other, size_t n
     return MSAMP_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Workspace of msamp_cast_to_fp8_intime_static: the same MSAMP_WORKSPACE_BYTES the other in-time entry points
+// are handed by their caller, but owned by the library, so that the call needs no allocation anywhere.  Every
+// GPU holds its own copy of the array at its own address; host code never uses the array's name as a pointer,
+// only the address hipGetSymbolAddress reports for the device that is current.
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[MSAMP_WORKSPACE_BYTES];
+
+static int static_workspace(void** ws) {
+    static std::mutex mu;
+    static void* ptrs[64];
+    static bool known[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    MSAMP_REQUIRE(dev >= 0 && dev < 64, MSAMP_ERR_SHAPE, "msamp_cast_to_fp8_intime_static: device index %d", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!known[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        MSAMP_REQUIRE(p != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_to_fp8_intime_static: no address for the static workspace");
+        ptrs[dev] = p;
+        known[dev] = true;
+    }
+    *ws = ptrs[dev];
+    return MSAMP_OK;
+}
+
 }    // namespace msamp
 
 using namespace msamp;
@@ -1250,6 +1278,20 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
     if (rc != MSAMP_OK) return rc;
     const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags, nullptr, nullptr, nullptr, 0, nullptr};
     return dispatch_cast(x, in_dtype, n, scale, nullptr, scale_inv, out, fp8_type, &it, st);
+}
+
+int msamp_cast_to_fp8_intime_static(const void* x, int in_dtype, size_t n, float* scale, float* amax, float* scale_inv,
+                                    uint8_t* out, int fp8_type, int margin, int flags, msamp_stream_t stream) {
+    MSAMP_REQUIRE(n <= MSAMP_STATIC_MAX_ELEMS, MSAMP_ERR_SHAPE,
+                  "msamp_cast_to_fp8_intime_static: n=%zu exceeds the limit of %llu elements", n,
+                  static_cast<unsigned long long>(MSAMP_STATIC_MAX_ELEMS));
+    void* ws = nullptr;
+    const int rc = static_workspace(&ws);
+    if (rc != MSAMP_OK) return rc;
+    // Nothing in the workspace has to start at zero for this path: the header words and the partial maxima are
+    // rewritten by every call's first kernel before its second reads them, and the slots through which the
+    // one-pass kernel's workgroups meet are tagged with a token that is new for every call.
+    return msamp_cast_to_fp8_intime(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, stream);
 }
 
 int msamp_cast_scaled_to_fp8(const void* x, int in_dtype, size_t n, const float* amax, const float* old_scale_inv,

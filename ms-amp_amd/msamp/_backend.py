@@ -34,6 +34,7 @@ _SIGNATURES = {
     'msamp_compute_scaling_factor': ([_vp, _vp, _i, _vp, _i, _f, _i, _vp], _i),
     'msamp_cast_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp], _i),
     'msamp_cast_to_fp8_intime': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp], _i),
+    'msamp_cast_to_fp8_intime_static': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _i, _i, _vp], _i),
     'msamp_cast_scaled_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp], _i),
     'msamp_add_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp, _vp], _i),
     'msamp_cast_from_fp8': ([_vp, _i, _sz, _vp, _vp, _i, _vp], _i),
@@ -222,6 +223,26 @@ def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_
             _ptr(workspace(x.device)),
             _stream()
         ), 'msamp_cast_to_fp8_intime'
+    )
+    return out
+
+
+STATIC_MAX_ELEMS = 1 << 32
+
+
+def cast_to_fp8_intime_static(x, scale, amax_cell, scale_inv, out, fp8_dt, margin=0, nan_to_inf=False, two_pass=False):
+    """cast_to_fp8_intime into the caller's `out`, with the library's own static workspace: the call allocates
+    nothing (for callers that cannot allocate).  Calls on one GPU must not overlap in time."""
+    lib = load()
+    _gpu(x, 'input')
+    _gpu(out, 'output')
+    if out.dtype != torch.uint8 or out.numel() != x.numel() or not out.is_contiguous():
+        raise ValueError('out must be a contiguous uint8 tensor with as many elements as the input')
+    _check(
+        lib.msamp_cast_to_fp8_intime_static(
+            _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _shared_device() else 0), _stream()
+        ), 'msamp_cast_to_fp8_intime_static'
     )
     return out
 
