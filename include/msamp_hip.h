@@ -43,6 +43,7 @@ enum {
     MSAMP_ERR_SHAPE = -2,     /* bad size, shape or alignment          */
     MSAMP_ERR_NULL = -3,      /* required pointer is NULL              */
     MSAMP_ERR_WORKSPACE = -4, /* workspace missing or too small        */
+    MSAMP_ERR_TIMEOUT = -5,   /* a kernel's bounded wait ran out (msamp_check_async_error) */
     MSAMP_ERR_HIP = -100      /* -100 - hipError_t of the failing call */
 };
 
@@ -60,6 +61,19 @@ enum {
 
 int msamp_hip_version(void);
 const char* msamp_last_error(void);
+
+/* The one-pass in-time cast and the fused GEMM + cast are kernels whose workgroups wait for each other, with a bounded
+ * wait.  A wait that runs out cannot be reported by the call that enqueued the kernel: the kernel then leaves a sticky
+ * non-zero code in the workspace (and a NaN amax when the collecting workgroup gave up), and this call reports it.  It
+ * copies the word to the host -- it SYNCHRONISES `stream` -- and returns MSAMP_OK, or MSAMP_ERR_TIMEOUT after clearing
+ * the word; the tensor and meta written by the failed kernel are invalid then, and the caller repeats the operation with
+ * MSAMP_FLAG_TWO_PASS.  No counterpart in the reference (its casts have no such kernels). */
+int msamp_check_async_error(void* workspace, msamp_stream_t stream);
+
+/* Number of polls after which the collecting workgroup of such a kernel gives up (default 2^20, a fraction of a second;
+ * the other workgroups wait four times as long for its post).  0 makes every wait give up at once without polling: a
+ * hook for testing the failure path with kernels that still exit normally. */
+void msamp_set_spin_limit(uint32_t polls);
 
 /* amax[0] = max|x| over n elements, NaN propagating (torch abs().max(), cast.py:34).
  * dtype: F32/F16/BF16.  workspace: MSAMP_WORKSPACE_BYTES. */

@@ -54,6 +54,10 @@ bool waiting_kernels_allowed(hipStream_t st) {
     return hipStreamIsCapturing(st, &capture) == hipSuccess && capture == hipStreamCaptureStatusNone;
 }
 
+static std::atomic<uint32_t> g_spin_limit{1u << 20};    // a fraction of a second of polling
+
+uint32_t collector_spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
+
 uint32_t next_tokens(uint32_t count) {
     for (;;) {
         const uint32_t first = g_token.fetch_add(count) + 1;
@@ -68,5 +72,27 @@ extern "C" {
 int msamp_hip_version(void) { return 100; }
 
 const char* msamp_last_error(void) { return msamp::g_err; }
+
+void msamp_set_spin_limit(uint32_t polls) { msamp::g_spin_limit.store(polls, std::memory_order_relaxed); }
+
+int msamp_check_async_error(void* workspace, msamp_stream_t stream) {
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_check_async_error: workspace required");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint32_t* word = static_cast<uint32_t*>(workspace) + msamp::kWsErrorWord;
+    uint32_t code = 0;
+    hipError_t e = hipMemcpyAsync(&code, word, sizeof(code), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return msamp::hip_fail(e, "msamp_check_async_error: reading the error word");
+    if (code == 0) return MSAMP_OK;
+    const uint32_t zero = 0;
+    e = hipMemcpyAsync(word, &zero, sizeof(zero), hipMemcpyHostToDevice, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return msamp::hip_fail(e, "msamp_check_async_error: clearing the error word");
+    msamp::set_error("a kernel whose workgroups wait for each other gave up waiting (code %u: %s%s): the tensor and meta it "
+                     "wrote are invalid; repeat the call with MSAMP_FLAG_TWO_PASS",
+                     code, (code & msamp::kErrCollectorGaveUp) ? "collecting workgroup " : "",
+                     (code & msamp::kErrFollowerGaveUp) ? "waiting workgroup" : "");
+    return MSAMP_ERR_TIMEOUT;
+}
 
 }    // extern "C"

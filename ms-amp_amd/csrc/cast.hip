@@ -288,7 +288,7 @@ __global__ __launch_bounds__(kCastThreads) void amax_finalize_kernel(const uint3
 // the way; every workgroup then derives the same scale by itself.  Tokens come from a host counter,
 // so slots never need clearing.  All workgroups must be resident together: the host launches at most
 // two per CU and keeps the kernel to one stream per device; the wait is bounded all the same, and a
-// wait that runs out reports NaN as the amax.
+// wait that runs out sets the workspace's sticky error word (and, when it is workgroup 0's, NaN as the amax).
 constexpr int kResThreads = 512;
 constexpr int kResVecs = 16;
 constexpr int kResBlocksPerCu = 2;
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
                                                                            float* scale, float* amax, float* scale_inv,
                                                                            uint64_t* slots, float fp_max, int margin,
                                                                            int flags, int rounds, uint32_t token,
-                                                                           uint32_t spin_limit) {
+                                                                           uint32_t spin_limit, uint32_t* error_word) {
     constexpr int EPT = 16 / sizeof(IT);
     using Raw = typename std::conditional<sizeof(IT) == 4, uint32_t, uint16_t>::type;
     __shared__ uint32_t red[kResThreads / kWave];
@@ -355,9 +355,9 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
         // token, in two words behind the slots; the others poll only those.
         uint64_t* post = slots + kMaxSlots;
         if (blockIdx.x == 0) {
-            uint32_t spins = 0, mm;
-            bool all_in;
-            do {
+            uint32_t mm = 0;
+            bool all_in = false;
+            for (uint32_t spins = 0; !all_in && spins < spin_limit; ++spins) {
                 // all slots of one poll are requested together; the ones past the grid are read and ignored
                 uint64_t sv[kMaxSlots / kWave];
 #pragma unroll
@@ -372,11 +372,17 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
                     mm = umax(mm, live ? static_cast<uint32_t>(sv[j]) : 0u);
                 }
                 all_in = __all(ok);
-            } while (!all_in && ++spins < spin_limit);
+            }
             mm = wave_max_u32(mm);
             if (tid == 0) {
                 float am = __uint_as_float(mm);
-                if (!all_in) am = __uint_as_float(0x7fc00000u);    // the wait ran out: make the failure visible
+                // The wait ran out: the amax becomes NaN, the rule then keeps the old scale, and both are still posted,
+                // so every workgroup that sees the post quantizes with one and the same scale; the sticky error word
+                // tells the host.
+                if (!all_in) {
+                    am = __uint_as_float(0x7fc00000u);
+                    report_wait_expired(error_word, kErrCollectorGaveUp);
+                }
                 else if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
                 const float s = scale_rule(am, old_scale, fp_max, margin);
                 const uint64_t tag = static_cast<uint64_t>(token) << 32;
@@ -389,14 +395,16 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
                 *scale_inv = 1.0f / s;
             }
         } else if (tid == 0) {
-            uint32_t spins = 0;
-            uint64_t pa, ps;
-            bool posted;
-            do {
+            // wait for workgroup 0's post, longer than it waits itself: it posts even when it gives up
+            uint64_t pa = 0, ps = 0;
+            bool posted = false;
+            const uint64_t follower_limit = static_cast<uint64_t>(spin_limit) * kFollowerSpinFactor;
+            for (uint64_t spins = 0; !posted && spins < follower_limit; ++spins) {
                 pa = __hip_atomic_load(post, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 ps = __hip_atomic_load(post + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 posted = static_cast<uint32_t>(pa >> 32) == token && static_cast<uint32_t>(ps >> 32) == token;
-            } while (!posted && ++spins < spin_limit);
+            }
+            if (!posted) report_wait_expired(error_word, kErrFollowerGaveUp);    // no post at all: NaN codes from here
             s_amax = posted ? static_cast<uint32_t>(pa) : 0x7fc00000u;
             s_scale = posted ? static_cast<uint32_t>(ps) : 0x7fc00000u;
         }
@@ -943,8 +951,8 @@ static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const flo
 // true if the runtime confirms kResBlocksPerCu workgroups of this kernel fit one CU (asked once per kernel)
 static bool fits_resident(const void* fn) {
     static std::mutex mu;
-    static const void* known[16];
-    static bool fits[16];
+    static const void* known[32];
+    static bool fits[32];
     static int n_known = 0;
     std::lock_guard<std::mutex> lock(mu);
     for (int i = 0; i < n_known; ++i)
@@ -952,7 +960,7 @@ static bool fits_resident(const void* fn) {
     int blocks = 0;
     const bool ok = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, fn, kResThreads, 0) == hipSuccess &&
                     blocks >= kResBlocksPerCu;
-    if (n_known < 16) {
+    if (n_known < 32) {
         known[n_known] = fn;
         fits[n_known++] = ok;
     }
@@ -971,7 +979,6 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
     if (max_blocks > static_cast<size_t>(kMaxSlots)) max_blocks = kMaxSlots;
     if (nvec == 0 || nvec > max_blocks * kResThreads * kResVecs) return 1;
     if (!waiting_kernels_allowed(st)) return 1;
-    if (!fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, MSAMP_DT_E4M3, kResVecs>))) return 1;
     // as many workgroups as there are runs of kResThreads vectors, up to the resident limit
     size_t g = (nvec + kResThreads - 1) / kResThreads;
     g = g > max_blocks ? max_blocks : g;
@@ -980,14 +987,21 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
     const uint32_t token = next_tokens(1);
     uint64_t* slots = reinterpret_cast<uint64_t*>(static_cast<char*>(ws) + kWsSlotBytes);
     const float fp_max = fp8_max(fp8_type);
-    const uint32_t spin_limit = 1u << 20;    // a fraction of a second of polling
+    const uint32_t spin_limit = collector_spin_limit();
+    uint32_t* error_word = static_cast<uint32_t*>(ws) + kWsErrorWord;
+    // the runtime must confirm, for the very instantiation that is launched, that kResBlocksPerCu workgroups fit a CU
+    bool fits = true;
 #define LAUNCH(FMT, R) \
-    hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT, R>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit)
+    do { \
+        fits = fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, FMT, R>)); \
+        if (fits) hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT, R>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit, error_word); \
+    } while (0)
 #define LAUNCH_R(FMT) \
     do { if (rounds <= 4) LAUNCH(FMT, 4); else if (rounds <= 8) LAUNCH(FMT, 8); else LAUNCH(FMT, kResVecs); } while (0)
     if (fp8_type == MSAMP_DT_E4M3) LAUNCH_R(MSAMP_DT_E4M3); else LAUNCH_R(MSAMP_DT_E5M2);
 #undef LAUNCH_R
 #undef LAUNCH
+    if (!fits) return 1;
     MSAMP_CHECK_LAUNCH("cast_intime_resident_kernel");
     return MSAMP_OK;
 }

@@ -20,6 +20,8 @@ int hip_fail(hipError_t e, const char* what);
 bool waiting_kernels_allowed(hipStream_t st);
 // `count` consecutive non-zero tokens, unique in this process
 uint32_t next_tokens(uint32_t count);
+// how many times the collecting workgroup of a waiting kernel polls before it gives up (msamp_set_spin_limit)
+uint32_t collector_spin_limit();
 
 #define MSAMP_REQUIRE(cond, code, ...)  \
     do {                                \
@@ -198,6 +200,17 @@ __device__ __forceinline__ float dequant1(uint32_t byte) {
 
 // ---- meeting place of the kernels whose workgroups wait for each other --------------------------------
 // `kMaxSlots` eight-byte {token, max} slots start at byte kWsSlotBytes of the workspace; two post words follow.
+// Word kWsErrorWord of the workspace is sticky: a kernel whose bounded wait runs out stores a non-zero code there
+// (a vector store), and msamp_check_async_error reports and clears it.  The collecting workgroup (0) gives up
+// after `spin_limit` polls and then still posts (a NaN amax and the old scale), so that every workgroup that sees
+// the post quantizes with the same scale; the others wait kFollowerSpinFactor times as long for that post, and a
+// workgroup that never sees it writes NaN codes.  Either way the error word is set.
+constexpr int kWsErrorWord = 8;
+constexpr uint32_t kFollowerSpinFactor = 4;
+constexpr uint32_t kErrCollectorGaveUp = 1, kErrFollowerGaveUp = 2;
+__device__ __forceinline__ void report_wait_expired(uint32_t* error_word, uint32_t code) {
+    __hip_atomic_fetch_or(error_word, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 constexpr int kWsSlotBytes = 8192;
 constexpr int kMaxSlots = 512;
 static_assert(kWsSlotBytes + (kMaxSlots + 2) * 8 <= MSAMP_WORKSPACE_BYTES, "slots exceed the workspace");

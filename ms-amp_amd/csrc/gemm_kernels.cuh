@@ -1,0 +1,867 @@
+// FP8 GEMM for gfx950: D[N][M] = (B[N][K] . A[M][K]^T) * a_scale_inv * b_scale_inv (+bias) (+D).
+//
+// Both operands are K-contiguous, which is the layout the 32x32x64 FP8 MFMA wants: a lane holds
+// 32 consecutive K bytes of one row.  Inside the kernel the operand that supplies D's rows is X
+// (= B of the API, N rows) and the one that supplies D's columns is Y (= A of the API, M rows).
+//
+// Block tile BR x BC over K slices of 128 bytes, four wavefronts in a 2 x 2 arrangement, LDS
+// double-buffered with a 16-byte-chunk XOR swizzle that keeps both the 128-bit tile writes and
+// the 128-bit fragment reads off shared banks.  Tiles are handed to workgroups so that the
+// workgroups of one XCD (one L2) work on neighbouring tiles.
+#pragma once
+#include "common.cuh"
+#include "gemm_call.h"
+
+#include <atomic>
+
+#include <type_traits>
+
+namespace msamp {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kGemmThreads = 256;
+
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row & 7) ^ ((row >> 3) & 1)); }
+
+template <int ROWS, bool KGUARD>
+struct TileLoader {
+    static constexpr int kIters = ROWS * 8 / kGemmThreads;
+    uint4 regs[kIters];
+
+    // rows beyond `nrows` are clamped (their products land in output rows that are never stored);
+    // with KGUARD, K chunks beyond `K` read as zero (without it K is a multiple of the stage).
+    __device__ __forceinline__ void gload(const uint8_t* __restrict__ base, int row0, int nrows, int K, int k0) {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < kIters; ++i) {
+            const int idx = t + kGemmThreads * i;
+            const int r = idx >> 3, c = idx & 7;
+            int gr = row0 + r;
+            gr = gr < nrows ? gr : nrows - 1;
+            const int kk = k0 + c * 16;
+            if (!KGUARD || kk < K) {
+                regs[i] = *reinterpret_cast<const uint4*>(base + static_cast<size_t>(gr) * K + kk);
+            } else {
+                regs[i] = make_uint4(0, 0, 0, 0);
+            }
+        }
+    }
+    __device__ __forceinline__ void lstore(uint8_t* lds) const {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < kIters; ++i) {
+            const int idx = t + kGemmThreads * i;
+            const int r = idx >> 3, c = idx & 7;
+            *reinterpret_cast<uint4*>(lds + r * kBK + (swz(r, c) << 4)) = regs[i];
+        }
+    }
+};
+
+// 32 K-bytes of one tile row for this lane: chunks 2*kc, 2*kc+1 of the 128-byte row
+__device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int kc) {
+    const v4i lo = *reinterpret_cast<const v4i*>(lds + row * kBK + (swz(row, 2 * kc) << 4));
+    const v4i hi = *reinterpret_cast<const v4i*>(lds + row * kBK + (swz(row, 2 * kc + 1) << 4));
+    v8i f;
+    f[0] = lo[0], f[1] = lo[1], f[2] = lo[2], f[3] = lo[3];
+    f[4] = hi[0], f[5] = hi[1], f[6] = hi[2], f[7] = hi[3];
+    return f;
+}
+
+template <int XF, int YF>
+__device__ __forceinline__ v16f mfma(const v8i& x, const v8i& y, const v16f& c) {
+    constexpr int cb = (XF == MSAMP_DT_E4M3) ? 0 : 1;
+    constexpr int bl = (YF == MSAMP_DT_E4M3) ? 0 : 1;
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, cb, bl, 0, 0, 0, 0);
+}
+
+template <typename OT>
+__device__ __forceinline__ void store_out(OT* p, float v, bool accumulate) {
+    if (accumulate) v += Elem<OT>::load(p);
+    Elem<OT>::store(p, v);
+}
+
+__device__ __forceinline__ float load_bias(const void* bias, int dt, int i) {
+    if (dt == MSAMP_DT_F32) return static_cast<const float*>(bias)[i];
+    if (dt == MSAMP_DT_F16) return f16_bits_to_float(static_cast<const uint16_t*>(bias)[i]);
+    return bf16_bits_to_float(static_cast<const uint16_t*>(bias)[i]);
+}
+
+// workgroup id -> tile, keeping the workgroups of one XCD on adjacent tiles and walking groups of
+// `kGroup` tile rows column by column so that the X and Y panels of a group stay in that L2
+__device__ __forceinline__ void tile_of_block(int tiles_r, int tiles_c, int& tr, int& tc) {
+    constexpr int kXcd = 8, kGroup = 8;
+    const int nt = tiles_r * tiles_c;
+    int id = blockIdx.x;
+    if (nt % kXcd == 0) id = (id % kXcd) * (nt / kXcd) + id / kXcd;
+    const int per_group = kGroup * tiles_c;
+    const int g = id / per_group;
+    const int first_r = g * kGroup;
+    const int rows_here = (tiles_r - first_r) < kGroup ? (tiles_r - first_r) : kGroup;
+    const int in_g = id - g * per_group;
+    tr = first_r + in_g % rows_here;
+    tc = in_g / rows_here;
+}
+
+template <int BR, int BC, int XF, int YF, typename OT, bool KGUARD>
+__global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* __restrict__ X,
+                                                                 const uint8_t* __restrict__ Y, OT* __restrict__ D,
+                                                                 int NR, int NC, int K,
+                                                                 const float* __restrict__ x_scale_inv,
+                                                                 const float* __restrict__ y_scale_inv, int accumulate,
+                                                                 const void* __restrict__ bias, int bias_dt) {
+    constexpr int WR = BR / 2, WC = BC / 2;    // wave tile
+    constexpr int TR = WR / 32, TC = WC / 32;  // MFMA tiles per wave
+    constexpr int kStage = (BR + BC) * kBK;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    int tr, tc;
+    tile_of_block((NR + BR - 1) / BR, (NC + BC - 1) / BC, tr, tc);
+    const int row0 = tr * BR, col0 = tc * BC;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    v16f acc[TR][TC];
+#pragma unroll
+    for (int i = 0; i < TR; ++i)
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    TileLoader<BR, KGUARD> lx;
+    TileLoader<BC, KGUARD> ly;
+    const int nk = (K + kBK - 1) / kBK;
+    // The K slices are walked in ascending order, 64 bytes of K per MFMA, exactly as the direct-to-LDS kernel below
+    // walks them: the two kernels add up the same blocks in the same order and agree to the bit.  (Walking them in
+    // an order rotated per workgroup, to spread the memory channels, was measured slower: 2-4 % at 2048 x 2048 x 4096,
+    // 10-14 % at 4096 x 4096 x 4112.)
+    auto slice = [&](int kt) { return kt * kBK; };
+    lx.gload(X, row0, NR, K, slice(0));
+    ly.gload(Y, col0, NC, K, slice(0));
+    lx.lstore(smem);
+    ly.lstore(smem + BR * kBK);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const uint8_t* sx = smem + (kt & 1) * kStage;
+        const uint8_t* sy = sx + BR * kBK;
+        if (kt + 1 < nk) {
+            lx.gload(X, row0, NR, K, slice(kt + 1));
+            ly.gload(Y, col0, NC, K, slice(kt + 1));
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            v8i fx[TR], fy[TC];
+#pragma unroll
+            for (int i = 0; i < TR; ++i) fx[i] = read_frag(sx, wr * WR + i * 32 + l32, ks * 2 + lh);
+#pragma unroll
+            for (int j = 0; j < TC; ++j) fy[j] = read_frag(sy, wc * WC + j * 32 + l32, ks * 2 + lh);
+#pragma unroll
+            for (int i = 0; i < TR; ++i)
+#pragma unroll
+                for (int j = 0; j < TC; ++j) acc[i][j] = mfma<XF, YF>(fx[i], fy[j], acc[i][j]);
+        }
+        if (kt + 1 < nk) {
+            uint8_t* nx = smem + ((kt + 1) & 1) * kStage;
+            lx.lstore(nx);
+            ly.lstore(nx + BR * kBK);
+        }
+        __syncthreads();
+    }
+
+    const float alpha = (*x_scale_inv) * (*y_scale_inv);
+#pragma unroll
+    for (int j = 0; j < TC; ++j) {
+        const int col = col0 + wc * WC + j * 32 + l32;
+        if (col >= NC) continue;
+        const float bv = bias != nullptr ? load_bias(bias, bias_dt, col) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TR; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = row0 + wr * WR + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (row < NR) {
+                    store_out<OT>(D + static_cast<size_t>(row) * NC + col, fmaf(acc[i][j][r], alpha, bv), accumulate != 0);
+                }
+            }
+        }
+    }
+}
+
+
+
+// two floats -> packed 16-bit pair with the hardware's round-to-nearest-even converters
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+// four consecutive elements of an output row straight from the accumulators, one by one: ragged edges,
+// bias and accumulation, all in float32 with a single rounding to the output type
+template <typename OT>
+__device__ __noinline__ void store_quad_slow(OT* D, int row, int col, int NR, int NC, float alpha, float v0, float v1,
+                                             float v2, float v3, int accumulate, const void* bias, int bias_dt) {
+    if (row >= NR) return;
+    const float v[4] = {v0, v1, v2, v3};
+    for (int e = 0; e < 4; ++e) {
+        if (col + e >= NC) break;
+        const float bv = bias != nullptr ? load_bias(bias, bias_dt, col + e) : 0.0f;
+        store_out<OT>(D + static_cast<size_t>(row) * NC + col + e, fmaf(v[e], alpha, bv), accumulate != 0);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Main kernel: 256 x 256 output tile over 128-byte K slices, four wavefronts each owning a 128 x 128
+// quadrant (16 accumulators of the 32x32x64 FP8 MFMA = 256 accumulation registers per lane).
+//  * Tiles travel global -> LDS with the direct-to-LDS load: no staging registers, no LDS stores.  A
+//    lane group of 8 fetches one whole 128-byte line (full-line requests are what the L2 serves best).
+//  * Two 64 KiB LDS stages.  A slice is computed in two 64-byte sub-steps; the fragments of the next
+//    sub-step are read while the 16 MFMAs of the current one execute (two register buffers).
+//  * One workgroup barrier per slice, between the sub-steps: by then every wave holds the whole slice
+//    in registers, so the stage is refilled right away with the slice after next (all 16 loads during
+//    the second sub-step, which leaves them a whole sub-step to land).
+//  * LDS reads and tile loads are interleaved with the MFMAs one at a time, so that neither the LDS nor
+//    the vector-memory queue backs up and stalls the MFMA stream.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+constexpr int kDmaStage = 2 * kDmaTile * kBK;    // X + Y slice: 64 KiB
+
+// s_waitcnt vmcnt(N), leaving the other counters unconstrained (gfx9 encoding: vmcnt = [3:0] and [15:14])
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+//  * XT / YT: that operand is handed over K-major, T[K][rows] with the rows contiguous (the transpose of
+//    what the product needs), so that callers need not materialize transposed copies.  Its slice sits in
+//    LDS as 128 k-rows of 256 bytes (same 32 KiB), filled by the same eight 1 KiB loads, and its
+//    fragments come from the transposing LDS read: a 16-lane group reads eight k-rows of 16 bytes and
+//    lane i receives byte i of each, i.e. eight consecutive k for its row -- four such reads make the
+//    32-byte operand of the MFMA.  The 16-byte position inside a k-row is XOR-ed with k % 8 (on the global
+//    side again) so that the eight k-rows of one read fall into different banks.  Needs that operand's
+//    row count to be a multiple of 256.
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+//  * QF (an FP8 format, or 0): the output is not stored in OT but cast on to FP8 with in-time scaling in the same
+//    launch, the way cast_to_fp8 of the stored output would: D is rounded to OT in registers, max |D| is taken over
+//    the whole matrix, the scale follows from it, and the codes of D * scale are what reaches memory -- bit for
+//    bit what the two steps give, without D's trip through memory.  Every workgroup holds its tile in registers
+//    while the maxima meet (slots in the workspace, as in the one-pass in-time cast), so the launch must have all
+//    its workgroups on the chip at once: the host only takes this path for at most one tile per CU.
+// QuantArgs (the meta pointers and meeting slots of the fused cast) is declared in gemm_call.h
+
+// a * b rounded to OT (as the plain epilogue stores it) and widened again
+template <typename OT>
+__device__ __forceinline__ void round_pair(float a, float b, float& ra, float& rb) {
+    if constexpr (sizeof(OT) == 4) {
+        ra = a, rb = b;
+    } else if constexpr (__is_same(OT, bf16_t)) {
+        const uint32_t p = pack_bf16(a, b);
+        ra = __uint_as_float(p << 16), rb = __uint_as_float(p & 0xffff0000u);
+    } else {
+        const f32x2 v = {a, b};
+        const f16x2 h = __builtin_convertvector(v, f16x2);
+        ra = static_cast<float>(h[0]), rb = static_cast<float>(h[1]);
+    }
+}
+
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0>
+__global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
+                                                                     const uint8_t* __restrict__ Y, OT* __restrict__ D,
+                                                                     int NR, int NC, int K,
+                                                                     const float* __restrict__ x_scale_inv,
+                                                                     const float* __restrict__ y_scale_inv, int accumulate,
+                                                                     const void* __restrict__ bias, int bias_dt,
+                                                                     QuantArgs qa) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    int tr, tc;
+    tile_of_block((NR + kDmaTile - 1) / kDmaTile, (NC + kDmaTile - 1) / kDmaTile, tr, tc);
+    const int row0 = tr * kDmaTile, col0 = tc * kDmaTile;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wr = wave >> 1, wc = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+    // the output factor is fetched now: left to the epilogue, the two scalar loads sit on its critical path
+    float alpha_early = (*x_scale_inv) * (*y_scale_inv);
+    asm volatile("" : "+v"(alpha_early));
+
+    // ---- global -> LDS.  A stage holds 256 X rows then 256 Y rows, 128 bytes per row.  One wave
+    // instruction fills 8 rows (1 KiB, lane-contiguous): lane l lands in row l/8, 16-byte position l%8,
+    // and therefore fetches the logical chunk position ^ swizzle(row).  Rows past the end of the matrix
+    // are clamped to its last row (their results are never stored).
+    const int chunk = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)smem)));
+    // K-major operand: one wave instruction fills 4 k-rows of 256 bytes; lane l lands in k-row l/16,
+    // position l%16, and fetches the logical chunk position ^ (k-row % 8)
+    const int chunk_t = (lane & 15) ^ ((wave & 1) * 4 + (lane >> 4));
+    uint32_t xoff[8], yoff[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = (i * 4 + wave) * 8 + (lane >> 3);
+        int gx = row0 + r, gy = col0 + r;
+        gx = gx < NR ? gx : NR - 1;
+        gy = gy < NC ? gy : NC - 1;
+        const int krow = (i * 4 + wave) * 4 + (lane >> 4);
+        xoff[i] = XT ? static_cast<uint32_t>(krow) * static_cast<uint32_t>(NR) + row0 + chunk_t * 16
+                     : static_cast<uint32_t>(gx) * static_cast<uint32_t>(K) + chunk * 16;
+        yoff[i] = YT ? static_cast<uint32_t>(krow) * static_cast<uint32_t>(NC) + col0 + chunk_t * 16
+                     : static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
+    }
+    // one of the 16 loads of a slice (0..7: X rows, 8..15: Y rows), so they can be spread between MFMAs
+    auto dma = [&](int kt, int stage, int which) {
+        const bool is_x = which < 8;
+        const size_t slice = static_cast<size_t>(kt) * kBK;
+        const uint8_t* src = is_x ? X + (XT ? slice * NR : slice) : Y + (YT ? slice * NC : slice);
+        const uint32_t off = which < 8 ? xoff[which] : yoff[which - 8];
+        const uint32_t dst = lds_base + stage * kDmaStage + (which < 8 ? 0 : kDmaTile * kBK) + ((which & 7) * 4 + wave) * 1024;
+        // Written as assembly so that the compiler does not see an LDS write it cannot tell apart from
+        // the fragment reads: it would otherwise make every LDS read wait for all loads in flight.
+        // Completion is tracked by hand with wait_vmcnt<>() before the barriers below.  M0 holds the
+        // wave's LDS destination.
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + off) : "memory", "m0");
+    };
+
+    // ---- LDS -> fragments.  Row-major operand: this lane's row inside a 32-row block and its swizzled
+    // 16-byte chunks.  K-major operand: the address this lane contributes to a transposing read.
+    const int fsw = (lane & 7) ^ ((lane >> 3) & 1);
+    const int off_a = ((2 * lh) ^ fsw) << 4;    // sub-step 0, low half; high half is ^16, sub-step 1 is ^64
+    const int xrow = (wr * 128 + l32) * kBK;
+    const int yrow = kDmaTile * kBK + (wc * 128 + l32) * kBK;
+    const int i16 = lane & 15, tj = i16 >> 1, g1 = (lane >> 4) & 1;
+    const int t_lane = (lh * 32 + tj) * 256 + (i16 & 1) * 8;    // k-row and 8-byte half of this lane's address
+    // A sub-step needs 8 fragments of 8 registers (X blocks 0..3, Y blocks 0..3).  They arrive in pieces:
+    // two 16-byte reads per fragment of a row-major operand, four 8-byte transposing reads otherwise.
+    constexpr int kPX = XT ? 16 : 8, kPY = YT ? 16 : 8, kPieces = kPX + kPY;
+    auto read_piece = [&](int* dst, int stage, int ks, int p) {
+        const bool is_x = p < kPX;
+        const int q = is_x ? p : p - kPX;
+        const uint8_t* base = smem + stage * kDmaStage;
+        if ((is_x && !XT) || (!is_x && !YT)) {
+            const int blk = q >> 1, hf = q & 1;
+            const v4i val = *reinterpret_cast<const v4i*>(base + (is_x ? xrow : yrow) + blk * 32 * kBK +
+                                                          ((off_a ^ (ks * 64)) ^ (hf * 16)));
+            int* d = dst + ((is_x ? 0 : 4) + blk) * 8 + hf * 4;
+            d[0] = val[0], d[1] = val[1], d[2] = val[2], d[3] = val[3];
+        } else {
+            const int blk = q >> 2, qq = q & 3;
+            const int wq = is_x ? wr : wc;
+            const int addr = (is_x ? 0 : kDmaTile * kBK) + t_lane + (ks * 64 + qq * 8) * 256 + wq * 128 +
+                             (((blk * 2 + g1) ^ tj) << 4);
+            const v2i val = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+                (__attribute__((address_space(3))) v2i*)(base + addr));
+            int* d = dst + ((is_x ? 0 : 4) + blk) * 8 + qq * 2;
+            d[0] = val[0], d[1] = val[1];
+        }
+    };
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const int nk = K / kBK;
+    int fa[64], fb[64];    // fragments [X0..X3, Y0..Y3] x 8 registers, two buffers
+
+    // One sub-step: 16 MFMAs on `cur`, the fragment reads of the next sub-step into `nxt` and, if asked for, the
+    // 16 tile loads of slice ld_kt, one per MFMA.
+    // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row l%32, four
+    // consecutive D columns per register quad -- the layout the epilogue wants.
+    auto sub_step = [&](const int* cur, int* nxt, int rd_stage, int rd_ks, bool do_read, int ld_kt, int ld_stage,
+                        bool do_load) {
+        constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
+        constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {    // the Y fragment stays for four MFMAs in a row (measured 1 % faster than X staying)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = j * 4 + i;
+                const int* cx = cur + i * 8;
+                const int* cy = cur + (4 + j) * 8;
+                const v8i fx = {cx[0], cx[1], cx[2], cx[3], cx[4], cx[5], cx[6], cx[7]};
+                const v8i fy = {cy[0], cy[1], cy[2], cy[3], cy[4], cy[5], cy[6], cy[7]};
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fy, fx, acc[i][j], cb, bl, 0, 0, 0, 0);
+                if (do_read) {
+#pragma unroll
+                    for (int p = n * kPieces / 16; p < (n + 1) * kPieces / 16; ++p) read_piece(nxt, rd_stage, rd_ks, p);
+                }
+                if (do_load) dma(ld_kt, ld_stage, n);
+            }
+        }
+        static_for<16>([&](auto nc) {
+            constexpr int n = decltype(nc)::value;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, (n + 1) * kPieces / 16 - n * kPieces / 16, 0);    // its LDS reads
+        });
+    };
+
+    // prologue: slices 0 and 1; wait for slice 0; read its first fragments
+#pragma unroll
+    for (int w = 0; w < 16; ++w) dma(0, 0, w);
+    if (nk > 1) {
+#pragma unroll
+        for (int w = 0; w < 16; ++w) dma(1, 1, w);
+        wait_vmcnt<16>();
+    } else {
+        wait_vmcnt<0>();
+    }
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < kPieces; ++p) read_piece(fa, 0, 0, p);
+    // slice kt lives in stage kt & 1 and slice kt+1 is already on its way.  Sub-step 0: MFMAs on the first half,
+    // read the second half.  Barrier: slice kt+1 has landed, nobody needs the LDS copy of slice kt.  Sub-step 1:
+    // MFMAs on the second half, read the first half of slice kt+1, refill this stage with all of slice kt+2.
+    int kt = 0;
+    for (; kt + 3 < nk; kt += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            sub_step(fa, fb, u, 1, true, 0, 0, false);
+            wait_vmcnt<0>();
+            __syncthreads();
+            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, true);
+        }
+    }
+    for (; kt < nk; kt += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k1 = kt + u;
+            if (k1 < nk) {
+                sub_step(fa, fb, u, 1, true, 0, 0, false);
+                wait_vmcnt<0>();
+                __syncthreads();
+                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, k1 + 2 < nk);
+            }
+        }
+    }
+    // No barrier here: the last LDS reads of every wave were issued (and awaited) before the barrier of the last
+    // slice, and no load is in flight, so each wave may start on its patch as soon as its own MFMAs are done.
+
+    if constexpr (QF != 0) {
+        // ---- fused in-time cast (whole tiles only, no bias, no accumulation: the host sees to that)
+        __shared__ uint32_t q_red[kGemmThreads / kWave];
+        __shared__ uint32_t q_scale, q_amax;
+        const float alpha = alpha_early;
+        // max |acc| as an ordered bit pattern: NaN above Inf above everything finite, so a NaN reaches the amax
+        // as it does through abs().max()
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) m = umax(m, __float_as_uint(acc[i][j][r]) & 0x7fffffffu);
+        m = block_max_u32(m, q_red);    // valid in lane 0 of wave 0
+        const int tid = threadIdx.x;
+        if (tid == 0) {
+            // Scaling by |alpha| and rounding to OT never reorder magnitudes, so the maximum of the rounded outputs
+            // is the rounded, scaled maximum.
+            float am, unused;
+            round_pair<OT>(__uint_as_float(m) * fabsf(alpha), 0.0f, am, unused);
+            m = __float_as_uint(am) & 0x7fffffffu;
+            __hip_atomic_store(qa.slots + blockIdx.x, (static_cast<uint64_t>(qa.token) << 32) | m, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // Workgroup 0 collects the slots (its first wave), derives amax and scale and posts
+        // both, tagged with the token, in the two words behind the slots; the other workgroups poll only those.
+        // Every wait is bounded.  Workgroup 0 posts even when it gives up (NaN amax, old scale), and the others wait
+        // longer for the post than it waits for them; whoever gives up sets the sticky error word of the workspace.
+        uint64_t* post = qa.slots + kMaxSlots;
+        if (blockIdx.x == 0) {
+            if (tid < kWave) {
+                uint32_t mm = 0;
+                bool all_in = false;
+                for (uint32_t spins = 0; !all_in && spins < qa.spin_limit; ++spins) {
+                    uint64_t sv[kMaxSlots / kWave];
+#pragma unroll
+                    for (int j = 0; j < kMaxSlots / kWave; ++j)
+                        sv[j] = __hip_atomic_load(qa.slots + tid + j * kWave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    bool ok = true;
+                    mm = 0;
+#pragma unroll
+                    for (int j = 0; j < kMaxSlots / kWave; ++j) {
+                        const bool live = static_cast<uint32_t>(tid + j * kWave) < gridDim.x;
+                        ok = ok && (!live || static_cast<uint32_t>(sv[j] >> 32) == qa.token);
+                        mm = umax(mm, live ? static_cast<uint32_t>(sv[j]) : 0u);
+                    }
+                    all_in = __all(ok);
+                }
+                mm = wave_max_u32(mm);
+                if (tid == 0) {
+                    float am = __uint_as_float(mm);
+                    if (!all_in) {    // gave up: NaN amax, old scale, both still posted, sticky error word set
+                        am = __uint_as_float(0x7fc00000u);
+                        report_wait_expired(qa.error_word, kErrCollectorGaveUp);
+                    } else if ((qa.flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
+                    const float sc = scale_rule(am, *qa.scale, qa.fp_max, qa.margin);
+                    const uint64_t tag = static_cast<uint64_t>(qa.token) << 32;
+                    __hip_atomic_store(post, tag | __float_as_uint(am), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(post + 1, tag | __float_as_uint(sc), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    q_scale = __float_as_uint(sc);
+                    q_amax = __float_as_uint(am);
+                    *qa.amax = am;
+                    *qa.scale = sc;
+                    *qa.scale_inv = 1.0f / sc;
+                }
+            }
+        } else {
+            if (tid == 0) {
+                uint64_t pa = 0, ps = 0;
+                bool posted = false;
+                const uint64_t follower_limit = static_cast<uint64_t>(qa.spin_limit) * kFollowerSpinFactor;
+                for (uint64_t spins = 0; !posted && spins < follower_limit; ++spins) {
+                    pa = __hip_atomic_load(post, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ps = __hip_atomic_load(post + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    posted = static_cast<uint32_t>(pa >> 32) == qa.token && static_cast<uint32_t>(ps >> 32) == qa.token;
+                }
+                if (!posted) report_wait_expired(qa.error_word, kErrFollowerGaveUp);
+                q_amax = posted ? static_cast<uint32_t>(pa) : 0x7fc00000u;
+                q_scale = posted ? static_cast<uint32_t>(ps) : 0x7fc00000u;
+            }
+        }
+        __syncthreads();    // also: every wave is through with the stages, which the patches below reuse
+        const float sc = __uint_as_float(q_scale);
+        // with a positive finite amax and the scale derived from it nothing leaves the format and nothing is NaN:
+        // the clamp and the NaN patch of the general conversion can go
+        const bool in_range = __uint_as_float(q_amax) * sc <= qa.fp_max && __uint_as_float(q_amax) > 0.0f;
+        constexpr int kQPitch = 128 + 16;    // bytes per patch row: 128 codes and padding that staggers the banks
+        uint8_t* qpatch = smem + wave * (32 * kQPitch);
+        auto emit = [&](auto checked) {
+            constexpr bool kChecked = decltype(checked)::value;
+            static_for<4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                static_for<4>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        // the outputs as OT would hold them, then scaled
+                        float r0, r1, r2, r3;
+                        round_pair<OT>(acc[i][j][4 * q] * alpha, acc[i][j][4 * q + 1] * alpha, r0, r1);
+                        round_pair<OT>(acc[i][j][4 * q + 2] * alpha, acc[i][j][4 * q + 3] * alpha, r2, r3);
+                        uint32_t w;
+                        if constexpr (kChecked) w = quant4<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
+                        else w = quant4_in_range<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
+                        *reinterpret_cast<uint32_t*>(qpatch + l32 * kQPitch + j * 32 + q * 8 + lh * 4) = w;
+                    }
+                });
+                // the patch is private to this wave and the LDS serves one wave's requests in order: no waits here
+                auto rd = [&](int u) {
+                    return *reinterpret_cast<const uint4*>(qpatch + (u * 8 + (lane >> 3)) * kQPitch + (lane & 7) * 16);
+                };
+                const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3);
+                auto st = [&](int u, const uint4& v) {
+                    const int grow = row0 + wr * 128 + i * 32 + u * 8 + (lane >> 3);
+                    const int gcol = col0 + wc * 128 + (lane & 7) * 16;
+                    *reinterpret_cast<uint4*>(qa.q + static_cast<size_t>(grow) * NC + gcol) = v;
+                };
+                st(0, val0), st(1, val1), st(2, val2), st(3, val3);
+            });
+        };
+        if (in_range) emit(std::false_type{}); else emit(std::true_type{});
+        return;
+    }
+
+    // ---- epilogue: per 32-row block, accumulators -> this wave's LDS patch -> 16-byte row stores
+    constexpr int kEsz = static_cast<int>(sizeof(OT));
+    constexpr int kPitch = 128 * kEsz + 16;    // bytes per patch row (padding staggers the banks)
+    uint8_t* patch = smem + wave * (32 * kPitch);
+    const float alpha = alpha_early;
+    const bool vec_ok = (NC % (16 / kEsz) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
+    const bool plain = vec_ok && !accumulate && bias == nullptr;
+    constexpr int kChunksPerRow = 128 * kEsz / 16;      // 16 (2-byte) or 32 (float)
+    constexpr int kRowsPerPass = 64 / kChunksPerRow;    // 4 or 2
+    constexpr int kElemsPerChunk = 16 / kEsz;           // 8 or 4
+    if (!plain && vec_ok) {
+        // ---- bias and / or accumulation with 16-byte row accesses: the raw float32 accumulators of a 32-row block go
+        // through a per-wave float32 patch, each lane picks up one 16-byte segment of an output row, reads the old
+        // output there if it is to be added, and stores fma(acc, alpha, bias) (+ old) rounded once -- the expression of
+        // the element-wise path below and of the generic kernel.  A lane's columns are the same in every pass, so
+        // its bias values are fetched once.
+        constexpr int kFPitch = 128 * 4 + 16;    // bytes per float32 patch row
+        uint8_t* fpatch = smem + wave * (32 * kFPitch);
+        const int pc = lane % kChunksPerRow, prl = lane / kChunksPerRow;
+        const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
+        const bool col_ok = gcol < NC;
+        float bv[kElemsPerChunk];
+#pragma unroll
+        for (int e = 0; e < kElemsPerChunk; ++e) bv[e] = (bias != nullptr && col_ok) ? load_bias(bias, bias_dt, gcol + e) : 0.0f;
+        constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
+        constexpr int kGroup = 4;                     // passes whose old outputs are in flight together
+        static_for<4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            static_for<4>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    *reinterpret_cast<float4*>(fpatch + l32 * kFPitch + (j * 32 + q * 8 + lh * 4) * 4) =
+                        make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+                }
+            });
+            // the patch is private to this wave and the LDS serves one wave's requests in order: no waits needed
+            static_for<kPasses / kGroup>([&](auto gc) {
+                constexpr int p0 = decltype(gc)::value * kGroup;
+                uint4 old[kGroup];
+                bool ok[kGroup];
+#pragma unroll
+                for (int u = 0; u < kGroup; ++u) {
+                    const int grow = row0 + wr * 128 + i * 32 + (p0 + u) * kRowsPerPass + prl;
+                    ok[u] = col_ok && grow < NR;
+                    old[u] = make_uint4(0, 0, 0, 0);
+                    if (accumulate && ok[u]) old[u] = *reinterpret_cast<const uint4*>(D + static_cast<size_t>(grow) * NC + gcol);
+                }
+#pragma unroll
+                for (int u = 0; u < kGroup; ++u) {
+                    const int pr = (p0 + u) * kRowsPerPass + prl;
+                    const int grow = row0 + wr * 128 + i * 32 + pr;
+                    const float* src = reinterpret_cast<const float*>(fpatch + pr * kFPitch + pc * kElemsPerChunk * 4);
+                    float r[kElemsPerChunk], o[kElemsPerChunk];
+                    const float4 a0 = *reinterpret_cast<const float4*>(src);
+                    r[0] = a0.x, r[1] = a0.y, r[2] = a0.z, r[3] = a0.w;
+                    if constexpr (kElemsPerChunk == 8) {
+                        const float4 a1 = *reinterpret_cast<const float4*>(src + 4);
+                        r[4] = a1.x, r[5] = a1.y, r[6] = a1.z, r[7] = a1.w;
+                    }
+                    if constexpr (kEsz == 4) {
+                        o[0] = __uint_as_float(old[u].x), o[1] = __uint_as_float(old[u].y);
+                        o[2] = __uint_as_float(old[u].z), o[3] = __uint_as_float(old[u].w);
+                    } else {
+                        In16<OT>::decode(old[u], o);
+                    }
+#pragma unroll
+                    for (int e = 0; e < kElemsPerChunk; ++e) {
+                        r[e] = fmaf(r[e], alpha, bv[e]);
+                        if (accumulate) r[e] += o[e];
+                    }
+                    uint4 v;
+                    if constexpr (kEsz == 4) {
+                        v = make_uint4(__float_as_uint(r[0]), __float_as_uint(r[1]), __float_as_uint(r[2]), __float_as_uint(r[3]));
+                    } else if constexpr (__is_same(OT, bf16_t)) {
+                        v = make_uint4(pack_bf16(r[0], r[1]), pack_bf16(r[2], r[3]), pack_bf16(r[4], r[5]), pack_bf16(r[6], r[7]));
+                    } else {
+                        v = make_uint4(pack_f16(r[0], r[1]), pack_f16(r[2], r[3]), pack_f16(r[4], r[5]), pack_f16(r[6], r[7]));
+                    }
+                    if (ok[u]) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
+                }
+            });
+        });
+        return;
+    }
+    if (!plain) {
+        static_for<4>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            static_for<4>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    store_quad_slow<OT>(D, row0 + wr * 128 + i * 32 + l32, col0 + wc * 128 + j * 32 + q * 8 + lh * 4, NR, NC,
+                                        alpha, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                        acc[i][j][4 * q + 3], accumulate, bias, bias_dt);
+                }
+            });
+        });
+        return;
+    }
+    static_for<4>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        static_for<4>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int c = j * 32 + q * 8 + lh * 4;
+                uint8_t* dst = patch + l32 * kPitch + c * kEsz;
+                const float v0 = acc[i][j][4 * q] * alpha, v1 = acc[i][j][4 * q + 1] * alpha;
+                const float v2 = acc[i][j][4 * q + 2] * alpha, v3 = acc[i][j][4 * q + 3] * alpha;
+                if constexpr (kEsz == 4) {
+                    *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
+                } else if constexpr (__is_same(OT, bf16_t)) {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(v0, v1), pack_bf16(v2, v3));
+                } else {
+                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_f16(v0, v1), pack_f16(v2, v3));
+                }
+            }
+        });
+        // no wait between the writes above and the reads below, nor before the next block's writes: the patch is
+        // private to this wave and the LDS serves one wave's requests in order
+        constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
+        static_for<kPasses / 8>([&](auto gc) {
+            constexpr int p0 = decltype(gc)::value * 8;
+            // eight reads in flight together, then the eight stores (named values: an array here ends up in scratch)
+            auto rd = [&](int u) {
+                const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
+                return *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
+            };
+            const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3), val4 = rd(4), val5 = rd(5), val6 = rd(6),
+                        val7 = rd(7);
+            auto st = [&](int u, const uint4& v) {
+                const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
+                const int pc = lane % kChunksPerRow;
+                const int grow = row0 + wr * 128 + i * 32 + pr;
+                const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
+                if (grow < NR && gcol < NC) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
+            };
+            st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
+        });
+    });
+}
+
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
+static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                           const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    constexpr int smem = 2 * kDmaStage;
+    static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT>;
+    if (!configured.load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel)");
+        configured.store(true, std::memory_order_release);
+    }
+    const int tiles = ((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys,
+                       accumulate, bias, bias_dt, QuantArgs{});
+    MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel");
+    return MSAMP_OK;
+}
+
+// the same kernel with the in-time cast to FP8 fused in (see QF above); the caller has checked the shape
+template <int XF, int YF, typename OT, bool XT, bool YT, int QF>
+static int launch_gemm_dma_quant(const uint8_t* X, const uint8_t* Y, int NR, int NC, int K, const float* xs, const float* ys,
+                                 const QuantArgs& qa, hipStream_t st) {
+    constexpr int smem = 2 * kDmaStage;
+    static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, QF>;
+    if (!configured.load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel, fused cast)");
+        configured.store(true, std::memory_order_release);
+    }
+    // its workgroups wait for each other, one per CU: the runtime must confirm that one fits (asked once per instantiation)
+    static std::atomic<int> resident{-1};
+    int fits = resident.load(std::memory_order_acquire);
+    if (fits < 0) {
+        int blocks = 0;
+        fits = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void*>(kern), kGemmThreads, smem) == hipSuccess &&
+               blocks >= 1;
+        resident.store(fits, std::memory_order_release);
+    }
+    if (!fits) return MSAMP_NOT_FUSED;
+    const int tiles = (NR / kDmaTile) * (NC / kDmaTile);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(nullptr), NR, NC, K, xs, ys, 0,
+                       static_cast<const void*>(nullptr), 0, qa);
+    MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel (fused cast)");
+    return MSAMP_OK;
+}
+
+template <int BR, int BC, int XF, int YF, typename OT, bool KGUARD>
+static int launch_gemm_k(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                       const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    constexpr int smem = 2 * (BR + BC) * kBK;
+    static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
+    auto kern = fp8_gemm_kernel<BR, BC, XF, YF, OT, KGUARD>;
+    if (!configured.load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_kernel)");
+        configured.store(true, std::memory_order_release);
+    }
+    const int tiles = ((NR + BR - 1) / BR) * ((NC + BC - 1) / BC);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys,
+                       accumulate, bias, bias_dt);
+    MSAMP_CHECK_LAUNCH("fp8_gemm_kernel");
+    return MSAMP_OK;
+}
+
+template <int BR, int BC, int XF, int YF, typename OT>
+static int launch_gemm(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                       const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    if (K % kBK == 0) return launch_gemm_k<BR, BC, XF, YF, OT, false>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    return launch_gemm_k<BR, BC, XF, YF, OT, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+}
+
+template <int XF, int YF, typename OT>
+static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                     const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    // the direct-to-LDS kernel needs whole 128-byte K slices and 32-bit row offsets; where it can run it is the
+    // faster one at every size (measured 2.2x from a single 256 x 256 tile up to 121 tiles).  Everything else takes
+    // the generic register-staged kernel with 128 x 128 tiles.
+    const bool fits32 = static_cast<unsigned long long>(NR) * K < (1ull << 32) && static_cast<unsigned long long>(NC) * K < (1ull << 32);
+    if (K % kBK == 0 && fits32)
+        return launch_gemm_dma<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    return launch_gemm<128, 128, XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+}
+
+template <int XF, int YF>
+static int pick_out(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, int NR, int NC, int K, const float* xs,
+                    const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    switch (d_dtype) {
+        case MSAMP_DT_F32:
+            return pick_tile<XF, YF, float>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+        case MSAMP_DT_F16:
+            return pick_tile<XF, YF, f16_t>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+        default:
+            return pick_tile<XF, YF, bf16_t>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    }
+}
+
+template <int XF, int YF, bool XT, bool YT>
+static int pick_out_kmajor(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, int NR, int NC, int K, const float* xs,
+                           const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    switch (d_dtype) {
+        case MSAMP_DT_F32:
+            return launch_gemm_dma<XF, YF, float, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+        case MSAMP_DT_F16:
+            return launch_gemm_dma<XF, YF, f16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+        default:
+            return launch_gemm_dma<XF, YF, bf16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    }
+}
+
+template <int XF, int YF, bool T>
+static int pick_out_quant(const uint8_t* X, const uint8_t* Y, int d_dtype, int NR, int NC, int K, const float* xs, const float* ys,
+                          const QuantArgs& qa, hipStream_t st) {
+    switch (d_dtype) {
+        case MSAMP_DT_F32:
+            return launch_gemm_dma_quant<XF, YF, float, T, T, MSAMP_DT_E4M3>(X, Y, NR, NC, K, xs, ys, qa, st);
+        case MSAMP_DT_F16:
+            return launch_gemm_dma_quant<XF, YF, f16_t, T, T, MSAMP_DT_E4M3>(X, Y, NR, NC, K, xs, ys, qa, st);
+        default:
+            return launch_gemm_dma_quant<XF, YF, bf16_t, T, T, MSAMP_DT_E4M3>(X, Y, NR, NC, K, xs, ys, qa, st);
+    }
+}
+
+
+// Everything behind the C entry points for one pair of operand formats.  gemm_inst.hip instantiates it once per
+// pair (four translation units, so that they compile side by side).
+template <int XF, int YF>
+int run_gemm_pair(const GemmCall& c) {
+    if (c.qa != nullptr) {
+        if (c.xt) return pick_out_quant<XF, YF, true>(c.X, c.Y, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, *c.qa, c.st);
+        return pick_out_quant<XF, YF, false>(c.X, c.Y, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, *c.qa, c.st);
+    }
+    if (c.xt && c.yt)
+        return pick_out_kmajor<XF, YF, true, true>(c.X, c.Y, c.D, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, c.accumulate, c.bias, c.bias_dt, c.st);
+    if (c.yt)
+        return pick_out_kmajor<XF, YF, false, true>(c.X, c.Y, c.D, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, c.accumulate, c.bias, c.bias_dt, c.st);
+    return pick_out<XF, YF>(c.X, c.Y, c.D, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, c.accumulate, c.bias, c.bias_dt, c.st);
+}
+
+}    // namespace msamp

@@ -30,6 +30,8 @@ _vp, _i, _f, _d, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_d
 _SIGNATURES = {
     'msamp_hip_version': ([], _i),
     'msamp_last_error': ([], ctypes.c_char_p),
+    'msamp_check_async_error': ([_vp, _vp], _i),
+    'msamp_set_spin_limit': ([ctypes.c_uint32], None),
     'msamp_amax': ([_vp, _i, _sz, _vp, _vp, _vp], _i),
     'msamp_compute_scaling_factor': ([_vp, _vp, _i, _vp, _i, _f, _i, _vp], _i),
     'msamp_cast_to_fp8': ([_vp, _i, _sz, _vp, _vp, _vp, _vp, _i, _vp], _i),
@@ -122,6 +124,73 @@ def workspace(device):
         ws = torch.zeros(WORKSPACE_BYTES, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+# ---- failures of the kernels whose workgroups wait for each other ------------------------------------------
+ERR_TIMEOUT = -5
+WS_ERROR_BYTE = 32    # byte offset of the sticky error word in a workspace
+_force_two_pass = False
+_pending_error_reads = {}
+
+
+class WaitExpiredError(RuntimeError):
+    """A one-pass in-time cast or a fused GEMM + cast gave up waiting for its other workgroups."""
+
+
+def _two_pass_only():
+    return _force_two_pass or _shared_device()
+
+
+def check_async_error(block=True):
+    """Report a bounded wait that ran out in one of the kernels whose workgroups wait for each other (the one-pass
+    in-time cast, the fused GEMM + cast).  Such a failure cannot be seen by the call that enqueued the kernel; the
+    kernel leaves a sticky word in the workspace instead.
+
+    block=True reads the word of every workspace of this process now (synchronises their streams' work up to here).
+    block=False never waits: it looks at the copies of the words requested by the previous call -- if they have
+    arrived -- and requests new ones, so a training loop that calls it once per step learns of a failure a step or
+    two late without ever synchronising.  Either way a failure raises WaitExpiredError, after switching this
+    process to the two-pass kernels for good (same results, no waiting): the tensors and metas the failed kernel
+    wrote are invalid and the step must be repeated."""
+    global _force_two_pass
+    lib = load()
+    failed = None
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        return    # nothing here can be recorded into a graph, and the waiting kernels stay out of captured streams anyway
+    for key, ws in list(_workspaces.items()):
+        if not ws.is_cuda:
+            continue
+        if block:
+            with torch.cuda.device(ws.device):
+                rc = lib.msamp_check_async_error(_ptr(ws), key[2])
+            if rc == ERR_TIMEOUT:
+                failed = lib.msamp_last_error().decode(errors='replace')
+            elif rc != 0:
+                _check(rc, 'msamp_check_async_error')
+            continue
+        entry = _pending_error_reads.get(key)
+        if entry is None:
+            entry = {'host': torch.zeros(1, dtype=torch.int32, pin_memory=True), 'event': torch.cuda.Event(), 'in_flight': False}
+            _pending_error_reads[key] = entry
+        if entry['in_flight'] and entry['event'].query():
+            entry['in_flight'] = False
+            code = int(entry['host'].item())
+            if code != 0:
+                failed = f'a kernel whose workgroups wait for each other gave up waiting (code {code})'
+                ws[WS_ERROR_BYTE:WS_ERROR_BYTE + 4].zero_()
+        if not entry['in_flight']:
+            entry['host'].copy_(ws[WS_ERROR_BYTE:WS_ERROR_BYTE + 4].view(torch.int32), non_blocking=True)
+            entry['event'].record()
+            entry['in_flight'] = True
+    if failed is not None:
+        _force_two_pass = True
+        raise WaitExpiredError(failed + '; the tensors and metas it wrote are invalid. The process now uses the two-pass '
+                               'kernels only: repeat the step.')
+
+
+def set_spin_limit(polls):
+    """Polls after which a waiting kernel gives up (default 2**20); 0 = give up at once, for tests of that path."""
+    load().msamp_set_spin_limit(int(polls))
 
 
 # ---- scaling ------------------------------------------------------------------------------------
@@ -219,7 +288,7 @@ def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_
     _check(
         lib.msamp_cast_to_fp8_intime(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
-            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _shared_device() else 0),
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _two_pass_only() else 0),
             _ptr(workspace(x.device)),
             _stream()
         ), 'msamp_cast_to_fp8_intime'
@@ -241,7 +310,7 @@ def cast_to_fp8_intime_static(x, scale, amax_cell, scale_inv, out, fp8_dt, margi
     _check(
         lib.msamp_cast_to_fp8_intime_static(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
-            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _shared_device() else 0), _stream()
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _two_pass_only() else 0), _stream()
         ), 'msamp_cast_to_fp8_intime_static'
     )
     return out
@@ -256,7 +325,7 @@ def cast_to_fp8_gated(x, scale, amax_cell, scale_inv, fp8_dt, counter, window, m
     _check(
         lib.msamp_cast_to_fp8_gated(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
-            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _shared_device() else 0), _ptr(counter), window,
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _two_pass_only() else 0), _ptr(counter), window,
             _ptr(workspace(x.device)), _stream()
         ), 'msamp_cast_to_fp8_gated'
     )
@@ -425,7 +494,7 @@ def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, sc
     rc = lib.msamp_fp8_gemm_cast(
         _ptr(a), a_dt, _ptr(a_scale_inv), 1 if a_kmajor else 0, _ptr(b), b_dt, _ptr(b_scale_inv), 1 if b_kmajor else 0,
         _TORCH_TO_DT[hp_dtype], _ptr(out), q_dt, _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), m, n, k, margin,
-        (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _shared_device() else 0), _ptr(workspace(a.device)), _stream()
+        (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _two_pass_only() else 0), _ptr(workspace(a.device)), _stream()
     )
     if rc == NOT_FUSED:
         return None

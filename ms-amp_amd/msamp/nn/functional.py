@@ -10,9 +10,14 @@ from msamp.nn.state import model_state
 
 
 class _FP8GemmFunction(torch.autograd.Function):
-    """y = x W^T with x, W in E4M3; dx = dy W and dW = dy^T x with dy in E5M2; fp32 accumulation."""
+    """y = x W^T (+ bias) with x, W in E4M3; dx = dy W and dW = dy^T x with dy in E5M2; fp32 accumulation.
+
+    The reference adds the bias in a separate elementwise pass after the function (nn/functional.py:184-185); here it
+    rides in the epilogue of the forward GEMM (fma(acc, scale, bias), one rounding to the output type instead of
+    two) and its gradient, the column sums of dy in the output type, is returned from backward as autograd would
+    have formed it."""
     @staticmethod
-    def forward(ctx, input, weight, metas, dtype_holder):
+    def forward(ctx, input, weight, metas, dtype_holder, bias=None):
         ctx.metas = metas
         model_state.check_metas_in_flat(metas)
         input_fp8 = input.cast(Dtypes.kfloat8_e4m3, meta=metas['input'])
@@ -24,7 +29,11 @@ class _FP8GemmFunction(torch.autograd.Function):
         ctx.weight = weight
         ctx.output_dtype = dtype_holder.dtype
         ctx.output_qtype = Dtypes.dtype_to_qtype[dtype_holder.dtype]
-        return Gemm.fp8_gemm(weight_fp8, input_fp8, ctx.output_qtype, use_split_accumulator=False)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        ctx.need_bias_grad = bias is not None and bias.requires_grad
+        if bias is not None:
+            bias = bias.detach().to(ctx.output_dtype).contiguous()
+        return Gemm.fp8_gemm(weight_fp8, input_fp8, ctx.output_qtype, bias=bias, use_split_accumulator=False)
 
     @staticmethod
     def backward(ctx, output_grad):
@@ -77,7 +86,8 @@ class _FP8GemmFunction(torch.autograd.Function):
                     wgrad = wgrad.cast(Dtypes.kfloat8_e4m3, meta=metas['wgrad'], sync=True)
             ctx.weight.backward_grad_update(wgrad)
 
-        return input_grad, None, None, None
+        bias_grad = output_grad.sum(0).to(ctx.bias_dtype) if ctx.need_bias_grad else None
+        return input_grad, None, None, None, bias_grad
 
 
 class FunctionalOverider:
@@ -96,8 +106,8 @@ class FunctionalOverider:
     def _get_wrapper_for_linear(cls, old_fn):
         def new_fn(input, weight, bias=None):
             """linear(input, weight, bias=None): y = x A^T + b; `weight` may be a ScalingTensor carrying
-            `_scaling_metas`, in which case the three GEMMs run in FP8 and the bias is added afterwards
-            in the output dtype (the autocast dtype if autocast is on, else the input's)."""
+            `_scaling_metas`, in which case the three GEMMs run in FP8 and the bias, rounded to the output dtype
+            (the autocast dtype if autocast is on, else the input's), is added in the forward GEMM's epilogue."""
             if not isinstance(input, torch.Tensor):
                 raise TypeError(f'input should be a torch.Tensor. current type: {type(input)}')
             if not isinstance(weight, (torch.Tensor, ScalingTensor)):
@@ -117,9 +127,7 @@ class FunctionalOverider:
                 output_dtype = torch.get_autocast_dtype('cuda')
             else:
                 output_dtype = input.dtype
-            out = _FP8GemmFunction.apply(input, weight, weight._scaling_metas, cls.EMPTY_GRAD_TENSOR.type(output_dtype))
-            if bias is not None:
-                out = out + bias.type(output_dtype).view(1, -1)
+            out = _FP8GemmFunction.apply(input, weight, weight._scaling_metas, cls.EMPTY_GRAD_TENSOR.type(output_dtype), bias)
             if len(shape) != 2:
                 out = out.view(shape[:-1] + (-1, ))
             return out

@@ -25,6 +25,9 @@ class LBOptimizer(Optimizer):
         """One optimization step followed by the scaling-factor update of all FP8 layers."""
         rtn = self.lb_step(closure)
         self._update_scaling_factors()
+        # a bounded wait that ran out inside a cast or GEMM kernel of an earlier step surfaces here, without a
+        # device-to-host synchronisation (the copy of the error word requested by the previous step is looked at)
+        _backend.check_async_error(block=False)
         return rtn
 
     def all_reduce_grads(self, model):

@@ -145,6 +145,35 @@ def test_fp8linear_step_against_oracle_pipeline():
     assert same_float(metas['ograd'].amax[0], gm['amax'][0]) and same_float(metas['ograd'].scale, gm['scale'])
 
 
+def test_fp8linear_bias_rides_in_the_forward_gemm():
+    """The bias is added in the epilogue of the forward GEMM (one rounding): against the oracle with the bias, within
+    one ulp (of the larger of the bare and the biased output) of the reference's two steps (GEMM rounded, then + bias rounded), and the bias gradient is the
+    column sum of dy exactly as autograd forms it for `out + bias`."""
+    torch.manual_seed(11)
+    tokens, d_in, d_out = 512, 256, 384
+    lin = torch.nn.Linear(d_in, d_out, bias=True).cuda()
+    w_ref, b_ref = lin.weight.detach().cpu(), lin.bias.detach().clone()
+    model = LinearReplacer.replace(lin, Dtypes.kfloat16)
+    x = torch.randn(tokens, d_in, device='cuda', dtype=torch.bfloat16, requires_grad=True)
+    dy = torch.randn(tokens, d_out, device='cuda').bfloat16()
+    y = model(x)
+    y.backward(dy)
+    assert y.dtype == torch.bfloat16 and model.bias.grad.dtype == torch.float32
+    assert torch.equal(model.bias.grad, dy.sum(0).to(torch.float32))
+    y0 = torch.nn.functional.linear(x.detach(), model.weight, None)    # the same GEMM without the bias
+    two_step = (y0 + b_ref.bfloat16().view(1, -1)).float()
+    # the two-step result carries the rounding of the bare GEMM output as well: one ulp of the largest of the three
+    ulp = torch.maximum(torch.maximum(two_step.abs(), y.detach().float().abs()), y0.float().abs()) * 2.0**-7
+    assert ((y.detach().float() - two_step).abs() <= ulp).all()
+    assert not torch.equal(y.detach(), y0)
+    xm, wm = ocast.new_meta(), ocast.new_meta()
+    xq = ocast.cast_to_fp8(x.detach().cpu(), xm, fp8.E4M3, in_time=True)
+    w16 = ocast.cast_to_fp16(w_ref, wm, in_time=True)
+    wq, wm8 = ocast.scaled_fp16_to_fp8(w16, wm, fp8.E4M3)
+    want = ogemm.fp8_gemm(wq, wm8['scale_inv'], fp8.E4M3, xq, xm['scale_inv'], fp8.E4M3, bias=b_ref.cpu().bfloat16().float())
+    assert rel_fro(y.detach().float(), want) < 1e-2
+
+
 def _check_optimizer_step(torch_cls, lb_cls, diff=3e-4):
     x = torch.randn(4, 4, device='cuda')
     linear = torch.nn.Linear(4, 4).cuda()
