@@ -50,7 +50,8 @@ enum {
 /* flags of msamp_cast_to_fp8_intime / msamp_cast_transpose_intime */
 enum {
     MSAMP_FLAG_NAN_TO_INF = 1, /* amax: NaN/+Inf -> +Inf before the scale rule (cast.py:37-40, sync=True) */
-    MSAMP_FLAG_TWO_PASS = 2    /* never take the one-pass (register-resident, grid-barrier) kernel */
+    MSAMP_FLAG_TWO_PASS = 2,   /* never take the one-pass (register-resident, grid-barrier) kernel */
+    MSAMP_FLAG_NO_SPECULATION = 4 /* in-time casts: do not quantize with the old scale before the new one is known */
 };
 
 /* bytes of device workspace the amax and in-time entry points (msamp_amax, *_intime) need: partial

@@ -26,6 +26,9 @@ __device__ __forceinline__ void amax_publish(float* amax, float v) {
 // (float bit patterns of |x|, NaN patterns included).
 constexpr int kWsPartials = 16;
 constexpr int kMaxPartials = 1024;
+// word kWsSpecDone: non-zero when the first pass of an in-time cast also wrote the output, quantized with the scale
+// in force before the call (word 0); the second pass then only has to run when the rule gives another scale
+constexpr int kWsSpecDone = 9;
 
 struct InTimeArgs {
     const uint32_t* ws;    // nullptr: the scale comes from *scale_p
@@ -39,6 +42,7 @@ struct InTimeArgs {
     float* amax_copy;              // kRescale, nullable: receives a copy of the amax window
     int window;
     int32_t* counter_out;          // kRescale, nullable: set to 0 (the new meta's update count)
+    int speculative;               // kInTime: the first pass may already have written the output (see kWsSpecDone)
 };
 
 // Warm-up gate: the amax kernels of a gated cast run only while *counter < window (in-time scaling);
@@ -95,6 +99,8 @@ __global__ __launch_bounds__(THREADS) void cast_to_fp8_kernel(const IT* __restri
     float s;
     if constexpr (INTIME == kInTime) {
         s = resolve_in_time_scale(it, red, scale_inv);
+        // the first pass quantized with the scale it found in the meta, and the rule confirms that scale: done
+        if (it.speculative && it.ws[kWsSpecDone] != 0u && __float_as_uint(s) == it.ws[0]) return;
     } else if constexpr (INTIME == kRescale) {
         const float s_new = scale_rule(*it.known_amax, 1.0f, it.fp_max, it.margin);
         s = s_new * *it.old_scale_inv;
@@ -252,6 +258,78 @@ __global__ __launch_bounds__(kCastThreads) void amax_partial_kernel(const IT* __
     }
 }
 
+// First pass of the in-time cast of a tensor too large for the one-pass kernel, with the output written on
+// speculation: max|x| per workgroup as above, and every element quantized with the scale the meta holds before the
+// call.  A power-of-two scale rarely changes between two calls on the same meta; when the second pass finds that
+// the rule confirms it, it returns at once and x has been read once (sizeof(in) + 1 bytes per element instead of
+// 2 * sizeof(in) + 1).  Otherwise the second pass quantizes again with the new scale: the same bytes as without
+// speculation, since the output is not an input.  A meta that has never been used (amax 0, scale 1) is not
+// speculated on: the pass then only takes the maxima.
+constexpr int kSpecThreads = 512;
+
+template <typename IT, int FMT>
+__global__ __launch_bounds__(kSpecThreads) void cast_speculative_kernel(const IT* __restrict__ x, uint8_t* __restrict__ out,
+                                                                         size_t n, const float* scale, const float* amax,
+                                                                         uint32_t* ws, int vec_ok) {
+    constexpr int EPT = In16<IT>::EPT;
+    constexpr size_t TILE = static_cast<size_t>(kSpecThreads) * EPT * kCastUnroll;
+    __shared__ uint32_t red[kSpecThreads / kWave];
+    const int tid = threadIdx.x;
+    const float guess = *scale;
+    const bool spec = !(*amax == 0.0f && guess == 1.0f);
+    uint32_t m = 0;
+    const size_t ntiles = (n + TILE - 1) / TILE;
+    for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+        const size_t base = t * TILE;
+        if (vec_ok && base + TILE <= n) {
+            uint4 raw[kCastUnroll];
+#pragma unroll
+            for (int u = 0; u < kCastUnroll; ++u)
+                raw[u] = *reinterpret_cast<const uint4*>(x + base + (static_cast<size_t>(u) * kSpecThreads + tid) * EPT);
+#pragma unroll
+            for (int u = 0; u < kCastUnroll; ++u) {
+                const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if constexpr (sizeof(IT) == 4) m = umax(m, w[j] & 0x7fffffffu);
+                    else m = umax(m, umax((w[j] << 16) & 0x7fff0000u, w[j] & 0x7fff0000u));
+                }
+                if (spec) {
+                    float f[EPT];
+                    In16<IT>::decode(raw[u], f);
+                    uint32_t q[EPT / 4];
+#pragma unroll
+                    for (int j = 0; j < EPT / 4; ++j)
+                        q[j] = quant4<FMT>(f[4 * j] * guess, f[4 * j + 1] * guess, f[4 * j + 2] * guess, f[4 * j + 3] * guess);
+                    uint8_t* o = out + base + (static_cast<size_t>(u) * kSpecThreads + tid) * EPT;
+                    if constexpr (EPT == 4) *reinterpret_cast<uint32_t*>(o) = q[0];
+                    else *reinterpret_cast<uint2*>(o) = make_uint2(q[0], q[1]);
+                }
+            }
+        } else {
+            const size_t end = (base + TILE < n) ? base + TILE : n;
+            for (size_t i = base + tid; i < end; i += kSpecThreads) {
+                if constexpr (sizeof(IT) == 4) {
+                    m = umax(m, reinterpret_cast<const uint32_t*>(x)[i] & 0x7fffffffu);
+                } else {
+                    m = umax(m, (static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(x)[i]) << 16) & 0x7fff0000u);
+                }
+                if (spec) out[i] = static_cast<uint8_t>(quant1<FMT>(Elem<IT>::load(x + i) * guess));
+            }
+        }
+    }
+    m = block_max_u32(m, red);
+    if (tid == 0) {
+        if constexpr (sizeof(IT) == 2 && !__is_same(IT, bf16_t)) m = __float_as_uint(f16_bits_to_float(m >> 16));
+        ws[kWsPartials + blockIdx.x] = m;
+        if (blockIdx.x == 0) {
+            ws[0] = __float_as_uint(guess);
+            ws[1] = gridDim.x;
+            ws[kWsSpecDone] = spec ? 1u : 0u;
+        }
+    }
+}
+
 // reduce the partial maxima into amax[0] (and, if asked, run the scale rule) in one workgroup
 __global__ __launch_bounds__(kCastThreads) void amax_finalize_kernel(const uint32_t* ws, float* amax, float* scale,
                                                                       float* scale_inv, float fp_max, int margin, int flags,
@@ -301,7 +379,13 @@ __device__ __forceinline__ uint32_t abs_bits_hi(uint32_t raw) {    // raw elemen
 
 // R = vectors per lane the kernel is built for (the host picks the smallest of 4 / 8 / 16 that covers the
 // tensor, so that a small tensor does not pay for loads it has no use for).
-template <typename IT, int FMT, int R>
+// SPEC: quantize with the scale in force *before* the meeting and store, then meet: a power-of-two scale rarely
+// changes between two calls on the same meta, and when the rule confirms it the output is already in place --
+// the workgroups never sit idle between an all-loads and an all-stores phase, and early finishers' stores overlap
+// the late ones' loads.  When the scale did change, the run is quantized again from the registers, as without
+// SPEC.  Same bytes either way (the output is not an input).  A meta that has never been used (amax 0, scale 1)
+// is not speculated on.
+template <typename IT, int FMT, int R, bool SPEC>
 __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void cast_intime_resident_kernel(const IT* __restrict__ x,
                                                                            uint8_t* __restrict__ out, size_t n,
                                                                            float* scale, float* amax, float* scale_inv,
@@ -317,7 +401,9 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
     const uint32_t nvec = static_cast<uint32_t>(n / EPT);
     // each workgroup owns one contiguous run of rounds * kResThreads vectors
     const uint32_t v0 = blockIdx.x * static_cast<uint32_t>(rounds) * kResThreads + tid;
-    const float old_scale = *scale;    // read before any workgroup can pass the meeting and replace it
+    // read before any workgroup can pass the meeting and replace them
+    const float old_scale = *scale;
+    const float old_amax = *amax;
 
     uint4 v[R];
 #pragma unroll
@@ -344,12 +430,48 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
         }
     }
     m = block_max_u32(m, red);    // valid in lane 0 of wave 0
-    if (tid < kWave) {
-        if (tid == 0) {
-            if constexpr (sizeof(IT) == 2 && !__is_same(IT, bf16_t)) m = __float_as_uint(f16_bits_to_float(m >> 16));
-            __hip_atomic_store(slots + blockIdx.x, (static_cast<uint64_t>(token) << 32) | m, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) {
+        if constexpr (sizeof(IT) == 2 && !__is_same(IT, bf16_t)) m = __float_as_uint(f16_bits_to_float(m >> 16));
+        __hip_atomic_store(slots + blockIdx.x, (static_cast<uint64_t>(token) << 32) | m, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // quantize this lane's vectors (and the ragged end) with scale q and store them
+    auto emit = [&](float q, auto in_range_c, auto fenced_c) {
+        constexpr bool kInRange = decltype(in_range_c)::value, kFenced = decltype(fenced_c)::value;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            // after the meeting: keep only the raw words live across it, not values derived from them before it
+            if constexpr (kFenced) asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
+            const uint32_t idx = v0 + r * kResThreads;
+            if (r < rounds && idx < nvec) {
+                float f[EPT];
+                In16<IT>::decode(v[r], f);
+                uint32_t w[EPT / 4];
+#pragma unroll
+                for (int j = 0; j < EPT / 4; ++j) {
+                    if constexpr (kInRange) w[j] = quant4_in_range<FMT>(f[4 * j] * q, f[4 * j + 1] * q, f[4 * j + 2] * q, f[4 * j + 3] * q);
+                    else w[j] = quant4<FMT>(f[4 * j] * q, f[4 * j + 1] * q, f[4 * j + 2] * q, f[4 * j + 3] * q);
+                }
+                if constexpr (EPT == 4) reinterpret_cast<uint32_t*>(out)[idx] = w[0];
+                else reinterpret_cast<uint2*>(out)[idx] = make_uint2(w[0], w[1]);
+            }
         }
+        if (has_tail) {
+            float a;
+            if constexpr (sizeof(IT) == 4) a = __uint_as_float(tail_raw);
+            else if constexpr (__is_same(IT, bf16_t)) a = __uint_as_float(static_cast<uint32_t>(tail_raw) << 16);
+            else a = f16_bits_to_float(tail_raw);
+            out[tail0 + tid] = static_cast<uint8_t>(quant1<FMT>(a * q));
+        }
+    };
+    bool speculated = false;
+    if constexpr (SPEC) {
+        speculated = !(old_amax == 0.0f && old_scale == 1.0f);
+        if (speculated) emit(old_scale, std::false_type{}, std::false_type{});
+    }
+
+    if (tid < kWave) {
         // Workgroup 0 collects: it alone polls the slots (everyone polling them costs the workgroups still
         // loading a good part of their bandwidth), derives amax and scale and posts both, tagged with the
         // token, in two words behind the slots; the others poll only those.
@@ -382,8 +504,9 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
                 if (!all_in) {
                     am = __uint_as_float(0x7fc00000u);
                     report_wait_expired(error_word, kErrCollectorGaveUp);
+                } else if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) {
+                    am = __uint_as_float(0x7f800000u);
                 }
-                else if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
                 const float s = scale_rule(am, old_scale, fp_max, margin);
                 const uint64_t tag = static_cast<uint64_t>(token) << 32;
                 __hip_atomic_store(post, tag | __float_as_uint(am), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -411,50 +534,16 @@ __global__ __launch_bounds__(kResThreads) __attribute__((amdgpu_waves_per_eu(4, 
     }
     __syncthreads();
     const float s = __uint_as_float(s_scale);
+    if constexpr (SPEC) {
+        // the scale the output was written with stands: done.  Otherwise let those stores land before writing again.
+        if (speculated && __float_as_uint(s) == __float_as_uint(old_scale)) return;
+        if (speculated) __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0): loads and stores share the counter here
+    }
     // With a positive finite amax and the scale the rule derived from it, every |x| * s stays within the
     // format and nothing is NaN: the clamp and the NaN patch can go.
     const bool in_range = __uint_as_float(s_amax) * s <= fp_max && __uint_as_float(s_amax) > 0.0f;
-
-    if (in_range) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            // keep only the raw words live across the barrier, not values derived from them before it
-            asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
-            const uint32_t idx = v0 + r * kResThreads;
-            if (r < rounds && idx < nvec) {
-                float f[EPT];
-                In16<IT>::decode(v[r], f);
-                uint32_t w[EPT / 4];
-#pragma unroll
-                for (int j = 0; j < EPT / 4; ++j)
-                    w[j] = quant4_in_range<FMT>(f[4 * j] * s, f[4 * j + 1] * s, f[4 * j + 2] * s, f[4 * j + 3] * s);
-                if constexpr (EPT == 4) reinterpret_cast<uint32_t*>(out)[idx] = w[0];
-                else reinterpret_cast<uint2*>(out)[idx] = make_uint2(w[0], w[1]);
-            }
-        }
-    } else {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            asm volatile("" : "+v"(v[r].x), "+v"(v[r].y), "+v"(v[r].z), "+v"(v[r].w));
-            const uint32_t idx = v0 + r * kResThreads;
-            if (r < rounds && idx < nvec) {
-                float f[EPT];
-                In16<IT>::decode(v[r], f);
-                uint32_t w[EPT / 4];
-#pragma unroll
-                for (int j = 0; j < EPT / 4; ++j) w[j] = quant4<FMT>(f[4 * j] * s, f[4 * j + 1] * s, f[4 * j + 2] * s, f[4 * j + 3] * s);
-                if constexpr (EPT == 4) reinterpret_cast<uint32_t*>(out)[idx] = w[0];
-                else reinterpret_cast<uint2*>(out)[idx] = make_uint2(w[0], w[1]);
-            }
-        }
-    }
-    if (has_tail) {
-        float a;
-        if constexpr (sizeof(IT) == 4) a = __uint_as_float(tail_raw);
-        else if constexpr (__is_same(IT, bf16_t)) a = __uint_as_float(static_cast<uint32_t>(tail_raw) << 16);
-        else a = f16_bits_to_float(tail_raw);
-        out[tail0 + tid] = static_cast<uint8_t>(quant1<FMT>(a * s));
-    }
+    if (in_range) emit(s, std::true_type{}, std::true_type{});
+    else emit(s, std::false_type{}, std::true_type{});
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -968,7 +1057,7 @@ static bool fits_resident(const void* fn) {
 }
 
 // One-pass (register-resident) in-time cast; returns 1 if it does not apply and the two-pass path must run.
-template <typename IT>
+template <typename IT, bool SPEC>
 static int launch_resident(const IT* x, size_t n, float* scale, float* amax, float* scale_inv, uint8_t* out,
                            int fp8_type, int margin, int flags, void* ws, hipStream_t st) {
     constexpr int EPT = 16 / sizeof(IT);
@@ -993,8 +1082,8 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
     bool fits = true;
 #define LAUNCH(FMT, R) \
     do { \
-        fits = fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, FMT, R>)); \
-        if (fits) hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT, R>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit, error_word); \
+        fits = fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, FMT, R, SPEC>)); \
+        if (fits) hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT, R, SPEC>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit, error_word); \
     } while (0)
 #define LAUNCH_R(FMT) \
     do { if (rounds <= 4) LAUNCH(FMT, 4); else if (rounds <= 8) LAUNCH(FMT, 8); else LAUNCH(FMT, kResVecs); } while (0)
@@ -1008,15 +1097,51 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
 
 static int dispatch_resident(const void* x, int dtype, size_t n, float* scale, float* amax, float* scale_inv, uint8_t* out,
                              int fp8_type, int margin, int flags, void* ws, hipStream_t st) {
+    const bool spec = !(flags & MSAMP_FLAG_NO_SPECULATION);
+#define RESIDENT(T) \
+    (spec ? launch_resident<T, true>(static_cast<const T*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st) \
+          : launch_resident<T, false>(static_cast<const T*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st))
     switch (dtype) {
         case MSAMP_DT_F32:
-            return launch_resident(static_cast<const float*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st);
+            return RESIDENT(float);
         case MSAMP_DT_F16:
-            return launch_resident(static_cast<const f16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st);
+            return RESIDENT(f16_t);
         case MSAMP_DT_BF16:
-            return launch_resident(static_cast<const bf16_t*>(x), n, scale, amax, scale_inv, out, fp8_type, margin, flags, ws, st);
+            return RESIDENT(bf16_t);
     }
+#undef RESIDENT
     return 1;
+}
+
+template <typename IT>
+static int launch_speculative(const IT* x, size_t n, const float* scale, const float* amax, uint8_t* out, int fp8_type,
+                              uint32_t* ws, hipStream_t st) {
+    constexpr int EPT = In16<IT>::EPT;
+    const int vec_ok = aligned(x, 16) && aligned(out, EPT);
+    int grid = grid_for(n, static_cast<size_t>(kSpecThreads) * EPT * kCastUnroll);
+    const int cap = cu_count() * 2 < kMaxPartials ? cu_count() * 2 : kMaxPartials;
+    grid = grid < cap ? grid : cap;
+    if (fp8_type == MSAMP_DT_E4M3)
+        hipLaunchKernelGGL((cast_speculative_kernel<IT, MSAMP_DT_E4M3>), dim3(grid), dim3(kSpecThreads), 0, st, x, out, n, scale, amax, ws, vec_ok);
+    else
+        hipLaunchKernelGGL((cast_speculative_kernel<IT, MSAMP_DT_E5M2>), dim3(grid), dim3(kSpecThreads), 0, st, x, out, n, scale, amax, ws, vec_ok);
+    MSAMP_CHECK_LAUNCH("cast_speculative_kernel");
+    return MSAMP_OK;
+}
+
+static int dispatch_speculative(const void* x, int dtype, size_t n, const float* scale, const float* amax, uint8_t* out,
+                                int fp8_type, void* ws, hipStream_t st) {
+    uint32_t* w = static_cast<uint32_t*>(ws);
+    switch (dtype) {
+        case MSAMP_DT_F32:
+            return launch_speculative(static_cast<const float*>(x), n, scale, amax, out, fp8_type, w, st);
+        case MSAMP_DT_F16:
+            return launch_speculative(static_cast<const f16_t*>(x), n, scale, amax, out, fp8_type, w, st);
+        case MSAMP_DT_BF16:
+            return launch_speculative(static_cast<const bf16_t*>(x), n, scale, amax, out, fp8_type, w, st);
+    }
+    set_error("unsupported input dtype %d", dtype);
+    return MSAMP_ERR_DTYPE;
 }
 
 static int finalize_amax(void* ws, float* amax, float* scale, float* scale_inv, float fp_max, int margin, int flags,
@@ -1288,9 +1413,11 @@ int msamp_cast_to_fp8_intime(const void* x, int in_dtype, size_t n, float* scale
     hipStream_t st = static_cast<hipStream_t>(stream);
     int rc = dispatch_resident(x, in_dtype, n, scale, amax, scale_inv, out, fp8_type, margin, flags, workspace, st);
     if (rc <= 0) return rc;
-    rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
+    const int speculative = (flags & MSAMP_FLAG_NO_SPECULATION) ? 0 : 1;
+    if (speculative) rc = dispatch_speculative(x, in_dtype, n, scale, amax, out, fp8_type, workspace, st);
+    else rc = dispatch_amax(x, in_dtype, n, workspace, scale, st);
     if (rc != MSAMP_OK) return rc;
-    const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags, nullptr, nullptr, nullptr, 0, nullptr};
+    const InTimeArgs it = {static_cast<const uint32_t*>(workspace), scale, amax, fp8_max(fp8_type), margin, flags, nullptr, nullptr, nullptr, 0, nullptr, speculative};
     return dispatch_cast(x, in_dtype, n, scale, nullptr, scale_inv, out, fp8_type, &it, st);
 }
 

@@ -17,6 +17,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 DT_F32, DT_F16, DT_BF16, DT_E4M3, DT_E5M2 = 2, 3, 4, 5, 6
 FLAG_NAN_TO_INF = 1
 FLAG_TWO_PASS = 2
+FLAG_NO_SPECULATION = 4
 WORKSPACE_BYTES = 16384
 ADAMW_CHUNK = 16384
 
@@ -279,16 +280,18 @@ def _shared_device():
     return dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1
 
 
-def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_inf=False, two_pass=False):
+def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_inf=False, two_pass=False, speculate=True):
     """amax, scale rule, quantize and reciprocal in one call.  `two_pass` keeps the call off the
-    one-pass kernel whose workgroups wait for each other (same results either way)."""
+    one-pass kernel whose workgroups wait for each other; `speculate=False` keeps the kernels from
+    writing the output with the old scale before the new one is known (same results either way)."""
     lib = load()
     _gpu(x, 'input')
     out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
     _check(
         lib.msamp_cast_to_fp8_intime(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
-            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _two_pass_only() else 0),
+            (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if two_pass or _two_pass_only() else 0) |
+            (0 if speculate else FLAG_NO_SPECULATION),
             _ptr(workspace(x.device)),
             _stream()
         ), 'msamp_cast_to_fp8_intime'

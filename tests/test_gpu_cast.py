@@ -426,3 +426,59 @@ def test_window_update_sequence(be):
         bad = be.scale_update(scales, amaxs, 448.0, 0).cpu().bool()
         o_bad = scaling.update_scaling_factors(o_scales, o_amaxs, o_cnt, 448.0)
         assert torch.equal(bad, o_bad) and same_float(scales, o_scales) and same_float(amaxs, o_amaxs)
+
+
+def _spec_sequence(be, xs, fp8_dt, two_pass, nan_to_inf=False):
+    """The same calls on two metas: with speculation (the default) and with the plain kernels; everything must agree
+    after every call.  Returns the speculative side's outputs and meta snapshots."""
+    ms, mr = make_meta(), make_meta()
+    outs = []
+    for x in xs:
+        q = be.cast_to_fp8_intime(x, ms[0], ms[2][0:1], ms[1], fp8_dt, two_pass=two_pass, nan_to_inf=nan_to_inf)
+        r = be.cast_to_fp8_intime(x, mr[0], mr[2][0:1], mr[1], fp8_dt, two_pass=True, speculate=False, nan_to_inf=nan_to_inf)
+        torch.cuda.synchronize()
+        assert torch.equal(q, r)
+        assert same_float(ms[0], mr[0]) and same_float(ms[1], mr[1]) and same_float(ms[2], mr[2])
+        outs.append((q, ms[0].clone(), ms[1].clone(), ms[2].clone()))
+    return outs
+
+
+@pytest.mark.parametrize('two_pass', [False, True])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('fmt,dt', [(fp8.E4M3, 5), (fp8.E5M2, 6)])
+def test_speculative_in_time_cast_hit_miss_and_special_values(be, dtype, two_pass, fmt, dt):
+    """Speculation on the old scale (one-pass kernel: stores before the meeting; two-pass: stores in the first pass):
+    never-used meta, confirmed scale, changed scale (both directions), NaN / Inf / all-zero inputs, a ragged length --
+    bit-equal to the plain kernels after every call, and to the oracle."""
+    g = torch.Generator().manual_seed(21)
+    n = 1024 * 1024 + 13
+    x = (torch.randn(n, generator=g) * 3).to(dtype)
+    bad = x.clone()
+    bad[17], bad[n - 1] = float('nan'), float('inf')
+    inf = x.clone()
+    inf[5] = -float('inf')
+    cpu = [x, x, x * 8, x * 8, (x.float() * 2.0**-6).to(dtype), bad, x, torch.zeros(n, dtype=dtype), inf, x[:1000], x[:3]]
+    outs = _spec_sequence(be, [c.cuda() for c in cpu], dt, two_pass)
+    om = oracle_meta()
+    for c, (q, s, si, am) in zip(cpu, outs):
+        want = ocast.cast_to_fp8(c, om, fmt, in_time=True)
+        assert torch.equal(q.cpu(), want)
+        assert same_float(s, om['scale']) and same_float(si, om['scale_inv']) and same_float(am[0], om['amax'][0])
+    _spec_sequence(be, [c.cuda() for c in cpu[:6]], dt, two_pass, nan_to_inf=True)
+
+
+@pytest.mark.parametrize('dtype,n', [(torch.float32, 17 * 1024 * 1024 + 9), (torch.bfloat16, 34 * 1024 * 1024 + 24)])
+def test_speculative_in_time_cast_beyond_the_one_pass_limit(be, dtype, n):
+    """More than 64 MiB of input: two launches, the first one writing the output on speculation."""
+    g = torch.Generator(device='cuda').manual_seed(22)
+    x = (torch.randn(n, device='cuda', generator=g) * 0.01).to(dtype)
+    y = x.clone()
+    y[n // 3] = 50.0
+    outs = _spec_sequence(be, [x, x, y, y, x], be.DT_E4M3, False)
+    # the oracle on the first 2 Mi elements of the confirmed-scale call and of the changed-scale call
+    head = 2 * 1024 * 1024
+    for idx, src in ((1, x), (2, y)):
+        q, s, si, am = outs[idx]
+        assert am[0].item() == src.float().abs().max().item()
+        want = fp8.encode(src[:head].float().cpu() * s.cpu(), fp8.E4M3)
+        assert torch.equal(q[:head].cpu(), want)
