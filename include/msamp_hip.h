@@ -248,8 +248,8 @@ int msamp_fp8_gemm(const uint8_t* a, int a_type, const float* a_scale_inv, const
  * with M contiguous, likewise b_kmajor for [K][N].  The backward GEMMs of a linear layer
  * (nn/functional.py:84-111 of the reference) then read W, x and dy as they are, and the explicit FP8
  * transposes (transformer_engine_wrapper.py:165-176) are not needed.  Results are bit-identical to
- * msamp_fp8_gemm on transposed copies (every kernel behind these entry points adds up the same 64-byte blocks of K
- * in ascending order).  Supported: a K-major alone, or both; k % 128 == 0 and the row
+ * msamp_fp8_gemm on transposed copies (every kernel behind these entry points adds up the same 128-byte blocks of K
+ * in ascending order).  Supported: a K-major alone, or both; k a multiple of 128 and at least 256, and the row
  * count of every K-major operand (m, and n if b_kmajor) a multiple of 256; otherwise MSAMP_ERR_SHAPE. */
 int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
                           int b_type, const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int m, int n, int k,
@@ -262,7 +262,7 @@ int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv
  * msamp_fp8_gemm_kmajor into a d_dtype buffer followed by msamp_cast_to_fp8_intime of that buffer gives, without the
  * buffer.  flags and workspace as for msamp_cast_to_fp8_intime.
  * Returns MSAMP_NOT_FUSED (1), having done nothing, when the fused form does not apply and the caller has to take
- * the two steps: it needs m and n multiples of 256, k a multiple of 128, at most one 256 x 256 output tile per
+ * the two steps: it needs m and n multiples of 256, k a multiple of 128 and at least 256, at most one 256 x 256 output tile per
  * compute unit (its workgroups wait for each other), q_type E4M3, both operands K-major or neither, a stream on which
  * such kernels are allowed (not capturing, the device's first), and no MSAMP_FLAG_TWO_PASS. */
 #define MSAMP_NOT_FUSED 1

@@ -16,7 +16,7 @@ static int dispatch_pair(int x_type, int y_type, const GemmCall& c) {
 // K-major operands: only the direct-to-LDS kernel reads them, so the shape must suit it
 static bool kmajor_shape_ok(int NR, int NC, int K, bool xt, bool yt) {
     const bool fits32 = static_cast<unsigned long long>(NR) * K < (1ull << 32) && static_cast<unsigned long long>(NC) * K < (1ull << 32);
-    return K % kBK == 0 && fits32 && (!xt || NR % kDmaTile == 0) && (!yt || NC % kDmaTile == 0);
+    return K % kBK == 0 && K >= 2 * kBK && fits32 && (!xt || NR % kDmaTile == 0) && (!yt || NC % kDmaTile == 0);
 }
 
 }    // namespace msamp
@@ -39,7 +39,7 @@ extern "C" int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_
     const bool both = a_kmajor && b_kmajor, neither = !a_kmajor && !b_kmajor;
     const long tiles = static_cast<long>(n / kDmaTile) * (m / kDmaTile);
     const bool fits32 = static_cast<unsigned long long>(n) * k < (1ull << 32) && static_cast<unsigned long long>(m) * k < (1ull << 32);
-    if (q_type != MSAMP_DT_E4M3 || !(both || neither) || m % kDmaTile || n % kDmaTile || k % kBK || !fits32 ||
+    if (q_type != MSAMP_DT_E4M3 || !(both || neither) || m % kDmaTile || n % kDmaTile || k % kBK || k < 2 * kBK || !fits32 ||
         tiles > cu_count() || tiles > kMaxSlots || workspace == nullptr || (flags & MSAMP_FLAG_TWO_PASS))
         return MSAMP_NOT_FUSED;
     if (!waiting_kernels_allowed(st)) return MSAMP_NOT_FUSED;
@@ -65,7 +65,7 @@ extern "C" int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* 
     MSAMP_REQUIRE(bias == nullptr || is_hp(bias_dtype), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_kmajor: bias dtype %d", bias_dtype);
     MSAMP_REQUIRE(a_kmajor, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_kmajor: b may be K-major only together with a");
     MSAMP_REQUIRE(m > 0 && n > 0 && k > 0 && kmajor_shape_ok(n, m, k, b_kmajor != 0, true), MSAMP_ERR_SHAPE,
-                  "msamp_fp8_gemm_kmajor: m=%d n=%d k=%d (k %% 128 and the K-major operands' rows %% 256 must be 0)", m, n, k);
+                  "msamp_fp8_gemm_kmajor: m=%d n=%d k=%d (k must be a multiple of 128 and at least 256, the K-major operands' rows multiples of 256)", m, n, k);
     MSAMP_REQUIRE(a && b && d && a_scale_inv && b_scale_inv, MSAMP_ERR_NULL, "msamp_fp8_gemm_kmajor: null pointer");
     MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16), MSAMP_ERR_SHAPE, "msamp_fp8_gemm_kmajor: operands must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);

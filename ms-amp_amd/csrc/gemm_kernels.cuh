@@ -20,7 +20,6 @@ namespace msamp {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int kGemmThreads = 256;
 
@@ -70,11 +69,15 @@ __device__ __forceinline__ v8i read_frag(const uint8_t* lds, int row, int kc) {
     return f;
 }
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// 16 x 16 x 128 FP8 MFMA (the non-scaled form: block scales 0).  On this part it sustains about a tenth more
+// throughput under the power limit than the 32 x 32 x 64 form on the same data.
 template <int XF, int YF>
-__device__ __forceinline__ v16f mfma(const v8i& x, const v8i& y, const v16f& c) {
+__device__ __forceinline__ v4f mfma16(const v8i& x, const v8i& y, const v4f& c) {
     constexpr int cb = (XF == MSAMP_DT_E4M3) ? 0 : 1;
     constexpr int bl = (YF == MSAMP_DT_E4M3) ? 0 : 1;
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, cb, bl, 0, 0, 0, 0);
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, c, cb, bl, 0, 0, 0, 0);
 }
 
 template <typename OT>
@@ -113,7 +116,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
                                                                  const float* __restrict__ y_scale_inv, int accumulate,
                                                                  const void* __restrict__ bias, int bias_dt) {
     constexpr int WR = BR / 2, WC = BC / 2;    // wave tile
-    constexpr int TR = WR / 32, TC = WC / 32;  // MFMA tiles per wave
+    constexpr int TR = WR / 16, TC = WC / 16;  // MFMA tiles per wave
     constexpr int kStage = (BR + BC) * kBK;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -122,20 +125,20 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
     const int row0 = tr * BR, col0 = tc * BC;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wr = wave >> 1, wc = wave & 1;
-    const int l32 = lane & 31, lh = lane >> 5;
+    const int l16 = lane & 15, g4 = lane >> 4;
 
-    v16f acc[TR][TC];
+    v4f acc[TR][TC];
 #pragma unroll
     for (int i = 0; i < TR; ++i)
 #pragma unroll
         for (int j = 0; j < TC; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
     TileLoader<BR, KGUARD> lx;
     TileLoader<BC, KGUARD> ly;
     const int nk = (K + kBK - 1) / kBK;
-    // The K slices are walked in ascending order, 64 bytes of K per MFMA, exactly as the direct-to-LDS kernel below
+    // The K slices are walked in ascending order, 128 bytes of K per MFMA, exactly as the direct-to-LDS kernel below
     // walks them: the two kernels add up the same blocks in the same order and agree to the bit.  (Walking them in
     // an order rotated per workgroup, to spread the memory channels, was measured slower: 2-4 % at 2048 x 2048 x 4096,
     // 10-14 % at 4096 x 4096 x 4112.)
@@ -153,17 +156,17 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
             lx.gload(X, row0, NR, K, slice(kt + 1));
             ly.gload(Y, col0, NC, K, slice(kt + 1));
         }
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        {
+            // a lane holds, for row lane % 16 of a 16-row block, the 32 K-bytes (lane / 16) * 32 .. + 31 of the slice
             v8i fx[TR], fy[TC];
 #pragma unroll
-            for (int i = 0; i < TR; ++i) fx[i] = read_frag(sx, wr * WR + i * 32 + l32, ks * 2 + lh);
+            for (int i = 0; i < TR; ++i) fx[i] = read_frag(sx, wr * WR + i * 16 + l16, g4);
 #pragma unroll
-            for (int j = 0; j < TC; ++j) fy[j] = read_frag(sy, wc * WC + j * 32 + l32, ks * 2 + lh);
+            for (int j = 0; j < TC; ++j) fy[j] = read_frag(sy, wc * WC + j * 16 + l16, g4);
 #pragma unroll
             for (int i = 0; i < TR; ++i)
 #pragma unroll
-                for (int j = 0; j < TC; ++j) acc[i][j] = mfma<XF, YF>(fx[i], fy[j], acc[i][j]);
+                for (int j = 0; j < TC; ++j) acc[i][j] = mfma16<XF, YF>(fx[i], fy[j], acc[i][j]);
         }
         if (kt + 1 < nk) {
             uint8_t* nx = smem + ((kt + 1) & 1) * kStage;
@@ -173,17 +176,18 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* _
         __syncthreads();
     }
 
+    // srcA = X rows: a lane holds D column (Y row) lane % 16 of a block and the four D rows (lane / 16) * 4 .. + 3
     const float alpha = (*x_scale_inv) * (*y_scale_inv);
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
-        const int col = col0 + wc * WC + j * 32 + l32;
+        const int col = col0 + wc * WC + j * 16 + l16;
         if (col >= NC) continue;
         const float bv = bias != nullptr ? load_bias(bias, bias_dt, col) : 0.0f;
 #pragma unroll
         for (int i = 0; i < TR; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = row0 + wr * WR + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+            for (int r = 0; r < 4; ++r) {
+                const int row = row0 + wr * WR + i * 16 + g4 * 4 + r;
                 if (row < NR) {
                     store_out<OT>(D + static_cast<size_t>(row) * NC + col, fmaf(acc[i][j][r], alpha, bv), accumulate != 0);
                 }
@@ -231,14 +235,14 @@ __device__ __noinline__ void store_quad_slow(OT* D, int row, int col, int NR, in
 
 // ---------------------------------------------------------------------------------------------
 // Main kernel: 256 x 256 output tile over 128-byte K slices, four wavefronts each owning a 128 x 128
-// quadrant (16 accumulators of the 32x32x64 FP8 MFMA = 256 accumulation registers per lane).
+// quadrant (8 x 8 accumulators of the 16x16x128 FP8 MFMA = 256 accumulation registers per lane).
 //  * Tiles travel global -> LDS with the direct-to-LDS load: no staging registers, no LDS stores.  A
 //    lane group of 8 fetches one whole 128-byte line (full-line requests are what the L2 serves best).
-//  * Two 64 KiB LDS stages.  A slice is computed in two 64-byte sub-steps; the fragments of the next
-//    sub-step are read while the 16 MFMAs of the current one execute (two register buffers).
-//  * One workgroup barrier per slice, between the sub-steps: by then every wave holds the whole slice
-//    in registers, so the stage is refilled right away with the slice after next (all 16 loads during
-//    the second sub-step, which leaves them a whole sub-step to land).
+//  * Two 64 KiB LDS stages.  A slice is computed in four quarters of 16 MFMAs (X half x Y half); the fragment
+//    half the next quarters need is read while the current one executes.
+//  * One workgroup barrier per slice, after the second quarter: by then every wave holds the whole slice
+//    in registers, so the stage is refilled right away with the slice after next (its 16 loads spread over
+//    the last two quarters, which leaves them half a slice to land).
 //  * LDS reads and tile loads are interleaved with the MFMAs one at a time, so that neither the LDS nor
 //    the vector-memory queue backs up and stalls the MFMA stream.
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -285,7 +289,7 @@ __device__ __forceinline__ void round_pair(float a, float b, float& ra, float& r
     }
 }
 
-template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0>
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0, bool ODD_NK = false>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
                                                                      const uint8_t* __restrict__ Y, OT* __restrict__ D,
                                                                      int NR, int NC, int K,
@@ -299,7 +303,6 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     const int row0 = tr * kDmaTile, col0 = tc * kDmaTile;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wr = wave >> 1, wc = wave & 1;
-    const int l32 = lane & 31, lh = lane >> 5;
     // the output factor is fetched now: left to the epilogue, the two scalar loads sit on its critical path
     float alpha_early = (*x_scale_inv) * (*y_scale_inv);
     asm volatile("" : "+v"(alpha_early));
@@ -341,123 +344,144 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + off) : "memory", "m0");
     };
 
-    // ---- LDS -> fragments.  Row-major operand: this lane's row inside a 32-row block and its swizzled
-    // 16-byte chunks.  K-major operand: the address this lane contributes to a transposing read.
+    // ---- LDS -> fragments of the 16x16x128 MFMA: a lane holds, for row lane % 16 of a 16-row block, the 32 K-bytes
+    // (lane / 16) * 32 .. + 31 of the 128-byte slice.  Row-major operand: two 16-byte reads at the swizzled chunks
+    // 2 * (lane / 16) and + 1.  K-major operand: four transposing reads, each handing a 16-lane group eight
+    // consecutive k of 16 rows.
     const int fsw = (lane & 7) ^ ((lane >> 3) & 1);
-    const int off_a = ((2 * lh) ^ fsw) << 4;    // sub-step 0, low half; high half is ^16, sub-step 1 is ^64
-    const int xrow = (wr * 128 + l32) * kBK;
-    const int yrow = kDmaTile * kBK + (wc * 128 + l32) * kBK;
-    const int i16 = lane & 15, tj = i16 >> 1, g1 = (lane >> 4) & 1;
-    const int t_lane = (lh * 32 + tj) * 256 + (i16 & 1) * 8;    // k-row and 8-byte half of this lane's address
-    // A sub-step needs 8 fragments of 8 registers (X blocks 0..3, Y blocks 0..3).  They arrive in pieces:
-    // two 16-byte reads per fragment of a row-major operand, four 8-byte transposing reads otherwise.
-    constexpr int kPX = XT ? 16 : 8, kPY = YT ? 16 : 8, kPieces = kPX + kPY;
-    auto read_piece = [&](int* dst, int stage, int ks, int p) {
-        const bool is_x = p < kPX;
-        const int q = is_x ? p : p - kPX;
+    const int l16 = lane & 15, g4 = lane >> 4;
+    const int off_lo = ((2 * g4) ^ fsw) << 4;    // low 16 bytes of this lane's 32; the high ones are at ^ 16
+    const int xrow = (wr * 128 + l16) * kBK;
+    const int yrow = kDmaTile * kBK + (wc * 128 + l16) * kBK;
+    const int tj = l16 >> 1;
+    const int t_lane = (g4 * 32 + tj) * 256 + (l16 & 1) * 8;    // k-row and 8-byte half of this lane's address
+    // The wave's 128 x 128 quadrant is 8 x 8 blocks of 16 x 16.  Fragments are kept by halves: fx[h] / fy[h] hold the
+    // four 16-row blocks 4h .. 4h+3 of X / Y (8 registers each).  A half arrives in pieces: two 16-byte reads per
+    // block of a row-major operand, four 8-byte transposing reads otherwise.
+    constexpr int kPX = XT ? 16 : 8, kPY = YT ? 16 : 8;
+    auto read_piece = [&](int* dst, int stage, bool is_x, int half, int p) {
         const uint8_t* base = smem + stage * kDmaStage;
         if ((is_x && !XT) || (!is_x && !YT)) {
-            const int blk = q >> 1, hf = q & 1;
-            const v4i val = *reinterpret_cast<const v4i*>(base + (is_x ? xrow : yrow) + blk * 32 * kBK +
-                                                          ((off_a ^ (ks * 64)) ^ (hf * 16)));
-            int* d = dst + ((is_x ? 0 : 4) + blk) * 8 + hf * 4;
+            const int b = p >> 1, hf = p & 1;
+            const v4i val = *reinterpret_cast<const v4i*>(base + (is_x ? xrow : yrow) + (half * 4 + b) * 16 * kBK +
+                                                          (off_lo ^ (hf * 16)));
+            int* d = dst + b * 8 + hf * 4;
             d[0] = val[0], d[1] = val[1], d[2] = val[2], d[3] = val[3];
         } else {
-            const int blk = q >> 2, qq = q & 3;
+            const int b = p >> 2, qq = p & 3;
             const int wq = is_x ? wr : wc;
-            const int addr = (is_x ? 0 : kDmaTile * kBK) + t_lane + (ks * 64 + qq * 8) * 256 + wq * 128 +
-                             (((blk * 2 + g1) ^ tj) << 4);
+            const int addr = (is_x ? 0 : kDmaTile * kBK) + t_lane + (qq * 8) * 256 + wq * 128 + (((half * 4 + b) ^ tj) << 4);
             const v2i val = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
                 (__attribute__((address_space(3))) v2i*)(base + addr));
-            int* d = dst + ((is_x ? 0 : 4) + blk) * 8 + qq * 2;
+            int* d = dst + b * 8 + qq * 2;
             d[0] = val[0], d[1] = val[1];
         }
     };
 
-    v16f acc[4][4];
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    v4f acc[8][8];    // acc[i][j]: D rows i * 16 + lane % 16, D columns j * 16 + (lane / 16) * 4 .. + 3 of the quadrant
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 8; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
     const int nk = K / kBK;
-    int fa[64], fb[64];    // fragments [X0..X3, Y0..Y3] x 8 registers, two buffers
+    int fx[2][32], fy[2][32];
 
-    // One sub-step: 16 MFMAs on `cur`, the fragment reads of the next sub-step into `nxt` and, if asked for, the
-    // 16 tile loads of slice ld_kt, one per MFMA.
-    // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row l%32, four
-    // consecutive D columns per register quad -- the layout the epilogue wants.
-    auto sub_step = [&](const int* cur, int* nxt, int rd_stage, int rd_ks, bool do_read, int ld_kt, int ld_stage,
-                        bool do_load) {
+    // One quarter of a slice: the 16 MFMAs of X half hx against Y half hy, with the reads of one fragment half
+    // (rd_x / rd_half from rd_stage into rd_dst) spread between them and, if asked for, eight of the 16 tile loads
+    // of slice ld_kt (ld_first .. ld_first + 7), one every other MFMA.
+    // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row lane % 16 of a block, four
+    // consecutive D columns -- the layout the epilogue wants.
+    auto quarter = [&](int hx, int hy, int* rd_dst, int rd_stage, bool rd_x, int rd_half, bool do_read, int ld_kt,
+                       int ld_stage, int ld_first, bool do_load) {
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
+        const int np = rd_x ? kPX : kPY;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {    // the Y fragment stays for four MFMAs in a row (measured 1 % faster than X staying)
+        for (int j = 0; j < 4; ++j) {    // the Y fragment stays for four MFMAs in a row
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int n = j * 4 + i;
-                const int* cx = cur + i * 8;
-                const int* cy = cur + (4 + j) * 8;
-                const v8i fx = {cx[0], cx[1], cx[2], cx[3], cx[4], cx[5], cx[6], cx[7]};
-                const v8i fy = {cy[0], cy[1], cy[2], cy[3], cy[4], cy[5], cy[6], cy[7]};
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fy, fx, acc[i][j], cb, bl, 0, 0, 0, 0);
+                const int* cx = fx[hx] + i * 8;
+                const int* cy = fy[hy] + j * 8;
+                const v8i vx = {cx[0], cx[1], cx[2], cx[3], cx[4], cx[5], cx[6], cx[7]};
+                const v8i vy = {cy[0], cy[1], cy[2], cy[3], cy[4], cy[5], cy[6], cy[7]};
+                acc[hx * 4 + i][hy * 4 + j] =
+                    __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vy, vx, acc[hx * 4 + i][hy * 4 + j], cb, bl, 0, 0, 0, 0);
                 if (do_read) {
 #pragma unroll
-                    for (int p = n * kPieces / 16; p < (n + 1) * kPieces / 16; ++p) read_piece(nxt, rd_stage, rd_ks, p);
+                    for (int p = n * np / 16; p < (n + 1) * np / 16; ++p) read_piece(rd_dst, rd_stage, rd_x, rd_half, p);
                 }
-                if (do_load) dma(ld_kt, ld_stage, n);
+                if (do_load && (n & 1)) dma(ld_kt, ld_stage, ld_first + (n >> 1));
             }
         }
+    };
+    // keeps the compiler's schedule to "one MFMA, then the LDS reads that belong to it"
+    auto pace = [&](bool rd_x, bool do_read) {
         static_for<16>([&](auto nc) {
             constexpr int n = decltype(nc)::value;
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, (n + 1) * kPieces / 16 - n * kPieces / 16, 0);    // its LDS reads
+            if (do_read) {
+                if (rd_x) __builtin_amdgcn_sched_group_barrier(0x100, (n + 1) * kPX / 16 - n * kPX / 16, 0);    // its LDS reads
+                else __builtin_amdgcn_sched_group_barrier(0x100, (n + 1) * kPY / 16 - n * kPY / 16, 0);
+            }
         });
     };
+    // Slice kt sits in stage st and slice kt + 1 is on its way into the other stage; X half 0 and Y half 0 of slice
+    // kt are in registers.  Quarters 1, 2: X0 x Y0 while Y half 1 arrives, X0 x Y1 while X half 1 arrives -- all of
+    // slice kt is in registers now.  Barrier: slice kt + 1 has landed and nobody needs the LDS copy of slice kt.
+    // Quarters 3, 4: X1 x Y0 while X half 0 of slice kt + 1 arrives, X1 x Y1 while its Y half 0 arrives; the stage of
+    // slice kt is refilled with slice kt + 2 meanwhile.
+    auto slice = [&](int st, bool has_next, int ld_kt, bool do_load) {
+        quarter(0, 0, fy[1], st, false, 1, true, 0, 0, 0, false);
+        pace(false, true);
+        quarter(0, 1, fx[1], st, true, 1, true, 0, 0, 0, false);
+        pace(true, true);
+        wait_vmcnt<0>();
+        __syncthreads();
+        quarter(1, 0, fx[0], st ^ 1, true, 0, has_next, ld_kt, st, 0, do_load);
+        pace(true, has_next);
+        quarter(1, 1, fy[0], st ^ 1, false, 0, has_next, ld_kt, st, 8, do_load);
+        pace(false, has_next);
+    };
 
-    // prologue: slices 0 and 1; wait for slice 0; read its first fragments
+    // prologue: slices 0 and 1 (the host sends no problem with fewer than two slices here); wait for slice 0; read
+    // its first fragment halves
 #pragma unroll
     for (int w = 0; w < 16; ++w) dma(0, 0, w);
-    if (nk > 1) {
 #pragma unroll
-        for (int w = 0; w < 16; ++w) dma(1, 1, w);
-        wait_vmcnt<16>();
-    } else {
-        wait_vmcnt<0>();
-    }
+    for (int w = 0; w < 16; ++w) dma(1, 1, w);
+    wait_vmcnt<16>();
     __syncthreads();
 #pragma unroll
-    for (int p = 0; p < kPieces; ++p) read_piece(fa, 0, 0, p);
-    // slice kt lives in stage kt & 1 and slice kt+1 is already on its way.  Sub-step 0: MFMAs on the first half,
-    // read the second half.  Barrier: slice kt+1 has landed, nobody needs the LDS copy of slice kt.  Sub-step 1:
-    // MFMAs on the second half, read the first half of slice kt+1, refill this stage with all of slice kt+2.
+    for (int p = 0; p < kPX; ++p) read_piece(fx[0], 0, true, 0, p);
+#pragma unroll
+    for (int p = 0; p < kPY; ++p) read_piece(fy[0], 0, false, 0, p);
+    // Two slices per turn of the loop (stage 0, stage 1).  What is left afterwards -- two slices when the slice count is
+    // even, three when it is odd (ODD_NK, chosen by the host) -- follows as straight-line code, so that no branch sits
+    // between the MFMAs: with branches there the compiler no longer accumulates in place and shuffles the
+    // accumulators between registers.
     int kt = 0;
     for (; kt + 3 < nk; kt += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            sub_step(fa, fb, u, 1, true, 0, 0, false);
-            wait_vmcnt<0>();
-            __syncthreads();
-            sub_step(fb, fa, u ^ 1, 0, true, kt + u + 2, u, true);
-        }
+        slice(0, true, kt + 2, true);
+        slice(1, true, kt + 3, true);
     }
-    for (; kt < nk; kt += 2) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const int k1 = kt + u;
-            if (k1 < nk) {
-                sub_step(fa, fb, u, 1, true, 0, 0, false);
-                wait_vmcnt<0>();
-                __syncthreads();
-                sub_step(fb, fa, u ^ 1, 0, k1 + 1 < nk, k1 + 2, u, k1 + 2 < nk);
-            }
-        }
+    if constexpr (ODD_NK) {
+        slice(0, true, kt + 2, true);
+        slice(1, true, 0, false);
+        slice(0, false, 0, false);
+    } else {
+        slice(0, true, 0, false);
+        slice(1, false, 0, false);
     }
     // No barrier here: the last LDS reads of every wave were issued (and awaited) before the barrier of the last
     // slice, and no load is in flight, so each wave may start on its patch as soon as its own MFMAs are done.
 
+    // The epilogues below handle the quadrant in four units of 32 rows (two 16-row blocks): unit u, half h, column
+    // block j -> acc[2u + h][j], patch row h * 16 + lane % 16, patch columns j * 16 + (lane / 16) * 4 .. + 3.
     if constexpr (QF != 0) {
         // ---- fused in-time cast (whole tiles only, no bias, no accumulation: the host sees to that)
         __shared__ uint32_t q_red[kGemmThreads / kWave];
@@ -467,11 +491,11 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         // as it does through abs().max()
         uint32_t m = 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < 8; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) m = umax(m, __float_as_uint(acc[i][j][r]) & 0x7fffffffu);
+                for (int r = 0; r < 4; ++r) m = umax(m, __float_as_uint(acc[i][j][r]) & 0x7fffffffu);
         m = block_max_u32(m, q_red);    // valid in lane 0 of wave 0
         const int tid = threadIdx.x;
         if (tid == 0) {
@@ -513,7 +537,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     if (!all_in) {    // gave up: NaN amax, old scale, both still posted, sticky error word set
                         am = __uint_as_float(0x7fc00000u);
                         report_wait_expired(qa.error_word, kErrCollectorGaveUp);
-                    } else if ((qa.flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
+                    } else if ((qa.flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) {
+                        am = __uint_as_float(0x7f800000u);
+                    }
                     const float sc = scale_rule(am, *qa.scale, qa.fp_max, qa.margin);
                     const uint64_t tag = static_cast<uint64_t>(qa.token) << 32;
                     __hip_atomic_store(post, tag | __float_as_uint(am), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -549,29 +575,30 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         uint8_t* qpatch = smem + wave * (32 * kQPitch);
         auto emit = [&](auto checked) {
             constexpr bool kChecked = decltype(checked)::value;
-            static_for<4>([&](auto ic) {
-                constexpr int i = decltype(ic)::value;
-                static_for<4>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
+            static_for<4>([&](auto uc) {
+                constexpr int u = decltype(uc)::value;
+                static_for<2>([&](auto hc) {
+                    constexpr int h = decltype(hc)::value;
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
+                    for (int j = 0; j < 8; ++j) {
                         // the outputs as OT would hold them, then scaled
+                        const v4f a = acc[2 * u + h][j];
                         float r0, r1, r2, r3;
-                        round_pair<OT>(acc[i][j][4 * q] * alpha, acc[i][j][4 * q + 1] * alpha, r0, r1);
-                        round_pair<OT>(acc[i][j][4 * q + 2] * alpha, acc[i][j][4 * q + 3] * alpha, r2, r3);
+                        round_pair<OT>(a[0] * alpha, a[1] * alpha, r0, r1);
+                        round_pair<OT>(a[2] * alpha, a[3] * alpha, r2, r3);
                         uint32_t w;
                         if constexpr (kChecked) w = quant4<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
                         else w = quant4_in_range<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
-                        *reinterpret_cast<uint32_t*>(qpatch + l32 * kQPitch + j * 32 + q * 8 + lh * 4) = w;
+                        *reinterpret_cast<uint32_t*>(qpatch + (h * 16 + l16) * kQPitch + j * 16 + g4 * 4) = w;
                     }
                 });
                 // the patch is private to this wave and the LDS serves one wave's requests in order: no waits here
-                auto rd = [&](int u) {
-                    return *reinterpret_cast<const uint4*>(qpatch + (u * 8 + (lane >> 3)) * kQPitch + (lane & 7) * 16);
+                auto rd = [&](int t) {
+                    return *reinterpret_cast<const uint4*>(qpatch + (t * 8 + (lane >> 3)) * kQPitch + (lane & 7) * 16);
                 };
                 const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3);
-                auto st = [&](int u, const uint4& v) {
-                    const int grow = row0 + wr * 128 + i * 32 + u * 8 + (lane >> 3);
+                auto st = [&](int t, const uint4& v) {
+                    const int grow = row0 + wr * 128 + u * 32 + t * 8 + (lane >> 3);
                     const int gcol = col0 + wc * 128 + (lane & 7) * 16;
                     *reinterpret_cast<uint4*>(qa.q + static_cast<size_t>(grow) * NC + gcol) = v;
                 };
@@ -582,7 +609,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         return;
     }
 
-    // ---- epilogue: per 32-row block, accumulators -> this wave's LDS patch -> 16-byte row stores
+    // ---- epilogue: per 32-row unit, accumulators -> this wave's LDS patch -> 16-byte row stores
     constexpr int kEsz = static_cast<int>(sizeof(OT));
     constexpr int kPitch = 128 * kEsz + 16;    // bytes per patch row (padding staggers the banks)
     uint8_t* patch = smem + wave * (32 * kPitch);
@@ -593,7 +620,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     constexpr int kRowsPerPass = 64 / kChunksPerRow;    // 4 or 2
     constexpr int kElemsPerChunk = 16 / kEsz;           // 8 or 4
     if (!plain && vec_ok) {
-        // ---- bias and / or accumulation with 16-byte row accesses: the raw float32 accumulators of a 32-row block go
+        // ---- bias and / or accumulation with 16-byte row accesses: the raw float32 accumulators of a 32-row unit go
         // through a per-wave float32 patch, each lane picks up one 16-byte segment of an output row, reads the old
         // output there if it is to be added, and stores fma(acc, alpha, bias) (+ old) rounded once -- the expression of
         // the element-wise path below and of the generic kernel.  A lane's columns are the same in every pass, so
@@ -608,14 +635,15 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         for (int e = 0; e < kElemsPerChunk; ++e) bv[e] = (bias != nullptr && col_ok) ? load_bias(bias, bias_dt, gcol + e) : 0.0f;
         constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
         constexpr int kGroup = 4;                     // passes whose old outputs are in flight together
-        static_for<4>([&](auto ic) {
-            constexpr int i = decltype(ic)::value;
-            static_for<4>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
+        static_for<4>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            static_for<2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    *reinterpret_cast<float4*>(fpatch + l32 * kFPitch + (j * 32 + q * 8 + lh * 4) * 4) =
-                        make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+                for (int j = 0; j < 8; ++j) {
+                    const v4f a = acc[2 * u + h][j];
+                    *reinterpret_cast<float4*>(fpatch + (h * 16 + l16) * kFPitch + (j * 16 + g4 * 4) * 4) =
+                        make_float4(a[0], a[1], a[2], a[3]);
                 }
             });
             // the patch is private to this wave and the LDS serves one wave's requests in order: no waits needed
@@ -624,16 +652,16 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 uint4 old[kGroup];
                 bool ok[kGroup];
 #pragma unroll
-                for (int u = 0; u < kGroup; ++u) {
-                    const int grow = row0 + wr * 128 + i * 32 + (p0 + u) * kRowsPerPass + prl;
-                    ok[u] = col_ok && grow < NR;
-                    old[u] = make_uint4(0, 0, 0, 0);
-                    if (accumulate && ok[u]) old[u] = *reinterpret_cast<const uint4*>(D + static_cast<size_t>(grow) * NC + gcol);
+                for (int t = 0; t < kGroup; ++t) {
+                    const int grow = row0 + wr * 128 + u * 32 + (p0 + t) * kRowsPerPass + prl;
+                    ok[t] = col_ok && grow < NR;
+                    old[t] = make_uint4(0, 0, 0, 0);
+                    if (accumulate && ok[t]) old[t] = *reinterpret_cast<const uint4*>(D + static_cast<size_t>(grow) * NC + gcol);
                 }
 #pragma unroll
-                for (int u = 0; u < kGroup; ++u) {
-                    const int pr = (p0 + u) * kRowsPerPass + prl;
-                    const int grow = row0 + wr * 128 + i * 32 + pr;
+                for (int t = 0; t < kGroup; ++t) {
+                    const int pr = (p0 + t) * kRowsPerPass + prl;
+                    const int grow = row0 + wr * 128 + u * 32 + pr;
                     const float* src = reinterpret_cast<const float*>(fpatch + pr * kFPitch + pc * kElemsPerChunk * 4);
                     float r[kElemsPerChunk], o[kElemsPerChunk];
                     const float4 a0 = *reinterpret_cast<const float4*>(src);
@@ -643,10 +671,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                         r[4] = a1.x, r[5] = a1.y, r[6] = a1.z, r[7] = a1.w;
                     }
                     if constexpr (kEsz == 4) {
-                        o[0] = __uint_as_float(old[u].x), o[1] = __uint_as_float(old[u].y);
-                        o[2] = __uint_as_float(old[u].z), o[3] = __uint_as_float(old[u].w);
+                        o[0] = __uint_as_float(old[t].x), o[1] = __uint_as_float(old[t].y);
+                        o[2] = __uint_as_float(old[t].z), o[3] = __uint_as_float(old[t].w);
                     } else {
-                        In16<OT>::decode(old[u], o);
+                        In16<OT>::decode(old[t], o);
                     }
 #pragma unroll
                     for (int e = 0; e < kElemsPerChunk; ++e) {
@@ -661,37 +689,33 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     } else {
                         v = make_uint4(pack_f16(r[0], r[1]), pack_f16(r[2], r[3]), pack_f16(r[4], r[5]), pack_f16(r[6], r[7]));
                     }
-                    if (ok[u]) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
+                    if (ok[t]) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
                 }
             });
         });
         return;
     }
     if (!plain) {
-        static_for<4>([&](auto ic) {
+        static_for<8>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-            static_for<4>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    store_quad_slow<OT>(D, row0 + wr * 128 + i * 32 + l32, col0 + wc * 128 + j * 32 + q * 8 + lh * 4, NR, NC,
-                                        alpha, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                        acc[i][j][4 * q + 3], accumulate, bias, bias_dt);
-                }
-            });
+            for (int j = 0; j < 8; ++j) {
+                const v4f a = acc[i][j];
+                store_quad_slow<OT>(D, row0 + wr * 128 + i * 16 + l16, col0 + wc * 128 + j * 16 + g4 * 4, NR, NC, alpha, a[0], a[1],
+                                    a[2], a[3], accumulate, bias, bias_dt);
+            }
         });
         return;
     }
-    static_for<4>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        static_for<4>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
+    static_for<4>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        static_for<2>([&](auto hc) {
+            constexpr int h = decltype(hc)::value;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int c = j * 32 + q * 8 + lh * 4;
-                uint8_t* dst = patch + l32 * kPitch + c * kEsz;
-                const float v0 = acc[i][j][4 * q] * alpha, v1 = acc[i][j][4 * q + 1] * alpha;
-                const float v2 = acc[i][j][4 * q + 2] * alpha, v3 = acc[i][j][4 * q + 3] * alpha;
+            for (int j = 0; j < 8; ++j) {
+                const v4f a = acc[2 * u + h][j];
+                uint8_t* dst = patch + (h * 16 + l16) * kPitch + (j * 16 + g4 * 4) * kEsz;
+                const float v0 = a[0] * alpha, v1 = a[1] * alpha, v2 = a[2] * alpha, v3 = a[3] * alpha;
                 if constexpr (kEsz == 4) {
                     *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
                 } else if constexpr (__is_same(OT, bf16_t)) {
@@ -701,22 +725,22 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 }
             }
         });
-        // no wait between the writes above and the reads below, nor before the next block's writes: the patch is
+        // no wait between the writes above and the reads below, nor before the next unit's writes: the patch is
         // private to this wave and the LDS serves one wave's requests in order
         constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
         static_for<kPasses / 8>([&](auto gc) {
             constexpr int p0 = decltype(gc)::value * 8;
             // eight reads in flight together, then the eight stores (named values: an array here ends up in scratch)
-            auto rd = [&](int u) {
-                const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
+            auto rd = [&](int t) {
+                const int pr = (p0 + t) * kRowsPerPass + lane / kChunksPerRow;
                 return *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
             };
             const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3), val4 = rd(4), val5 = rd(5), val6 = rd(6),
                         val7 = rd(7);
-            auto st = [&](int u, const uint4& v) {
-                const int pr = (p0 + u) * kRowsPerPass + lane / kChunksPerRow;
+            auto st = [&](int t, const uint4& v) {
+                const int pr = (p0 + t) * kRowsPerPass + lane / kChunksPerRow;
                 const int pc = lane % kChunksPerRow;
-                const int grow = row0 + wr * 128 + i * 32 + pr;
+                const int grow = row0 + wr * 128 + u * 32 + pr;
                 const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
                 if (grow < NR && gcol < NC) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
             };
@@ -725,12 +749,14 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     });
 }
 
-template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
-static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
-                           const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+// The kernel is built once for an even and once for an odd number of K slices (its last slices are straight-line
+// code); ODD picks the one that fits K.
+template <int XF, int YF, typename OT, bool XT, bool YT, bool ODD>
+static int launch_gemm_dma_parity(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                                  const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     constexpr int smem = 2 * kDmaStage;
     static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
-    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT>;
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, 0, ODD>;
     if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel)");
@@ -743,13 +769,20 @@ static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, 
     return MSAMP_OK;
 }
 
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
+static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                           const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    if ((K / kBK) & 1) return launch_gemm_dma_parity<XF, YF, OT, XT, YT, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    return launch_gemm_dma_parity<XF, YF, OT, XT, YT, false>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+}
+
 // the same kernel with the in-time cast to FP8 fused in (see QF above); the caller has checked the shape
-template <int XF, int YF, typename OT, bool XT, bool YT, int QF>
-static int launch_gemm_dma_quant(const uint8_t* X, const uint8_t* Y, int NR, int NC, int K, const float* xs, const float* ys,
-                                 const QuantArgs& qa, hipStream_t st) {
+template <int XF, int YF, typename OT, bool XT, bool YT, int QF, bool ODD>
+static int launch_gemm_dma_quant_parity(const uint8_t* X, const uint8_t* Y, int NR, int NC, int K, const float* xs,
+                                        const float* ys, const QuantArgs& qa, hipStream_t st) {
     constexpr int smem = 2 * kDmaStage;
     static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
-    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, QF>;
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, QF, ODD>;
     if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel, fused cast)");
@@ -770,6 +803,13 @@ static int launch_gemm_dma_quant(const uint8_t* X, const uint8_t* Y, int NR, int
                        static_cast<const void*>(nullptr), 0, qa);
     MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel (fused cast)");
     return MSAMP_OK;
+}
+
+template <int XF, int YF, typename OT, bool XT, bool YT, int QF>
+static int launch_gemm_dma_quant(const uint8_t* X, const uint8_t* Y, int NR, int NC, int K, const float* xs, const float* ys,
+                                 const QuantArgs& qa, hipStream_t st) {
+    if ((K / kBK) & 1) return launch_gemm_dma_quant_parity<XF, YF, OT, XT, YT, QF, true>(X, Y, NR, NC, K, xs, ys, qa, st);
+    return launch_gemm_dma_quant_parity<XF, YF, OT, XT, YT, QF, false>(X, Y, NR, NC, K, xs, ys, qa, st);
 }
 
 template <int BR, int BC, int XF, int YF, typename OT, bool KGUARD>
@@ -800,11 +840,11 @@ static int launch_gemm(const uint8_t* X, const uint8_t* Y, void* D, int NR, int 
 template <int XF, int YF, typename OT>
 static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                      const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
-    // the direct-to-LDS kernel needs whole 128-byte K slices and 32-bit row offsets; where it can run it is the
+    // the direct-to-LDS kernel needs whole 128-byte K slices, at least two of them, and 32-bit row offsets; where it can run it is the
     // faster one at every size (measured 2.2x from a single 256 x 256 tile up to 121 tiles).  Everything else takes
     // the generic register-staged kernel with 128 x 128 tiles.
     const bool fits32 = static_cast<unsigned long long>(NR) * K < (1ull << 32) && static_cast<unsigned long long>(NC) * K < (1ull << 32);
-    if (K % kBK == 0 && fits32)
+    if (K % kBK == 0 && K >= 2 * kBK && fits32)
         return launch_gemm_dma<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
     return launch_gemm<128, 128, XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
 }

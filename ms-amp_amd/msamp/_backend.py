@@ -440,7 +440,7 @@ def gemm_kmajor_supported(m, n, k, a_kmajor, b_kmajor):
     """Shapes the kernel reads K-major operands for (see msamp_fp8_gemm_kmajor)."""
     if b_kmajor and not a_kmajor:
         return False
-    return k % 128 == 0 and (not a_kmajor or m % 256 == 0) and (not b_kmajor or n % 256 == 0) and \
+    return k % 128 == 0 and k >= 256 and (not a_kmajor or m % 256 == 0) and (not b_kmajor or n % 256 == 0) and \
         m * k < 2**32 and n * k < 2**32
 
 
