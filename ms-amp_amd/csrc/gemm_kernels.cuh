@@ -331,12 +331,14 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                      : static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
     }
     // one of the 16 loads of a slice (0..7: X rows, 8..15: Y rows), so they can be spread between MFMAs
-    auto dma = [&](int kt, int stage, int which) {
+    auto dma = [&](int kt, int stage, int which) __attribute__((always_inline)) {
         const bool is_x = which < 8;
         const size_t slice = static_cast<size_t>(kt) * kBK;
         const uint8_t* src = is_x ? X + (XT ? slice * NR : slice) : Y + (YT ? slice * NC : slice);
         const uint32_t off = which < 8 ? xoff[which] : yoff[which - 8];
-        const uint32_t dst = lds_base + stage * kDmaStage + (which < 8 ? 0 : kDmaTile * kBK) + ((which & 7) * 4 + wave) * 1024;
+        // (wave-uniform by construction; the readfirstlane keeps it in a scalar register whatever the compiler makes of it)
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + stage * kDmaStage + (which < 8 ? 0 : kDmaTile * kBK) +
+                                                            ((which & 7) * 4 + wave) * 1024);
         // Written as assembly so that the compiler does not see an LDS write it cannot tell apart from
         // the fragment reads: it would otherwise make every LDS read wait for all loads in flight.
         // Completion is tracked by hand with wait_vmcnt<>() before the barriers below.  M0 holds the
@@ -359,7 +361,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // four 16-row blocks 4h .. 4h+3 of X / Y (8 registers each).  A half arrives in pieces: two 16-byte reads per
     // block of a row-major operand, four 8-byte transposing reads otherwise.
     constexpr int kPX = XT ? 16 : 8, kPY = YT ? 16 : 8;
-    auto read_piece = [&](int* dst, int stage, bool is_x, int half, int p) {
+    auto read_piece = [&](int* dst, int stage, bool is_x, int half, int p) __attribute__((always_inline)) {
         const uint8_t* base = smem + stage * kDmaStage;
         if ((is_x && !XT) || (!is_x && !YT)) {
             const int b = p >> 1, hf = p & 1;
@@ -396,7 +398,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row lane % 16 of a block, four
     // consecutive D columns -- the layout the epilogue wants.
     auto quarter = [&](int hx, int hy, int* rd_dst, int rd_stage, bool rd_x, int rd_half, bool do_read, int ld_kt,
-                       int ld_stage, int ld_first, bool do_load) {
+                       int ld_stage, int ld_first, bool do_load) __attribute__((always_inline)) {
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
         const int np = rd_x ? kPX : kPY;
@@ -416,36 +418,25 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     for (int p = n * np / 16; p < (n + 1) * np / 16; ++p) read_piece(rd_dst, rd_stage, rd_x, rd_half, p);
                 }
                 if (do_load && (n & 1)) dma(ld_kt, ld_stage, ld_first + (n >> 1));
+                // Nothing moves across: one MFMA, then the reads and the load that go with it.  Left a free hand, the
+                // scheduler stretches the fragments' live ranges until the register allocator no longer updates the 64
+                // accumulators in place and copies them around between the MFMAs.
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-    };
-    // keeps the compiler's schedule to "one MFMA, then the LDS reads that belong to it"
-    auto pace = [&](bool rd_x, bool do_read) {
-        static_for<16>([&](auto nc) {
-            constexpr int n = decltype(nc)::value;
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
-            if (do_read) {
-                if (rd_x) __builtin_amdgcn_sched_group_barrier(0x100, (n + 1) * kPX / 16 - n * kPX / 16, 0);    // its LDS reads
-                else __builtin_amdgcn_sched_group_barrier(0x100, (n + 1) * kPY / 16 - n * kPY / 16, 0);
-            }
-        });
     };
     // Slice kt sits in stage st and slice kt + 1 is on its way into the other stage; X half 0 and Y half 0 of slice
     // kt are in registers.  Quarters 1, 2: X0 x Y0 while Y half 1 arrives, X0 x Y1 while X half 1 arrives -- all of
     // slice kt is in registers now.  Barrier: slice kt + 1 has landed and nobody needs the LDS copy of slice kt.
     // Quarters 3, 4: X1 x Y0 while X half 0 of slice kt + 1 arrives, X1 x Y1 while its Y half 0 arrives; the stage of
     // slice kt is refilled with slice kt + 2 meanwhile.
-    auto slice = [&](int st, bool has_next, int ld_kt, bool do_load) {
+    auto slice = [&](int st, bool has_next, int ld_kt, bool do_load) __attribute__((always_inline)) {
         quarter(0, 0, fy[1], st, false, 1, true, 0, 0, 0, false);
-        pace(false, true);
         quarter(0, 1, fx[1], st, true, 1, true, 0, 0, 0, false);
-        pace(true, true);
         wait_vmcnt<0>();
         __syncthreads();
         quarter(1, 0, fx[0], st ^ 1, true, 0, has_next, ld_kt, st, 0, do_load);
-        pace(true, has_next);
         quarter(1, 1, fy[0], st ^ 1, false, 0, has_next, ld_kt, st, 8, do_load);
-        pace(false, has_next);
     };
 
     // prologue: slices 0 and 1 (the host sends no problem with fewer than two slices here); wait for slice 0; read
@@ -462,8 +453,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     for (int p = 0; p < kPY; ++p) read_piece(fy[0], 0, false, 0, p);
     // Two slices per turn of the loop (stage 0, stage 1).  What is left afterwards -- two slices when the slice count is
     // even, three when it is odd (ODD_NK, chosen by the host) -- follows as straight-line code, so that no branch sits
-    // between the MFMAs: with branches there the compiler no longer accumulates in place and shuffles the
-    // accumulators between registers.
+    // between the MFMAs (another thing that makes the compiler shuffle the accumulators between registers).
     int kt = 0;
     for (; kt + 3 < nk; kt += 2) {
         slice(0, true, kt + 2, true);

@@ -119,7 +119,7 @@ def test_large_tiles_ragged_edges_accumulate_bias(be, m, n, k, out_dtype):
 
 
 @pytest.mark.parametrize('a_dt,b_dt', [(5, 5), (5, 6), (6, 5)])
-@pytest.mark.parametrize('m,n,k', [(256, 256, 128), (512, 768, 384), (1024, 300, 256), (4096, 4096, 512)])
+@pytest.mark.parametrize('m,n,k', [(256, 256, 256), (512, 768, 384), (1024, 300, 256), (4096, 4096, 512), (256, 512, 640)])
 @pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16])
 def test_kmajor_operands_match_transposed_copies(be, a_dt, b_dt, m, n, k, out_dtype):
     """Operands handed over as [K, rows] must give exactly what the row-major kernel gives on their transposed
@@ -154,7 +154,9 @@ def test_kmajor_rejects_unsupported_shapes(be):
     with pytest.raises(RuntimeError):
         be.fp8_gemm(a, 5, one, b, 5, one, torch.empty(64, 100, device='cuda'), a_kmajor=True)
     assert not be.gemm_kmajor_supported(100, 64, 128, True, False)
-    assert not be.gemm_kmajor_supported(256, 256, 128, False, True)
+    assert not be.gemm_kmajor_supported(256, 256, 256, False, True)
+    assert not be.gemm_kmajor_supported(256, 256, 128, True, True)    # a single 128-byte slice of K: not for this kernel
+    assert be.gemm_kmajor_supported(256, 256, 256, True, True)
 
 
 def test_k_not_multiple_of_16_is_padded_by_the_operator():
@@ -281,7 +283,7 @@ def _two_steps(be, a, a_dt, sa, b, b_dt, sb, hp, nan_to_inf, kmajor, old_scale=1
 
 
 @pytest.mark.parametrize('a_dt,b_dt', [(5, 6), (5, 5), (6, 6)])
-@pytest.mark.parametrize('m,n,k', [(256, 256, 128), (1024, 512, 384), (4096, 4096, 512), (2048, 8192, 256)])
+@pytest.mark.parametrize('m,n,k', [(256, 256, 256), (1024, 512, 384), (4096, 4096, 512), (2048, 8192, 256), (512, 256, 640)])
 @pytest.mark.parametrize('hp', [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize('kmajor', [True, False])
 def test_gemm_with_fused_cast_matches_the_two_steps(be, a_dt, b_dt, m, n, k, hp, kmajor):
@@ -306,7 +308,7 @@ def test_gemm_with_fused_cast_matches_the_two_steps(be, a_dt, b_dt, m, n, k, hp,
 def test_gemm_with_fused_cast_special_values(be, nan_to_inf, poison):
     """A NaN or Inf in the product (E5M2 operands carry them) reaches amax as through the two steps, the scale falls
     back to the old one; an all-zero product leaves amax 0 and the old scale."""
-    m, n, k = 512, 256, 128
+    m, n, k = 512, 256, 256
     a = _rand_fp8((k, m), 6, 1).cuda()    # both operands K-major, as the backward pass has them
     b = _rand_fp8((k, n), 6, 2).cuda()
     if poison == 'nan':
@@ -335,15 +337,16 @@ def test_gemm_with_fused_cast_declines_what_it_cannot_take(be):
         got = be.fp8_gemm_cast(a, 5, one, b, 5, one, torch.bfloat16, kw.pop('q_dt', 5), s, am, si, **kw)
         return got, float(s), float(si), float(am)
 
-    assert call(300, 256, 128) == (None, 2.0, 3.0, 5.0)
-    assert call(256, 256, 144) == (None, 2.0, 3.0, 5.0)
+    assert call(300, 256, 256) == (None, 2.0, 3.0, 5.0)
+    assert call(256, 256, 272) == (None, 2.0, 3.0, 5.0)
+    assert call(256, 256, 128) == (None, 2.0, 3.0, 5.0)    # a single slice of K
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     side = 256 * (int(cus ** 0.5) + 1)
-    assert call(side, side, 128) == (None, 2.0, 3.0, 5.0)
-    assert call(256, 256, 128, q_dt=6) == (None, 2.0, 3.0, 5.0)
-    assert call(256, 256, 128, a_kmajor=True) == (None, 2.0, 3.0, 5.0)    # mixed layouts
+    assert call(side, side, 256) == (None, 2.0, 3.0, 5.0)
+    assert call(256, 256, 256, q_dt=6) == (None, 2.0, 3.0, 5.0)
+    assert call(256, 256, 256, a_kmajor=True) == (None, 2.0, 3.0, 5.0)    # mixed layouts
     for layout in (dict(), dict(a_kmajor=True, b_kmajor=True)):
-        got, *_ = call(256, 256, 128, **layout)
+        got, *_ = call(256, 256, 256, **layout)
         assert got is not None
 
 
@@ -412,7 +415,7 @@ def test_gemm_with_fused_cast_many_random_cases(be):
 @pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16])
 def test_generic_and_direct_to_lds_kernels_agree_to_the_bit(be, m, n, k, out_dtype):
     """K a multiple of 128 goes to the direct-to-LDS kernel; the same operands with 16 zero bytes appended to every row
-    (K + 16) go to the generic kernel.  The zeros add nothing, and both kernels add up the 64-byte blocks of K in
+    (K + 16) go to the generic kernel.  The zeros add nothing, and both kernels add up the 128-byte blocks of K in
     ascending order, so the outputs must be equal bit for bit (which makes results independent of the dispatch)."""
     a, b = _gpu_codes((m, k), 5, 3 * m + k), _gpu_codes((n, k), 6, 7 * n + k)
     sa, sb = torch.tensor(0.5, device='cuda'), torch.tensor(0.25, device='cuda')
