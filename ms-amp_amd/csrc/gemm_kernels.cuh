@@ -94,10 +94,9 @@ __device__ __forceinline__ float load_bias(const void* bias, int dt, int i) {
 
 // workgroup id -> tile, keeping the workgroups of one XCD on adjacent tiles and walking groups of
 // `kGroup` tile rows column by column so that the X and Y panels of a group stay in that L2
-__device__ __forceinline__ void tile_of_block(int tiles_r, int tiles_c, int& tr, int& tc) {
+__device__ __forceinline__ void tile_of_id(int id, int tiles_r, int tiles_c, int& tr, int& tc) {
     constexpr int kXcd = 8, kGroup = 8;
     const int nt = tiles_r * tiles_c;
-    int id = blockIdx.x;
     if (nt % kXcd == 0) id = (id % kXcd) * (nt / kXcd) + id / kXcd;
     const int per_group = kGroup * tiles_c;
     const int g = id / per_group;
@@ -107,6 +106,7 @@ __device__ __forceinline__ void tile_of_block(int tiles_r, int tiles_c, int& tr,
     tr = first_r + in_g % rows_here;
     tc = in_g / rows_here;
 }
+__device__ __forceinline__ void tile_of_block(int tiles_r, int tiles_c, int& tr, int& tc) { tile_of_id(blockIdx.x, tiles_r, tiles_c, tr, tc); }
 
 template <int BR, int BC, int XF, int YF, typename OT, bool KGUARD>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_kernel(const uint8_t* __restrict__ X,
@@ -232,6 +232,7 @@ __device__ __noinline__ void store_quad_slow(OT* D, int row, int col, int NR, in
         store_out<OT>(D + static_cast<size_t>(row) * NC + col + e, fmaf(v[e], alpha, bv), accumulate != 0);
     }
 }
+
 
 // ---------------------------------------------------------------------------------------------
 // Main kernel: 256 x 256 output tile over 128-byte K slices, four wavefronts each owning a 128 x 128
@@ -466,6 +467,35 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     } else {
         slice(0, true, 0, false);
         slice(1, false, 0, false);
+    }
+    // The workgroup that follows this one on the CU is, as a rule, the one 256 ids on (same XCD).  Touch the first two K
+    // slices of its tile now -- one 4-byte load per 128-byte line, dropped into an LDS corner that nothing reads -- so that
+    // its prologue finds them in this XCD's L2 instead of waiting for HBM with the MFMA pipe idle.  The loads have no
+    // register destination, so nothing has to wait for them; the hardware drains them before the wave ends.
+    {
+        const int tiles_r = (NR + kDmaTile - 1) / kDmaTile, tiles_c = (NC + kDmaTile - 1) / kDmaTile;
+        const int nid = blockIdx.x + 256;
+        if (nid < tiles_r * tiles_c) {
+            int ntr, ntc;
+            tile_of_id(nid, tiles_r, tiles_c, ntr, ntc);
+            const int nr0 = ntr * kDmaTile, nc0 = ntc * kDmaTile;
+            // line L of an operand's 512: row-major, half L % 2 of row L / 2 (clamped like the tile loads); K-major (whole
+            // tiles only), half L % 2 of the tile's 256 bytes in k-row L / 2 (K >= 256 here)
+            auto line = [&](int L, bool is_x) __attribute__((always_inline)) -> const uint8_t* {
+                const int r = L >> 1, hf = (L & 1) * 128;
+                const uint8_t* base = is_x ? X : Y;
+                const int n = is_x ? NR : NC, first = is_x ? nr0 : nc0;
+                if (is_x ? XT : YT) return base + static_cast<size_t>(r) * n + first + hf;
+                const int row = first + r < n ? first + r : n - 1;
+                return base + static_cast<size_t>(row) * K + hf;
+            };
+            const int t = threadIdx.x;
+            const uint32_t dump = __builtin_amdgcn_readfirstlane(lds_base + 2 * kDmaStage - 256);
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off\n\tglobal_load_lds_dword %2, off\n\t"
+                         "global_load_lds_dword %3, off\n\tglobal_load_lds_dword %4, off"
+                         : : "s"(dump), "v"(line(t, true)), "v"(line(t + 256, true)), "v"(line(t, false)), "v"(line(t + 256, false))
+                         : "memory", "m0");
+        }
     }
     // No barrier here: the last LDS reads of every wave were issued (and awaited) before the barrier of the last
     // slice, and no load is in flight, so each wave may start on its patch as soon as its own MFMAs are done.
