@@ -94,8 +94,11 @@ def fp8_randn(shape, std, fp8_dt, seed):
 
 
 # ---- FP8Linear steps through the msamp API -------------------------------------------------------------------
-def bench_layer(cfg, steps, warmup):
-    """Forward + backward of every projection of `cfg` as FP8Linear modules, then the amax-window update."""
+def bench_layer(cfg, steps, warmup, micro_batches=1):
+    """Forward + backward of every projection of `cfg` as FP8Linear modules, then the amax-window update.  With
+    micro_batches > 1 every projection runs that many forward + backward passes before its gradient is dropped: from
+    the second on, the weight-gradient GEMM adds into the dequantized FP8 gradient of the passes before and the sum
+    is cast to E4M3 again (gradient accumulation)."""
     import torch
     import msamp    # noqa: F401
     from msamp import _backend
@@ -164,9 +167,10 @@ def bench_layer(cfg, steps, warmup):
     def step():
         for lin, dy in zip(model, ograds):
             x = inputs[lin.in_features]
-            lin(x).backward(dy)
+            for _ in range(micro_batches):
+                lin(x).backward(dy)
+                x.grad = None
             lin.weight.grad = None
-            x.grad = None
         opt._update_scaling_factors()
 
     try:
@@ -193,12 +197,12 @@ def bench_layer(cfg, steps, warmup):
     gemm_flops_total = sum(f for _, _, f in gemm_events)
     return {
         'ms_per_step': ms_per_step,
-        'step_tflops': flops / (ms_per_step * 1e-3) / 1e12,
+        'step_tflops': micro_batches * flops / (ms_per_step * 1e-3) / 1e12,
         'gemm_tflops': gemm_flops_total / (gemm_ms_total * 1e-3) / 1e12,
         'gemm_avg_launch_ms': gemm_ms_total / len(gemm_events),
         'gemm_avg_launch_flops': gemm_flops_total / len(gemm_events),
         'gemm_launches': len(gemm_events),
-        'gemms_per_step': 3 * len(cfg['proj']),
+        'gemms_per_step': 3 * len(cfg['proj']) * micro_batches,
     }
 
 
@@ -566,6 +570,15 @@ def main():
             'ms_per_step': round(c2['ms_per_step'], 4), 'step_tflops': round(c2['step_tflops'], 1),
             'gemm_tflops': round(c2['gemm_tflops'], 1), 'gemm_frac_mfma': round(c2['gemm_tflops'] / FP8_PEAK_TFLOPS, 4),
             'gemm_avg_launch_ms': round(c2['gemm_avg_launch_ms'], 4), 'gemm_launches': c2['gemm_launches'],
+        }
+        torch.cuda.empty_cache()
+        acc = bench_layer(LLAMA_7B, max(args.steps // 4, 20), 2, micro_batches=2)
+        result['c4_grad_accumulation_step'] = {
+            'workload': 'config 4 with two micro-batches per step: the second weight-gradient GEMM of every projection adds '
+                        'into the dequantized E4M3 gradient of the first and the sum is cast to E4M3 again',
+            'ms_per_step': round(acc['ms_per_step'], 4), 'step_tflops': round(acc['step_tflops'], 1),
+            'gemm_tflops': round(acc['gemm_tflops'], 1), 'gemm_frac_mfma': round(acc['gemm_tflops'] / FP8_PEAK_TFLOPS, 4),
+            'gemm_launches': acc['gemm_launches'], 'gemms_per_step': acc['gemms_per_step'],
         }
         torch.cuda.empty_cache()
         result['gemm_sweep'] = {'c4_llama7b': bench_gemm_sweep(LLAMA_7B, accumulate_row='gate')}

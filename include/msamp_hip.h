@@ -40,10 +40,11 @@ enum {
 enum {
     MSAMP_OK = 0,
     MSAMP_ERR_DTYPE = -1,     /* unsupported data type code            */
-    MSAMP_ERR_SHAPE = -2,     /* bad size, shape or alignment          */
+    MSAMP_ERR_SHAPE = -2,     /* bad size or shape                     */
     MSAMP_ERR_NULL = -3,      /* required pointer is NULL              */
     MSAMP_ERR_WORKSPACE = -4, /* workspace missing or too small        */
     MSAMP_ERR_TIMEOUT = -5,   /* a kernel's bounded wait ran out (msamp_check_async_error) */
+    MSAMP_ERR_ALIGNMENT = -6, /* a pointer is not aligned as the entry point requires */
     MSAMP_ERR_HIP = -100      /* -100 - hipError_t of the failing call */
 };
 

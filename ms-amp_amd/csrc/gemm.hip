@@ -33,7 +33,7 @@ extern "C" int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_
     MSAMP_REQUIRE(m > 0 && n > 0 && k > 0, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_cast: m=%d n=%d k=%d", m, n, k);
     MSAMP_REQUIRE(a && b && q && a_scale_inv && b_scale_inv && scale && amax && scale_inv, MSAMP_ERR_NULL,
                   "msamp_fp8_gemm_cast: null pointer");
-    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(q, 16), MSAMP_ERR_SHAPE,
+    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(q, 16), MSAMP_ERR_ALIGNMENT,
                   "msamp_fp8_gemm_cast: operands and output must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool both = a_kmajor && b_kmajor, neither = !a_kmajor && !b_kmajor;
@@ -67,7 +67,7 @@ extern "C" int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* 
     MSAMP_REQUIRE(m > 0 && n > 0 && k > 0 && kmajor_shape_ok(n, m, k, b_kmajor != 0, true), MSAMP_ERR_SHAPE,
                   "msamp_fp8_gemm_kmajor: m=%d n=%d k=%d (k must be a multiple of 128 and at least 256, the K-major operands' rows multiples of 256)", m, n, k);
     MSAMP_REQUIRE(a && b && d && a_scale_inv && b_scale_inv, MSAMP_ERR_NULL, "msamp_fp8_gemm_kmajor: null pointer");
-    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16), MSAMP_ERR_SHAPE, "msamp_fp8_gemm_kmajor: operands must be 16-byte aligned");
+    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16), MSAMP_ERR_ALIGNMENT, "msamp_fp8_gemm_kmajor: operands must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     // X = b (rows of D), Y = a (columns of D)
     const GemmCall c = {b, a, d, d_dtype, n, m, k, b_scale_inv, a_scale_inv, accumulate, bias, bias_dtype, b_kmajor != 0, true, nullptr, st};
@@ -84,7 +84,7 @@ extern "C" int msamp_fp8_gemm(const uint8_t* a, int a_type, const float* a_scale
     if (m == 0 || n == 0) return MSAMP_OK;
     MSAMP_REQUIRE(k > 0 && k % 16 == 0, MSAMP_ERR_SHAPE, "msamp_fp8_gemm: k=%d must be a positive multiple of 16", k);
     MSAMP_REQUIRE(a && b && d && a_scale_inv && b_scale_inv, MSAMP_ERR_NULL, "msamp_fp8_gemm: null pointer");
-    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16), MSAMP_ERR_SHAPE, "msamp_fp8_gemm: operands must be 16-byte aligned");
+    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16), MSAMP_ERR_ALIGNMENT, "msamp_fp8_gemm: operands must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     // X = b (rows of D), Y = a (columns of D)
     const GemmCall c = {b, a, d, d_dtype, n, m, k, b_scale_inv, a_scale_inv, accumulate, bias, bias_dtype, false, false, nullptr, st};

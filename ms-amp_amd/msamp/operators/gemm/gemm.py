@@ -17,6 +17,13 @@ class Gemm:
         """Smallest multiple of base that is >= value."""
         return (value + base - 1) // base * base
 
+    @staticmethod
+    def _aligned(payload):
+        """The kernels fetch operands 16 bytes at a time.  A payload that starts elsewhere (a view into a flat buffer
+        at an odd offset) is copied to a fresh allocation first, as the reference pads and copies what its library
+        cannot take (msamp/operators/gemm/gemm.py:107-121)."""
+        return payload if payload.data_ptr() % 16 == 0 else payload.clone()
+
     @classmethod
     def kmajor_supported(cls, m, n, k, a_kmajor=True, b_kmajor=False):
         """True if fp8_gemm reads K-major operands of this problem in place (else it transposes them first)."""
@@ -35,7 +42,8 @@ class Gemm:
         if meta.scaling_mode() != 'in_time' or (a_kmajor != b_kmajor):
             return None
         payload = _backend.fp8_gemm_cast(
-            mat_a.value, int(mat_a.qtype), mat_a.meta.scale_inv, mat_b.value, int(mat_b.qtype), mat_b.meta.scale_inv,
+            cls._aligned(mat_a.value), int(mat_a.qtype), mat_a.meta.scale_inv, cls._aligned(mat_b.value), int(mat_b.qtype),
+            mat_b.meta.scale_inv,
             Dtypes.get_dtype_from_qtype(out_qtype), int(meta.qtype), meta.scale, meta.amax[0:1], meta.scale_inv,
             nan_to_inf=sync, a_kmajor=a_kmajor, b_kmajor=b_kmajor
         )
@@ -75,8 +83,8 @@ class Gemm:
                 else:
                     assert out.is_cuda and out.is_contiguous() and out.dtype == out_dtype
                 _backend.fp8_gemm(
-                    mat_a.value, int(mat_a.qtype), mat_a.meta.scale_inv, mat_b.value, int(mat_b.qtype), mat_b.meta.scale_inv,
-                    out, accumulate, bias, a_kmajor=a_kmajor, b_kmajor=b_kmajor
+                    cls._aligned(mat_a.value), int(mat_a.qtype), mat_a.meta.scale_inv, cls._aligned(mat_b.value),
+                    int(mat_b.qtype), mat_b.meta.scale_inv, out, accumulate, bias, a_kmajor=a_kmajor, b_kmajor=b_kmajor
                 )
                 return out
             if a_kmajor:
@@ -86,7 +94,7 @@ class Gemm:
 
         M, K = mat_a.shape
         N = len(mat_b)
-        a, b = mat_a.value, mat_b.value
+        a, b = cls._aligned(mat_a.value), cls._aligned(mat_b.value)
         pK = cls._round2times(K, cls._te_base) - K
         if pK > 0:
             a = F.pad(a, (0, pK))

@@ -39,6 +39,12 @@ class LBAdamW(LBAdamWBase):
             return False
         if m.qtype != Dtypes.kfloat8_e4m3 or v.qtype != Dtypes.kfloat16:
             return False
+        # The fused kernel always derives the weight's new scale from the amax of the updated weight.  The per-tensor
+        # recipe re-quantizes through param.cast(), which does that only under in-time scaling (reference
+        # msamp/optim/adamw.py:172-174 with msamp/common/tensor/cast.py:31-44); a weight meta in any other mode takes
+        # the per-tensor path.
+        if p.meta.scaling_mode() != 'in_time':
+            return False
         tensors = (p.value, g.value, m.value, v.value)
         if not all(t.is_cuda and t.is_contiguous() and t.numel() == p.value.numel() for t in tensors):
             return False

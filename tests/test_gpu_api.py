@@ -145,6 +145,78 @@ def test_fp8linear_step_against_oracle_pipeline():
     assert same_float(metas['ograd'].amax[0], gm['amax'][0]) and same_float(metas['ograd'].scale, gm['scale'])
 
 
+def _code_rank(q):
+    """FP8 codes (sign-magnitude bytes) as integers ordered like the values they stand for."""
+    q = q.to(torch.int16)
+    return torch.where(q >= 128, 127 - q, q)
+
+
+def test_full_size_fp8linear_step_with_delayed_scaling_against_oracle_pipeline():
+    """x[8192, 4096], W[4096, 4096] in bfloat16: 17 steps fill the 16-deep amax windows of `input` and `ograd`, so the
+    18th step -- on new data of another magnitude -- quantizes with the scale the window holds (delayed scaling, reference
+    msamp/common/tensor/cast.py:31-44 and msamp/optim/optimizer.py:91-108).  That step through the module API against
+    the oracle's casts, window updates and GEMMs: metas to the bit, y and dx within the GEMM bar, the FP8 weight
+    gradient within one code (values next to zero: within 2**-7 of the scaled range)."""
+    from oracle import scaling as oscaling
+    torch.manual_seed(21)
+    tokens, d_in, d_out, window = 8192, 4096, 4096, 16
+    lin = torch.nn.Linear(d_in, d_out, bias=False).cuda().bfloat16()
+    w_ref = lin.weight.detach().cpu()
+    model = LinearReplacer.replace(lin, Dtypes.kbfloat16)
+    opt = LBAdamW(model.parameters(), lr=0.0)    # drives the window update only
+    assert model.scaling_metas['input'].window_size == window
+    x1 = torch.randn(tokens, d_in, device='cuda', dtype=torch.bfloat16)
+    dy1 = (torch.randn(tokens, d_out, device='cuda') * 1e-3).bfloat16()
+    for _ in range(17):
+        model(x1).backward(dy1)
+        model.weight.grad = None
+        opt._update_scaling_factors()
+    assert not model.scaling_metas['input'].is_in_time_scaling() and not model.scaling_metas['ograd'].is_in_time_scaling()
+    # new data, 1.4 times larger: some of it saturates under the window's scale, in the kernel as in the oracle
+    x2 = (torch.randn(tokens, d_in, device='cuda') * 1.4).bfloat16().requires_grad_()
+    dy2 = (torch.randn(tokens, d_out, device='cuda') * 1.4e-3).bfloat16()
+    y = model(x2)
+    y.backward(dy2)
+
+    def warmed_meta(first, fmt):
+        scales, amaxs, counters = torch.ones(1), torch.zeros(1, window), torch.zeros(1, dtype=torch.int32)
+        a1 = first.detach().abs().max().float().cpu()
+        for _ in range(17):
+            amaxs[0, 0] = torch.maximum(amaxs[0, 0], a1)
+            oscaling.update_scaling_factors(scales, amaxs, counters, fp8.FP_MAX[fmt], 0)
+        assert int(counters[0]) == 17
+        return {'scale': scales[0].clone(), 'scale_inv': torch.reciprocal(scales[0]), 'amax': amaxs[0].clone()}
+
+    xm, gm = warmed_meta(x1, fp8.E4M3), warmed_meta(dy1, fp8.E5M2)
+    wm, dwm = ocast.new_meta(), ocast.new_meta()
+    xq = ocast.cast_to_fp8(x2.detach().cpu(), xm, fp8.E4M3, in_time=False)
+    gq = ocast.cast_to_fp8(dy2.cpu(), gm, fp8.E5M2, in_time=False)
+    wq = ocast.cast_to_fp8(w_ref, wm, fp8.E4M3, in_time=True)
+    metas = model.scaling_metas
+    for name, om in (('input', xm), ('ograd', gm)):
+        assert same_float(metas[name].scale, om['scale']) and same_float(metas[name].scale_inv, om['scale_inv'])
+        assert same_float(metas[name].amax[0], om['amax'][0]) and int(metas[name].amax_counter) == 17
+    y_want = ogemm.fp8_gemm(wq, wm['scale_inv'], fp8.E4M3, xq, xm['scale_inv'], fp8.E4M3)
+    assert rel_fro(y.float().cpu(), y_want) < 1e-2
+    del y_want
+    dx_want = ogemm.fp8_gemm(wq.t().contiguous(), wm['scale_inv'], fp8.E4M3, gq, gm['scale_inv'], fp8.E5M2)
+    assert rel_fro(x2.grad.float().cpu(), dx_want) < 1e-2
+    del dx_want
+    dw_want = ogemm.fp8_gemm(xq.t().contiguous(), xm['scale_inv'], fp8.E4M3, gq.t().contiguous(), gm['scale_inv'], fp8.E5M2,
+                             out_dtype=torch.bfloat16)
+    dwq_want = ocast.cast_to_fp8(dw_want, dwm, fp8.E4M3, in_time=True, sync=True)
+    grad = model.weight.grad
+    assert isinstance(grad, ScalingTensor) and grad.qtype == Dtypes.kfloat8_e4m3
+    assert same_float(grad.meta.scale, dwm['scale'])
+    distance = (_code_rank(grad.value.cpu()) - _code_rank(dwq_want)).abs()
+    # Within one code wherever the code is a normal number.  Below that (|scaled value| < 2**-6, codes 2**-9 apart, which
+    # is 8e-6 of the tensor's amax) the GEMM's own error spans more than one code: there the values agree to 2**-7.
+    want_val, got_val = fp8.decode(dwq_want, fp8.E4M3), fp8.decode(grad.value.cpu(), fp8.E4M3)
+    normal = want_val.abs() >= 2.0**-6
+    assert int(distance[normal].max()) <= 1 and float((got_val - want_val)[~normal].abs().max()) <= 2.0**-7
+    assert float((distance != 0).float().mean()) < 0.005
+
+
 def test_fp8linear_bias_rides_in_the_forward_gemm():
     """The bias is added in the epilogue of the forward GEMM (one rounding): against the oracle with the bias, within
     one ulp (of the larger of the bare and the biased output) of the reference's two steps (GEMM rounded, then + bias rounded), and the bias gradient is the
@@ -206,6 +278,35 @@ def test_optimizers_track_torch_adamw():
         _check_optimizer_step(torch.optim.AdamW, partial(LBAdamW, **kw))
         _check_optimizer_step(torch.optim.AdamW, partial(DSAdam, **kw))
         _check_optimizer_step(torch.optim.Adam, partial(LBAdam, **kw))
+
+
+def test_fused_adamw_only_for_weights_under_in_time_scaling(monkeypatch):
+    """The fused kernel rescales the weight from its new amax; with in-time scaling off the reference keeps the stored
+    scale (msamp/optim/adamw.py:174 through msamp/common/tensor/cast.py:31-44), so such weights take the per-tensor path."""
+    torch.manual_seed(7)
+    linear = torch.nn.Linear(64, 32, bias=False).cuda()
+    x = torch.randn(16, 64, device='cuda')
+    results = {}
+    for in_time in (True, False):
+        model_state.clear()
+        model = LinearReplacer.replace(copy.deepcopy(linear), Dtypes.kfloat16)
+        opt = LBAdamW(model.parameters(), lr=0.05)
+        calls = []
+        fused_step = LBAdamW._fused_step
+        monkeypatch.setattr(LBAdamW, '_fused_step', lambda self, idx, *a, **k: (calls.append(len(idx)), fused_step(self, idx, *a, **k)))
+        model(x).sum().backward()
+        opt.all_reduce_grads(model)
+        scale_before = model.weight.meta.scale.clone()
+        with ScalingMeta.in_time_scaling_context(in_time):
+            opt.step()
+        monkeypatch.undo()
+        results[in_time] = (calls, scale_before, model.weight.meta.scale.clone(), model.weight.float())
+    calls, before, after, w_fused = results[True]
+    assert calls == [1]
+    calls, before, after, w_staged = results[False]
+    assert calls == [] and torch.equal(before, after)
+    # same update either way, up to the coarser grid of the kept scale
+    assert torch.allclose(w_fused, w_staged, rtol=0, atol=float(w_fused.abs().max()) * 2e-3)
 
 
 def test_historical_window_quantization():

@@ -143,6 +143,40 @@ def test_config5_weight_cast_full_size(be):
         del back, q2
 
 
+def test_config5_whole_layer_weight_casts(be):
+    """The seven weight matrices of one Llama-70B layer (q, k, v, o, gate, up, down: 855 638 016 bf16 elements), each
+    cast in-time twice in a row the way a training loop meets them: the first call finds a fresh meta, the second the
+    scale of the step before (the case the speculative kernels are written for), after the weights moved a little.
+    Every call: amax is the maximum, the scale follows the rule, the bytes equal those of the plain two-pass kernels
+    without speculation, and a slice equals the oracle's cast."""
+    shapes = dict(q=(8192, 8192), k=(1024, 8192), v=(1024, 8192), o=(8192, 8192), gate=(28672, 8192), up=(28672, 8192),
+                  down=(8192, 28672))
+    assert sum(r * c for r, c in shapes.values()) == 855_638_016
+    g = torch.Generator(device='cuda').manual_seed(70)
+    for i, (name, (rows, cols)) in enumerate(shapes.items()):
+        w = (torch.randn(rows, cols, generator=g, device='cuda') * 0.02).bfloat16()
+        s, si, am = make_meta()
+        for step in range(2):
+            if step == 1:
+                w = (w.float() * (1.0 + 0.001 * i) + 1e-4).bfloat16()
+            q = be.cast_to_fp8_intime(w, s, am[0:1], si, 5)
+            assert am[0].item() == w.abs().max().item(), name
+            assert same_float(s.cpu(), scaling.compute_scaling_factor(am[0].cpu(), torch.tensor(1.0), 448.0, 0)), name
+            assert same_float(si.cpu(), 1.0 / s.cpu()), name
+            s2, si2, am2 = make_meta()
+            plain = be.cast_to_fp8_intime(w, s2, am2[0:1], si2, 5, two_pass=True, speculate=False)
+            assert torch.equal(q, plain) and same_float(s, s2) and same_float(am[0], am2[0]), name
+            del plain
+            start = (rows * cols // 3) & ~15
+            part = slice(start, start + (1 << 18))
+            om = oracle_meta()
+            om['scale'].copy_(s.cpu())
+            want = ocast.cast_to_fp8(w.view(-1)[part].cpu(), om, FMT[5], in_time=False)
+            assert torch.equal(q.view(-1)[part].cpu(), want), name
+            del q
+        del w
+
+
 @pytest.mark.parametrize('dtype', [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize('n', [1, 3, 1000, 4097, 16384 * 3 + 5, 1 << 20])
 def test_in_time_cast_ragged_sizes(be, dtype, n):

@@ -171,6 +171,41 @@ def test_k_not_multiple_of_16_is_padded_by_the_operator():
     assert out.shape == (3, 5) and rel_fro(out, want) < TOL_F32
 
 
+def test_operands_at_odd_offsets_of_a_flat_buffer(be):
+    """A payload that is a view one byte into a flat buffer: the operator copies it to an aligned allocation and gives
+    the bits of the aligned call; the C entry point itself names the alignment in its error."""
+    import msamp    # noqa: F401
+    from msamp.common.dtype import Dtypes
+    from msamp.common.tensor import ScalingTensor
+    from msamp.operators.gemm import Gemm
+    g = torch.Generator().manual_seed(11)
+    for (m, n, k), kmajor in [((48, 40, 64), False), ((256, 512, 256), True), ((256, 256, 384), False)]:
+        sa = (torch.randn(m, k, generator=g).cuda()).cast(Dtypes.kfloat8_e4m3)
+        sb = (torch.randn(n, k, generator=g).cuda()).cast(Dtypes.kfloat8_e5m2)
+        want = Gemm.fp8_gemm(sa, sb, Dtypes.kbfloat16)
+        want_q = Gemm.fp8_gemm(sa, sb, Dtypes.kfloat32).cast(Dtypes.kfloat8_e4m3)
+
+        def shifted(t, transposed=False):
+            payload = t.value.t().contiguous() if transposed else t.value
+            flat = torch.empty(payload.numel() + 1, dtype=torch.uint8, device='cuda')
+            view = flat[1:].view(payload.shape)
+            view.copy_(payload)
+            assert view.data_ptr() % 16 == 1 and view.is_contiguous()
+            return ScalingTensor(view, t.meta)
+
+        ua, ub = shifted(sa, kmajor), shifted(sb)
+        got = Gemm.fp8_gemm(ua, ub, Dtypes.kbfloat16, a_kmajor=kmajor)
+        assert torch.equal(got, want)
+        if m % 256 == 0 and n % 256 == 0 and not kmajor:
+            from msamp.common.tensor import ScalingMeta
+            meta = ScalingMeta(Dtypes.kfloat8_e4m3, window_size=1)
+            fused = Gemm.fp8_gemm_cast(shifted(sa), ub, Dtypes.kfloat32, meta)
+            assert fused is not None and torch.equal(fused.value, want_q.value)
+        with pytest.raises(RuntimeError, match='aligned'):
+            out = torch.empty(n, m, dtype=torch.bfloat16, device='cuda')
+            be.fp8_gemm(shifted(sa).value, 5, sa.meta.scale_inv, ub.value, 6, sb.meta.scale_inv, out)
+
+
 def test_bad_arguments_raise(be):
     a = torch.zeros(16, 24, dtype=torch.uint8, device='cuda')
     si = torch.ones((), device='cuda')
@@ -219,7 +254,8 @@ def _gpu_codes(shape, fp8_dt, seed):
 
 
 @pytest.mark.parametrize('tokens,d_out,d_in', [(16384, 11008, 4096), (16384, 4096, 11008), (16384, 12288, 4096),
-                                               (16384, 8192, 28672), (16384, 10240, 8192)])
+                                               (16384, 4096, 4096), (16384, 8192, 28672), (16384, 10240, 8192),
+                                               (16384, 28672, 8192), (16384, 8192, 8192)])
 def test_llama_layer_shapes_sampled(be, tokens, d_out, d_in):
     """Forward, dgrad and wgrad of the Llama-7B / 70B projection shapes (K up to 28672), operands handed over the way
     the layer holds them (dgrad and wgrad read K-major operands in place).  Sampled rows and columns against the

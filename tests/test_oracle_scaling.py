@@ -119,3 +119,47 @@ def test_cast_state_machine_in_time_and_delayed():
     m4['scale'] = torch.tensor(8.0)
     ocast.cast_to_fp8(xn, m4, fp8.E4M3, in_time=True, sync=True)
     assert m4['amax'][0].item() == float('inf') and m4['scale'].item() == 0.125
+
+
+def test_scaled_fp16_to_fp8_reference_case_and_invariants():
+    """The reference's own case (tests/common/tensor/test_tensor.py:186-196): 2**-17 as a scaled float16 tensor, then
+    to E4M3, comes back exactly.  Worked by hand: amax 2**-17 gives the float16 scale 2**32 (payload 2**15) and the
+    E4M3 scale 2**25, so the payload is quantized with 2**25 / 2**32 = 2**-7 to 256 = code 0x78, and the new
+    scale_inv is 2**-25."""
+    for src in (torch.float16, torch.float32):
+        value = torch.tensor([2.0**-17], dtype=torch.float16).to(src)
+        m16 = ocast.new_meta()
+        v16 = ocast.cast_to_fp16(value, m16, in_time=True)
+        assert v16.dtype == torch.float16 and v16.item() == 2.0**15
+        assert m16['scale'].item() == 2.0**32 and m16['scale_inv'].item() == 2.0**-32
+        q, m8 = ocast.scaled_fp16_to_fp8(v16, m16, fp8.E4M3)
+        assert q.tolist() == [0x78] and m8['scale_inv'].item() == 2.0**-25 and m8['scale'].item() == 2.0**-7
+        assert m8['amax'][0].item() == 2.0**-17
+        assert (fp8.decode(q, fp8.E4M3) * m8['scale_inv']).item() == 2.0**-17
+    # Values with few significant bits survive the float16 stop unchanged, so the two-step route must give the codes
+    # and the scale_inv of the direct in-time cast (a missing or inverted factor fails here for every element).
+    g = torch.Generator().manual_seed(3)
+    x = torch.randint(-15, 16, (4096, ), generator=g).float() * torch.exp2(torch.randint(-6, 3, (4096, ), generator=g).float())
+    x[0] = 15 * 4.0    # the amax
+    for fmt in (fp8.E4M3, fp8.E5M2):
+        direct_meta = ocast.new_meta()
+        direct = ocast.cast_to_fp8(x, direct_meta, fmt, in_time=True)
+        m16 = ocast.new_meta()
+        v16 = ocast.cast_to_fp16(x, m16, in_time=True)
+        assert torch.equal(v16.float() * m16['scale_inv'], x)
+        q, m8 = ocast.scaled_fp16_to_fp8(v16, m16, fmt)
+        assert torch.equal(q, direct) and m8['scale_inv'].item() == direct_meta['scale_inv'].item()
+        assert m8['amax'][0].item() == 60.0
+
+
+def test_cast_again_after_the_scale_was_touched():
+    """tests/common/tensor/test_tensor.py:277-285: an in-time cast recomputes the scale, so doubling the stored scale
+    between two casts of one tensor changes nothing."""
+    x = torch.randn(64, generator=torch.Generator().manual_seed(0))
+    for fmt in (fp8.E4M3, fp8.E5M2):
+        meta = ocast.new_meta()
+        q1 = ocast.cast_to_fp8(x, meta, fmt, in_time=True)
+        first = fp8.decode(q1, fmt) * meta['scale_inv']
+        meta['scale'] = meta['scale'] * 2
+        q2 = ocast.cast_to_fp8(x, meta, fmt, in_time=True)
+        assert torch.equal(q1, q2) and torch.equal(fp8.decode(q2, fmt) * meta['scale_inv'], first)
