@@ -510,7 +510,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--skip-cpu', action='store_true', help='leave out the CPU-oracle baseline')
     ap.add_argument('--skip-extra', action='store_true', help='leave out the sweep, cast and Adam kernel sections')
-    ap.add_argument('--only', choices=('gemm_c4', 'gemm_c5', 'cast', 'adam'), default=None,
+    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'cast', 'adam'), default=None,
                     help='run one kernel section alone (after the calibration copy), for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -524,7 +524,9 @@ def main():
 
     pmc_calibration_copy()
     if args.only:
-        if args.only == 'gemm_c4':
+        if args.only == 'gemm_c2':
+            out = bench_gemm_sweep(CONFIG_2, iters=6)
+        elif args.only == 'gemm_c4':
             out = bench_gemm_sweep(LLAMA_7B, iters=3, accumulate_row='gate')
         elif args.only == 'gemm_c5':
             out = bench_gemm_sweep(LLAMA_70B, iters=3)

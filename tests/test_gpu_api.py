@@ -209,11 +209,12 @@ def test_full_size_fp8linear_step_with_delayed_scaling_against_oracle_pipeline()
     assert isinstance(grad, ScalingTensor) and grad.qtype == Dtypes.kfloat8_e4m3
     assert same_float(grad.meta.scale, dwm['scale'])
     distance = (_code_rank(grad.value.cpu()) - _code_rank(dwq_want)).abs()
-    # Within one code wherever the code is a normal number.  Below that (|scaled value| < 2**-6, codes 2**-9 apart, which
-    # is 8e-6 of the tensor's amax) the GEMM's own error spans more than one code: there the values agree to 2**-7.
+    # Within one code wherever codes are at least 2**-6 apart (|scaled value| >= 2**-3; the tensor's amax is scaled to
+    # 224 .. 448).  Closer to zero the codes are as fine as 2**-9 -- 8e-6 of the amax -- and the GEMM's own error spans
+    # more than one of them: there the values agree to 2**-7.
     want_val, got_val = fp8.decode(dwq_want, fp8.E4M3), fp8.decode(grad.value.cpu(), fp8.E4M3)
-    normal = want_val.abs() >= 2.0**-6
-    assert int(distance[normal].max()) <= 1 and float((got_val - want_val)[~normal].abs().max()) <= 2.0**-7
+    coarse = want_val.abs() >= 2.0**-3
+    assert int(distance[coarse].max()) <= 1 and float((got_val - want_val)[~coarse].abs().max()) <= 2.0**-7
     assert float((distance != 0).float().mean()) < 0.005
 
 
@@ -285,12 +286,16 @@ def test_fused_adamw_only_for_weights_under_in_time_scaling(monkeypatch):
     scale (msamp/optim/adamw.py:174 through msamp/common/tensor/cast.py:31-44), so such weights take the per-tensor path."""
     torch.manual_seed(7)
     linear = torch.nn.Linear(64, 32, bias=False).cuda()
+    with torch.no_grad():
+        # amax 0.1: the float16 payload's scale is 2**19 and the step below stays inside float16 under the kept scale
+        linear.weight.clamp_(-0.1, 0.1)
+        linear.weight[0, 0] = 0.1
     x = torch.randn(16, 64, device='cuda')
     results = {}
     for in_time in (True, False):
         model_state.clear()
         model = LinearReplacer.replace(copy.deepcopy(linear), Dtypes.kfloat16)
-        opt = LBAdamW(model.parameters(), lr=0.05)
+        opt = LBAdamW(model.parameters(), lr=0.01)
         calls = []
         fused_step = LBAdamW._fused_step
         monkeypatch.setattr(LBAdamW, '_fused_step', lambda self, idx, *a, **k: (calls.append(len(idx)), fused_step(self, idx, *a, **k)))
