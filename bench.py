@@ -348,8 +348,9 @@ def bench_grad_side(iters=10):
 
 
 def bench_adam(iters=5, total_params=1_000_000_000):
-    """Fused FP8 AdamW over 1.0e9 parameters held as [4096,1024] tensors (last one truncated):
-    E4M3 weights, E5M2 grads, E4M3 exp_avg, scaled-fp16 exp_avg_sq; step t=2."""
+    """Fused FP8 AdamW over 1.0e9 parameters held as [4096,1024] tensors (last one truncated): E4M3 weights, E5M2
+    grads, E4M3 exp_avg, scaled-fp16 exp_avg_sq, steps t = 2, 3, ...  Timed: the one-pass step between two sets of
+    payload buffers (the library's default through LBAdamW) and, beside it, the two-pass step in place."""
     import numpy as np
     import torch
     from msamp import _backend
@@ -380,21 +381,42 @@ def bench_adam(iters=5, total_params=1_000_000_000):
                      d['w'][1].data_ptr(), d['w'][2].data_ptr(), d['w'][3].data_ptr(), d['g'][2].data_ptr(),
                      d['m'][1].data_ptr(), d['m'][2].data_ptr(), d['m'][3].data_ptr(),
                      d['v'][1].data_ptr(), d['v'][2].data_ptr(), d['v'][3].data_ptr(), n, 0, 0, 0, 0))
-    desc = torch.from_numpy(np.asarray(rows, dtype=np.int64)).cuda()
     chunks = [(n + _backend.ADAMW_CHUNK - 1) // _backend.ADAMW_CHUNK for n in sizes]
     bm = np.stack([np.repeat(np.arange(len(sizes), dtype=np.int32), chunks),
                    np.concatenate([np.arange(c, dtype=np.int32) for c in chunks])], axis=1).copy()
     block_map = torch.from_numpy(bm).cuda()
-    state = {'t': 1}
+    # Two sets of payload buffers: a step reads one and writes the other (what LBAdamW(double_buffer=True) does), so
+    # there is a descriptor table and an output table per direction.
+    spare = [(torch.empty_like(d['w'][0]), torch.empty_like(d['m'][0]), torch.empty_like(d['v'][0])) for d in tensors]
+    swapped = [tuple(r) for r in rows]
+    swapped = [(sp[0].data_ptr(), r[1], sp[1].data_ptr(), sp[2].data_ptr()) + r[4:] for r, sp in zip(swapped, spare)]
+    descs = [torch.from_numpy(np.asarray(rows, dtype=np.int64)).cuda(), torch.from_numpy(np.asarray(swapped, dtype=np.int64)).cuda()]
+    outs = [torch.tensor([[sp[0].data_ptr(), sp[1].data_ptr(), sp[2].data_ptr(), 0] for sp in spare], dtype=torch.int64).cuda(),
+            torch.tensor([[r[0], r[2], r[3], 0] for r in rows], dtype=torch.int64).cuda()]
+    redo = torch.zeros(len(sizes), dtype=torch.int32, device='cuda')
+    hyper = (3e-4, 0.9, 0.95, 1e-8, 0.1)
+    state = {'t': 1, 'side': 0}
 
     def step():
         state['t'] += 1
-        _backend.adamw_fused(desc, len(sizes), block_map, block_map.shape[0], _backend.DT_E4M3, _backend.DT_E5M2, 3e-4, 0.9,
-                             0.95, 1e-8, 0.1, state['t'], True, False, False, True, blocks_per_tensor=chunks)
+        i = state['side']
+        _backend.adamw_fused_speculative(descs[i], outs[i], redo, len(sizes), block_map, block_map.shape[0], _backend.DT_E4M3,
+                                         _backend.DT_E5M2, *hyper, state['t'], True, False, False, True)
+        state['side'] = 1 - i
 
-    ms = _time_gpu(step, iters, warm=2)
+    def step_in_place():
+        state['t'] += 1
+        _backend.adamw_fused(descs[state['side']], len(sizes), block_map, block_map.shape[0], _backend.DT_E4M3,
+                             _backend.DT_E5M2, *hyper, state['t'], True, False, False, True, blocks_per_tensor=chunks)
+
+    # 40 untimed steps first: the moments start far from where this gradient takes them, and while they travel there
+    # their power-of-two scales change every few steps, which a training run past its first steps does not see
+    ms = _time_gpu(step, iters, warm=40)
+    redone = int(redo.sum().item())
+    ms_in_place = _time_gpu(step_in_place, iters, warm=2)
     return {'ms': ms, 'Gparams_per_s': total_params / ms / 1e6, 'GBps_algorithmic': total_params * 9 / ms / 1e6,
-            'tensors': len(sizes), 'params': total_params}
+            'tensors': len(sizes), 'params': total_params, 'tensors_redone_in_last_step': redone,
+            'in_place_ms': ms_in_place, 'in_place_GBps_algorithmic': total_params * 9 / ms_in_place / 1e6}
 
 
 # ---- CPU baseline: the oracle on the host cores --------------------------------------------------------------
@@ -600,7 +622,11 @@ def main():
             'fused_adamw': {'ms': round(adam['ms'], 3), 'Gparams_per_s': round(adam['Gparams_per_s'], 1),
                             'GBps': round(adam['GBps_algorithmic'], 1),
                             'frac_hbm': round(adam['GBps_algorithmic'] / HBM_PEAK_GBS, 4), 'params': adam['params'],
-                            'tensors': adam['tensors']},
+                            'tensors': adam['tensors'], 'tensors_redone_in_last_step': adam['tensors_redone_in_last_step'],
+                            'mode': 'one pass between two sets of payload buffers (LBAdamW double_buffer=True)',
+                            'in_place_two_pass': {'ms': round(adam['in_place_ms'], 3),
+                                                  'GBps': round(adam['in_place_GBps_algorithmic'], 1),
+                                                  'frac_hbm': round(adam['in_place_GBps_algorithmic'] / HBM_PEAK_GBS, 4)}},
             'grad_side': _round_kernels(grad_side),
         }
     if not args.skip_cpu:

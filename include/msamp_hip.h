@@ -329,6 +329,32 @@ int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int3
                           int tensor_scale, const int32_t* blocks_per_tensor, int group_blocks,
                           msamp_stream_t stream);
 
+/* Output buffers of one tensor for the speculative form below: same sizes and types as the descriptor's weight,
+ * exp_avg and exp_avg_sq payloads, not overlapping them. */
+typedef struct msamp_adamw_buffers {
+    void* weight;
+    uint8_t* exp_avg;
+    uint16_t* exp_avg_sq;
+    uint64_t reserved;
+} msamp_adamw_buffers;
+
+/* msamp_adamw_fp8_fused with separate output buffers, in ONE pass over the data when the scales hold (not in the
+ * reference, whose optimizer is LBAdamW.adamw_fn, adamw.py:148-199, with two passes over every tensor).  Scales are
+ * powers of two and seldom change between steps, so the first launch reads w/g/m/v once, quantizes p', m', v' with
+ * the scales each tensor has NOW into outputs[t], and collects the three maxima; the second derives the scales from
+ * them as msamp_adamw_fp8_fused does, rewrites the metas and sets redo[t] = 1 where a scale differs from the one
+ * used; the third repeats exactly those tensors from their (untouched) inputs with the new scales.  On return the
+ * new payloads of EVERY tensor are in outputs[t] -- the same bits msamp_adamw_fp8_fused leaves in place -- the metas
+ * are updated, and the descriptors' weight / exp_avg / exp_avg_sq buffers still hold the old state: the caller swaps
+ * the two sets of buffers.  9 instead of 14 bytes of HBM traffic per parameter, at the price of 4 bytes per parameter
+ * of memory.  `outputs`: DEVICE array of n_tensors entries; `redo`: DEVICE array of n_tensors int32 written by the
+ * call (1 = the tensor took the second round).  Other arguments as for msamp_adamw_fp8_fused. */
+int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_adamw_buffers* outputs, int32_t* redo,
+                                      int n_tensors, const int32_t* block_map, int n_blocks, int weight_dtype,
+                                      int grad_dtype, double lr, double beta1, double beta2, double eps,
+                                      double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
+                                      int tensor_scale, msamp_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

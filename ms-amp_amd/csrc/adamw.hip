@@ -287,7 +287,8 @@ __global__ __launch_bounds__(kAdamThreads) void fused_amax_kernel(msamp_adamw_te
     }
 }
 
-__global__ void fused_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, float w_fp_max, int tensor_scale) {
+__global__ void fused_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, float w_fp_max, int tensor_scale,
+                                    int32_t* redo) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;    // `tensors` is pre-offset to the group's first tensor
     if (t >= n_tensors) return;
     msamp_adamw_tensor& d = tensors[t];
@@ -297,11 +298,17 @@ __global__ void fused_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, 
     d.saved[1] = 1.0f / *d.m_scale;
     d.saved[2] = 1.0f / *d.v_scale;
     const float ws = scale_rule(ap, *d.w_scale, w_fp_max, 0);
+    const float ms = tensor_scale ? scale_rule(am, 1.0f, 448.0f, 0) : 1.0f;
+    const float vs = tensor_scale ? scale_rule(av, 1.0f, 65504.0f, 0) : 1.0f;
+    // after the speculative pass (which used the scales as they were): is any of them different now?
+    if (redo != nullptr)
+        redo[t] = (__float_as_uint(ws) != __float_as_uint(*d.w_scale) || __float_as_uint(ms) != __float_as_uint(*d.m_scale) ||
+                   __float_as_uint(vs) != __float_as_uint(*d.v_scale))
+                      ? 1
+                      : 0;
     *d.w_scale = ws;
     *d.w_scale_inv = 1.0f / ws;
     *d.w_amax = ap;
-    const float ms = tensor_scale ? scale_rule(am, 1.0f, 448.0f, 0) : 1.0f;
-    const float vs = tensor_scale ? scale_rule(av, 1.0f, 65504.0f, 0) : 1.0f;
     *d.m_scale = ms;
     *d.m_scale_inv = 1.0f / ms;
     *d.m_amax = am;
@@ -351,9 +358,9 @@ __device__ __forceinline__ uint32_t quant_weight_exact(float pj, float m_new, fl
 
 // One lane's 16 elements of the second pass: requantized weight, exp_avg and exp_avg_sq are stored at element i.
 template <int WDT, bool L2>
-__device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i, float* p, const float* g, float* m,
-                                           float* v, float w_si, float g_si, float inv_m, float inv_v, float ws, float ms,
-                                           float vs, const AdamConsts& k) {
+__device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i, float* p, const float* g,
+                                           float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
+                                           float ms, float vs, const AdamConsts& k) {
     uint32_t wq[kEPT];
 #pragma unroll
     for (int j = 0; j < kEPT; ++j) {
@@ -378,7 +385,7 @@ __device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i
         v[j] = v_new * vs;
     }
     if constexpr (WDT == MSAMP_DT_F16) {
-        uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(d.weight) + i);
+        uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
         o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
         o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
     } else {
@@ -387,10 +394,10 @@ __device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i
         o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
         o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(d.weight) + i) = o;
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
     }
-    store_w16<MSAMP_DT_E4M3>(d.exp_avg, i, m);
-    store_w16<MSAMP_DT_F16>(d.exp_avg_sq, i, v);
+    store_w16<MSAMP_DT_E4M3>(m_out, i, m);
+    store_w16<MSAMP_DT_F16>(v_out, i, v);
 }
 
 // Second pass: recompute m', v' exactly and requantize them; for the weight, quantize both ends of the
@@ -399,10 +406,18 @@ __device__ __forceinline__ void write_step(const msamp_adamw_tensor& d, size_t i
 template <int WDT, int GDT, bool L2>
 __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_tensor* __restrict__ tensors,
                                                                     const int32_t* __restrict__ block_map,
-                                                                    AdamConsts k) {
+                                                                    AdamConsts k,
+                                                                    const msamp_adamw_buffers* __restrict__ outs,
+                                                                    const int32_t* __restrict__ redo) {
     const int b = gridDim.x - 1 - blockIdx.x;    // back to front: most recently read chunks first
     const int t = block_map[2 * b], chunk = block_map[2 * b + 1];
+    // after the speculative pass: only the tensors whose scales it guessed wrong are done again, from the untouched
+    // inputs, into the same output buffers
+    if (redo != nullptr && redo[t] == 0) return;
     msamp_adamw_tensor& d = tensors[t];
+    void* w_out = outs ? outs[t].weight : d.weight;
+    uint8_t* m_out = outs ? outs[t].exp_avg : d.exp_avg;
+    uint16_t* v_out = outs ? outs[t].exp_avg_sq : d.exp_avg_sq;
     const size_t n = d.numel;
     const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
     const float w_si = d.saved[0], g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv, inv_m = d.saved[1], inv_v = d.saved[2];
@@ -413,7 +428,7 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            write_step<WDT, L2>(d, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
+            write_step<WDT, L2>(w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
@@ -421,11 +436,136 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
             float pj, g_plain, m_new, v_new;
             prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
                     g_plain, m_new, v_new);
-            store_w1<WDT>(d.weight, i, param_update(pj, m_new, v_new, k) * ws);
+            store_w1<WDT>(w_out, i, param_update(pj, m_new, v_new, k) * ws);
             if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
-            store_w1<MSAMP_DT_E4M3>(d.exp_avg, i, m_new * ms);
-            store_w1<MSAMP_DT_F16>(d.exp_avg_sq, i, v_new * vs);
+            store_w1<MSAMP_DT_E4M3>(m_out, i, m_new * ms);
+            store_w1<MSAMP_DT_F16>(v_out, i, v_new * vs);
         }
+    }
+}
+
+// ---- speculative single pass -------------------------------------------------------------------
+// The scales of a tensor are powers of two and seldom change from one step to the next.  With separate output
+// buffers the step can therefore be taken in ONE pass over the data: quantize p', m', v' with the scales the tensor
+// has now, find the three maxima on the way, and let fused_scales_kernel compare the scales the rule gives with the
+// ones used.  Where they agree the output is what the two passes above produce, bit for bit; a tensor where they do
+// not is done again by fused_write_kernel from its inputs, which this pass does not touch.
+//
+// One lane's 16 elements: as write_step, plus the maxima.  |m'| and |v'| are exact.  For |p'| the estimate gives
+// |p_est| - err <= |p'| <= |p_est| + err; only elements whose upper end reaches the best lower end seen so far are
+// evaluated exactly, and the element that attains the maximum always is.
+template <int WDT, bool L2>
+__device__ __forceinline__ void spec_step(void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i, float* p, const float* g,
+                                          float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
+                                          float ms, float vs, const AdamConsts& k, float& floor_p, uint32_t& mxp,
+                                          float& mxm, float& mxv) {
+    uint32_t wq[kEPT];
+    float hi[kEPT], mm[kEPT], vv[kEPT];
+    float lo_max = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kEPT; ++j) {
+        float pj, g_plain, m_new, v_new, p_est, err;
+        prepare<L2>(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+        mxm = fmaxf(mxm, fabsf(m_new));
+        mxv = fmaxf(mxv, fabsf(v_new));
+        estimate(pj, m_new, v_new, k, p_est, err);
+        const float lo = (p_est - err) * ws, up = (p_est + err) * ws;
+        bool same;
+        uint32_t code;
+        if constexpr (WDT == MSAMP_DT_F16) {
+            code = float_to_f16_bits(lo);
+            same = code == float_to_f16_bits(up);
+        } else {
+            const uint32_t two = cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(up), 0u, false);
+            code = two & 0xffu;
+            same = code == ((two >> 8) & 0xffu);
+        }
+        if (!(same && err < __uint_as_float(0x7f800000u))) code = quant_weight_exact<WDT>(pj, m_new, v_new, ws, k);
+        wq[j] = code;
+        hi[j] = fabsf(p_est) + err;                       // NaN for anything non-finite: evaluated exactly below
+        lo_max = fmaxf(lo_max, fabsf(p_est) - err);       // fmaxf skips a NaN
+        p[j] = pj, mm[j] = m_new, vv[j] = v_new;
+        if constexpr (L2) moments(m[j], v[j], g_plain, inv_m, inv_v, k, m_new, v_new);    // stored moments ignore the L2 term
+        m[j] = m_new * ms;
+        v[j] = v_new * vs;
+    }
+    if constexpr (WDT == MSAMP_DT_F16) {
+        uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
+        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
+        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
+    } else {
+        uint4 o;
+        o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
+        o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
+        o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
+        o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
+    }
+    store_w16<MSAMP_DT_E4M3>(m_out, i, m);
+    store_w16<MSAMP_DT_F16>(v_out, i, v);
+    floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
+    const float skip_below = floor_p * 0.999999f;    // room for the roundings of the bounds themselves
+#pragma unroll
+    for (int j = 0; j < kEPT; ++j) {
+        if (!(hi[j] < skip_below)) {
+            const uint32_t ab = __float_as_uint(param_update(p[j], mm[j], vv[j], k)) & 0x7fffffffu;
+            mxp = ab > mxp ? ab : mxp;
+        }
+    }
+}
+
+template <int WDT, int GDT, bool L2>
+__global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_tensor* __restrict__ tensors,
+                                                                   const int32_t* __restrict__ block_map, AdamConsts k,
+                                                                   const msamp_adamw_buffers* __restrict__ outs) {
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
+    msamp_adamw_tensor& d = tensors[t];
+    void* w_out = outs[t].weight;
+    uint8_t* m_out = outs[t].exp_avg;
+    uint16_t* v_out = outs[t].exp_avg_sq;
+    const size_t n = d.numel;
+    const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
+    const float w_si = *d.w_scale_inv, g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv;
+    const float ws = *d.w_scale, ms = *d.m_scale, vs = *d.v_scale;    // the guess: the scales in force
+    const float inv_m = 1.0f / ms, inv_v = 1.0f / vs;
+    uint32_t mxp = 0;
+    float mxm = 0.0f, mxv = 0.0f;
+    float floor_p = __uint_as_float(__hip_atomic_load(&d.acc[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    if (!(floor_p >= 0.0f)) floor_p = 0.0f;
+    if (base + MSAMP_ADAMW_CHUNK <= n) {
+#pragma unroll 1
+        for (int s = 0; s < kSteps; ++s) {
+            const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
+            float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
+            load16<WDT, GDT>(d, i, p, g, m, v);
+            spec_step<WDT, L2>(w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p, mxp,
+                               mxm, mxv);
+        }
+    } else {
+        for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
+            const float m_old = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v_old = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
+            float pj, g_plain, m_new, v_new;
+            prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
+                    g_plain, m_new, v_new);
+            const float pn = param_update(pj, m_new, v_new, k);
+            const uint32_t ab = __float_as_uint(pn) & 0x7fffffffu;
+            mxp = ab > mxp ? ab : mxp;
+            mxm = fmaxf(mxm, fabsf(m_new));
+            mxv = fmaxf(mxv, fabsf(v_new));
+            store_w1<WDT>(w_out, i, pn * ws);
+            if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
+            store_w1<MSAMP_DT_E4M3>(m_out, i, m_new * ms);
+            store_w1<MSAMP_DT_F16>(v_out, i, v_new * vs);
+        }
+    }
+    const uint32_t a = block_max_u32(mxp, red);
+    const uint32_t b = block_max_u32(__float_as_uint(mxm), red);
+    const uint32_t c = block_max_u32(__float_as_uint(mxv), red);
+    if (threadIdx.x == 0) {
+        if (a) atomicMax(&d.acc[0], a);
+        if (b) atomicMax(&d.acc[1], b);
+        if (c) atomicMax(&d.acc[2], c);
     }
 }
 
@@ -505,18 +645,11 @@ int msamp_adamw_fp8_stage2(const float* grad, size_t n, void* exp_avg, int exp_a
     return MSAMP_OK;
 }
 
-int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int32_t* block_map, int n_blocks,
-                          int weight_dtype, int grad_dtype, double lr, double beta1, double beta2, double eps,
-                          double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
-                          int tensor_scale, const int32_t* blocks_per_tensor, int group_blocks, msamp_stream_t stream) {
-    MSAMP_REQUIRE(n_tensors >= 0 && n_blocks >= 0, MSAMP_ERR_SHAPE, "msamp_adamw_fp8_fused: n_tensors=%d n_blocks=%d",
-                  n_tensors, n_blocks);
-    if (n_tensors == 0 || n_blocks == 0) return MSAMP_OK;
-    MSAMP_REQUIRE(tensors && block_map, MSAMP_ERR_NULL, "msamp_adamw_fp8_fused: null pointer");
-    MSAMP_REQUIRE(weight_dtype == MSAMP_DT_E4M3 || weight_dtype == MSAMP_DT_E5M2 || weight_dtype == MSAMP_DT_F16,
-                  MSAMP_ERR_DTYPE, "msamp_adamw_fp8_fused: weight dtype %d", weight_dtype);
-    MSAMP_REQUIRE(is_fp8(grad_dtype), MSAMP_ERR_DTYPE, "msamp_adamw_fp8_fused: grad dtype %d", grad_dtype);
-    AdamConsts k = {};
+// hyper-parameters of the fused step, narrowed the way the reference narrows them; returns whether the decay is an
+// L2 term on the gradient (Adam mode)
+static bool fused_consts(double lr, double beta1, double beta2, double eps, double weight_decay, int step,
+                         int bias_correction, int adam_mode, int maximize, AdamConsts& k) {
+    k = AdamConsts{};
     k.beta1 = static_cast<float>(beta1), k.beta2 = static_cast<float>(beta2);
     k.omb1 = 1.0f - k.beta1, k.omb2 = 1.0f - k.beta2;
     k.eps = static_cast<float>(eps);
@@ -534,30 +667,56 @@ int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int3
     k.bound_eps = k.eps > 0.0f ? nextafterf(static_cast<float>(abs_step / k.eps * widen), inf) : inf;
     if (!(k.bound_rsq >= 0.0f)) k.bound_rsq = inf;
     if (!(k.bound_eps >= 0.0f)) k.bound_eps = inf;
-    const float w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-#define FUSED_LAUNCH_WG(KERNEL, NB, BM, W, G)                                                                          \
+    return l2;
+}
+
+static int fused_args_ok(const char* who, const void* tensors, int n_tensors, const void* block_map, int n_blocks,
+                         int weight_dtype, int grad_dtype) {
+    MSAMP_REQUIRE(n_tensors >= 0 && n_blocks >= 0, MSAMP_ERR_SHAPE, "%s: n_tensors=%d n_blocks=%d", who, n_tensors, n_blocks);
+    if (n_tensors == 0 || n_blocks == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(tensors && block_map, MSAMP_ERR_NULL, "%s: null pointer", who);
+    MSAMP_REQUIRE(weight_dtype == MSAMP_DT_E4M3 || weight_dtype == MSAMP_DT_E5M2 || weight_dtype == MSAMP_DT_F16,
+                  MSAMP_ERR_DTYPE, "%s: weight dtype %d", who, weight_dtype);
+    MSAMP_REQUIRE(is_fp8(grad_dtype), MSAMP_ERR_DTYPE, "%s: grad dtype %d", who, grad_dtype);
+    return MSAMP_OK;
+}
+
+// launch KERNEL<weight type, gradient type, l2> for the runtime types
+#define FUSED_LAUNCH_WG(KERNEL, NB, W, G, ...)                                                                        \
     do {                                                                                                              \
         if (l2)                                                                                                       \
-            hipLaunchKernelGGL((KERNEL<W, G, true>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k);            \
+            hipLaunchKernelGGL((KERNEL<W, G, true>), dim3(NB), dim3(kAdamThreads), 0, st, __VA_ARGS__);               \
         else                                                                                                          \
-            hipLaunchKernelGGL((KERNEL<W, G, false>), dim3(NB), dim3(kAdamThreads), 0, st, tensors, BM, k);           \
+            hipLaunchKernelGGL((KERNEL<W, G, false>), dim3(NB), dim3(kAdamThreads), 0, st, __VA_ARGS__);              \
     } while (0)
-#define FUSED_LAUNCH(KERNEL, NB, BM)                                                                                  \
+#define FUSED_LAUNCH(KERNEL, NB, ...)                                                                                 \
     do {                                                                                                              \
         if (weight_dtype == MSAMP_DT_E4M3 && grad_dtype == MSAMP_DT_E4M3)                                             \
-            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E4M3, MSAMP_DT_E4M3);                                            \
+            FUSED_LAUNCH_WG(KERNEL, NB, MSAMP_DT_E4M3, MSAMP_DT_E4M3, __VA_ARGS__);                                   \
         else if (weight_dtype == MSAMP_DT_E4M3)                                                                       \
-            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E4M3, MSAMP_DT_E5M2);                                            \
+            FUSED_LAUNCH_WG(KERNEL, NB, MSAMP_DT_E4M3, MSAMP_DT_E5M2, __VA_ARGS__);                                   \
         else if (weight_dtype == MSAMP_DT_E5M2 && grad_dtype == MSAMP_DT_E4M3)                                        \
-            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E5M2, MSAMP_DT_E4M3);                                            \
+            FUSED_LAUNCH_WG(KERNEL, NB, MSAMP_DT_E5M2, MSAMP_DT_E4M3, __VA_ARGS__);                                   \
         else if (weight_dtype == MSAMP_DT_E5M2)                                                                       \
-            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_E5M2, MSAMP_DT_E5M2);                                            \
+            FUSED_LAUNCH_WG(KERNEL, NB, MSAMP_DT_E5M2, MSAMP_DT_E5M2, __VA_ARGS__);                                   \
         else if (grad_dtype == MSAMP_DT_E4M3)                                                                         \
-            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_F16, MSAMP_DT_E4M3);                                             \
+            FUSED_LAUNCH_WG(KERNEL, NB, MSAMP_DT_F16, MSAMP_DT_E4M3, __VA_ARGS__);                                    \
         else                                                                                                          \
-            FUSED_LAUNCH_WG(KERNEL, NB, BM, MSAMP_DT_F16, MSAMP_DT_E5M2);                                             \
+            FUSED_LAUNCH_WG(KERNEL, NB, MSAMP_DT_F16, MSAMP_DT_E5M2, __VA_ARGS__);                                    \
     } while (0)
+
+int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int32_t* block_map, int n_blocks,
+                          int weight_dtype, int grad_dtype, double lr, double beta1, double beta2, double eps,
+                          double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
+                          int tensor_scale, const int32_t* blocks_per_tensor, int group_blocks, msamp_stream_t stream) {
+    const int rc = fused_args_ok("msamp_adamw_fp8_fused", tensors, n_tensors, block_map, n_blocks, weight_dtype, grad_dtype);
+    if (rc != MSAMP_OK || n_tensors == 0 || n_blocks == 0) return rc;
+    AdamConsts k;
+    const bool l2 = fused_consts(lr, beta1, beta2, eps, weight_decay, step, bias_correction, adam_mode, maximize, k);
+    const float w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const msamp_adamw_buffers* in_place = nullptr;
+    const int32_t* every_tensor = nullptr;
     // Groups of whole tensors, each small enough that what the first pass read (5 B/param) and what
     // the second writes (4 B/param) stay in the 256 MB Infinity Cache: the second pass then re-reads
     // from cache and HBM sees 9 B/param.  Without the per-tensor block counts everything is one group.
@@ -575,21 +734,46 @@ int msamp_adamw_fp8_fused(msamp_adamw_tensor* tensors, int n_tensors, const int3
         MSAMP_REQUIRE(b1 <= n_blocks, MSAMP_ERR_SHAPE, "msamp_adamw_fp8_fused: blocks_per_tensor exceeds n_blocks");
         const int nb = b1 - b0, nt = t1 - t0;
         if (nb > 0) {
-            FUSED_LAUNCH(fused_amax_kernel, nb, block_map + 2 * b0);
+            FUSED_LAUNCH(fused_amax_kernel, nb, tensors, block_map + 2 * b0, k);
             MSAMP_CHECK_LAUNCH("fused_amax_kernel");
         }
         hipLaunchKernelGGL(fused_scales_kernel, dim3((nt + 63) / 64), dim3(64), 0, st, tensors + t0, nt, w_fp_max,
-                           tensor_scale);
+                           tensor_scale, static_cast<int32_t*>(nullptr));
         MSAMP_CHECK_LAUNCH("fused_scales_kernel");
         if (nb > 0) {
-            FUSED_LAUNCH(fused_write_kernel, nb, block_map + 2 * b0);
+            FUSED_LAUNCH(fused_write_kernel, nb, tensors, block_map + 2 * b0, k, in_place, every_tensor);
             MSAMP_CHECK_LAUNCH("fused_write_kernel");
         }
         t0 = t1, b0 = b1;
     }
-#undef FUSED_LAUNCH
-#undef FUSED_LAUNCH_WG
     return MSAMP_OK;
 }
+
+int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_adamw_buffers* outputs, int32_t* redo,
+                                      int n_tensors, const int32_t* block_map, int n_blocks, int weight_dtype,
+                                      int grad_dtype, double lr, double beta1, double beta2, double eps,
+                                      double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
+                                      int tensor_scale, msamp_stream_t stream) {
+    const int rc = fused_args_ok("msamp_adamw_fp8_fused_speculative", tensors, n_tensors, block_map, n_blocks, weight_dtype,
+                                 grad_dtype);
+    if (rc != MSAMP_OK || n_tensors == 0 || n_blocks == 0) return rc;
+    MSAMP_REQUIRE(outputs && redo, MSAMP_ERR_NULL, "msamp_adamw_fp8_fused_speculative: null outputs or redo");
+    AdamConsts k;
+    const bool l2 = fused_consts(lr, beta1, beta2, eps, weight_decay, step, bias_correction, adam_mode, maximize, k);
+    const float w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    FUSED_LAUNCH(fused_spec_kernel, n_blocks, tensors, block_map, k, outputs);
+    MSAMP_CHECK_LAUNCH("fused_spec_kernel");
+    hipLaunchKernelGGL(fused_scales_kernel, dim3((n_tensors + 63) / 64), dim3(64), 0, st, tensors, n_tensors, w_fp_max,
+                       tensor_scale, redo);
+    MSAMP_CHECK_LAUNCH("fused_scales_kernel");
+    // the tensors whose scales changed, again, with the scales just written; every other workgroup returns at once
+    const int32_t* redo_in = redo;
+    FUSED_LAUNCH(fused_write_kernel, n_blocks, tensors, block_map, k, outputs, redo_in);
+    MSAMP_CHECK_LAUNCH("fused_write_kernel");
+    return MSAMP_OK;
+}
+#undef FUSED_LAUNCH
+#undef FUSED_LAUNCH_WG
 
 }    // extern "C"

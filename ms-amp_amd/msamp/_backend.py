@@ -58,6 +58,7 @@ _SIGNATURES = {
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_adamw_fp8_fused_speculative': ([_vp, _vp, _vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -622,6 +623,7 @@ def adamw_stage2(grad, exp_avg, exp_avg_dt, old_factor, new_factor, beta1, exp_a
 
 
 ADAMW_DESC_WORDS = 19    # int64 words per msamp_adamw_tensor (152 bytes)
+ADAMW_BUFFER_WORDS = 4    # int64 words per msamp_adamw_buffers (weight, exp_avg, exp_avg_sq, reserved)
 
 
 # chunks per cache-resident group of the fused AdamW step; 0 = one group (the kernels are compute-bound, so
@@ -644,4 +646,26 @@ def adamw_fused(desc, n_tensors, block_map, n_blocks, weight_dt, grad_dt, lr, be
             step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0, 1 if tensor_scale else 0,
             ctypes.cast(bpt, ctypes.c_void_p) if bpt is not None else None, gb if bpt is not None else 0, _stream()
         ), 'msamp_adamw_fp8_fused'
+    )
+
+
+def adamw_fused_speculative(desc, outputs, redo, n_tensors, block_map, n_blocks, weight_dt, grad_dt, lr, beta1, beta2, eps,
+                            weight_decay, step, bias_correction, adam_mode, maximize, tensor_scale):
+    """The fused step in one pass into separate buffers.  `outputs`: int64 device tensor [n_tensors, ADAMW_BUFFER_WORDS]
+    of output pointers; `redo`: int32 device tensor [n_tensors], set by the call where a tensor took the second round.
+    On return every tensor's new payloads are in its output buffers; the inputs still hold the old state."""
+    lib = load()
+    _gpu(desc, 'descriptor table')
+    _gpu(outputs, 'output table')
+    _gpu(redo, 'redo flags')
+    if outputs.dtype != torch.int64 or outputs.numel() != n_tensors * ADAMW_BUFFER_WORDS or not outputs.is_contiguous():
+        raise ValueError('outputs must be a contiguous int64 tensor of n_tensors x %d words' % ADAMW_BUFFER_WORDS)
+    if redo.dtype != torch.int32 or redo.numel() != n_tensors or not redo.is_contiguous():
+        raise ValueError('redo must be a contiguous int32 tensor of n_tensors flags')
+    _check(
+        lib.msamp_adamw_fp8_fused_speculative(
+            _ptr(desc), _ptr(outputs), _ptr(redo), n_tensors, _ptr(block_map), n_blocks, weight_dt, grad_dt, lr, beta1, beta2,
+            eps, weight_decay, step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0,
+            1 if tensor_scale else 0, _stream()
+        ), 'msamp_adamw_fp8_fused_speculative'
     )

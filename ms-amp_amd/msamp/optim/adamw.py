@@ -22,9 +22,17 @@ class LBAdamW(LBAdamWBase):
     """AdamW with low-bit moments (default: E4M3 exp_avg, scaled-fp16 exp_avg_sq)."""
     def __init__(self, params, lr=1e-3, bias_correction=True, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2,
                  amsgrad=False, *, maximize=False, exp_avg_dtype=torch.uint8, exp_avg_sq_dtype=torch.float16,
-                 tensor_scale=True):
+                 tensor_scale=True, double_buffer=True):
+        """double_buffer (not in the reference): the fused step writes the new weight and moment payloads into a second
+        set of buffers (4 more bytes per parameter) and swaps the two sets afterwards, which lets it read every tensor
+        once instead of twice; the values are the same bit for bit.  The payload tensors (`.value`) remain the same
+        objects, but their memory alternates between two addresses: pass False when something holds those addresses
+        (a captured graph of the forward pass, views taken of `.value`).  Payloads that are themselves views of other
+        storage (a flat buffer) and steps taken under stream capture keep the in-place step."""
         self.tensor_scale = tensor_scale
+        self.double_buffer = double_buffer
         self._fused_cache = {}
+        self._spare = {}    # id(parameter) -> [weight, exp_avg, exp_avg_sq] payload buffers not in use right now
         super().__init__(
             params, lr=lr, bias_correction=bias_correction, betas=betas, eps=eps, weight_decay=weight_decay,
             amsgrad=False, maximize=maximize, exp_avg_dtype=exp_avg_dtype, exp_avg_sq_dtype=exp_avg_sq_dtype
@@ -80,12 +88,55 @@ class LBAdamW(LBAdamWBase):
         ps, gs = [params[i] for i in idx], [grads[i] for i in idx]
         ms, vs = [exp_avgs[i] for i in idx], [exp_avg_sqs[i] for i in idx]
         wq, gq = ps[0].qtype, gs[0].qtype
+        if self.double_buffer and self._can_swap(ps, ms, vs):
+            # the payload pointers alternate between two sets from step to step: one cached table per set
+            key = (int(wq), int(gq), id(ps[0]), ps[0].value.data_ptr())
+            desc, block_map, n_blocks, _ = self._fused_tables(key, ps, gs, ms, vs)
+            spares = [self._spare_buffers(p, m, v) for p, m, v in zip(ps, ms, vs)]
+            outputs, redo = self._output_tables(key, spares)
+            _backend.adamw_fused_speculative(
+                desc, outputs, redo, len(ps), block_map, n_blocks, int(wq), int(gq), lr, beta1, beta2, eps, weight_decay, step,
+                self.bias_correction, self.use_adam, maximize, self.tensor_scale
+            )
+            # the payload tensors stay the objects they were and trade their memory with the spares
+            for p, m, v, spare in zip(ps, ms, vs, spares):
+                for i, t in enumerate((p.value, m.value, v.value)):
+                    old = t.data
+                    t.data = spare[i]
+                    spare[i] = old
+            return
         key = (int(wq), int(gq), id(ps[0]))
         desc, block_map, n_blocks, chunks = self._fused_tables(key, ps, gs, ms, vs)
         _backend.adamw_fused(
             desc, len(ps), block_map, n_blocks, int(wq), int(gq), lr, beta1, beta2, eps, weight_decay, step,
             self.bias_correction, self.use_adam, maximize, self.tensor_scale, blocks_per_tensor=chunks
         )
+
+    @staticmethod
+    def _can_swap(ps, ms, vs):
+        """Swapping payload tensors is safe when nothing else aliases them and no graph is recording their addresses."""
+        if torch.cuda.is_current_stream_capturing():
+            return False
+        return all(t.value._base is None for group in (ps, ms, vs) for t in group)
+
+    def _spare_buffers(self, p, m, v):
+        spare = self._spare.get(id(p))
+        current = (p.value, m.value, v.value)
+        if spare is None or any(s.shape != c.shape or s.dtype != c.dtype or s.device != c.device for s, c in zip(spare, current)):
+            spare = [torch.empty_like(c) for c in current]
+            self._spare[id(p)] = spare
+        return spare
+
+    def _output_tables(self, key, spares):
+        rows = tuple((s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), 0) for s in spares)
+        cached = self._fused_cache.get(('out', ) + key)
+        if cached is not None and cached[0] == rows:
+            return cached[1], cached[2]
+        device = spares[0][0].device
+        outputs = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), _backend.ADAMW_BUFFER_WORDS)).to(device)
+        redo = torch.zeros(len(rows), dtype=torch.int32, device=device)
+        self._fused_cache[('out', ) + key] = (rows, outputs, redo)
+        return outputs, redo
 
     # ---- per-tensor path (reference recipe) -----------------------------------------------
     def _staged_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, state_steps, *, beta1, beta2, lr, weight_decay,

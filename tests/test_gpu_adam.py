@@ -73,6 +73,23 @@ def _fused(be, tensors, w_dt, g_dt, step, **kw):
     block_map = torch.from_numpy(bm).cuda()
     hyper = dict(HYPER)
     hyper.update(kw)
+    if hyper.get('speculative'):
+        # one pass into separate buffers: afterwards the inputs are untouched and the outputs hold the new state
+        before = [(d['w'].clone(), d['m'].clone(), d['v'].clone()) for d in dev]
+        outs = [(torch.full_like(d['w'], 0x55), torch.full_like(d['m'], 0x55), torch.full_like(d['v'], 0x55)) for d in dev]
+        table = torch.tensor([[o[0].data_ptr(), o[1].data_ptr(), o[2].data_ptr(), 0] for o in outs], dtype=torch.int64).cuda()
+        redo = torch.full((len(dev), ), -1, dtype=torch.int32, device='cuda')
+        be.adamw_fused_speculative(desc, table, redo, len(tensors), block_map, block_map.shape[0], w_dt, g_dt, hyper['lr'],
+                                   hyper['beta1'], hyper['beta2'], hyper['eps'], hyper['weight_decay'], step,
+                                   hyper.get('bias_correction', True), hyper.get('adam_mode', False),
+                                   hyper.get('maximize', False), hyper.get('tensor_scale', True))
+        torch.cuda.synchronize()
+        for d, b, o, r in zip(dev, before, outs, redo.tolist()):
+            assert torch.equal(d['w'], b[0]) and torch.equal(d['m'], b[1]) and torch.equal(d['v'].view(torch.int16), b[2].view(torch.int16))
+            d['w'], d['m'], d['v'] = o
+            d['redo'] = r
+        assert (desc[:, 15].cpu() == 0).all()
+        return dev
     be.adamw_fused(desc, len(tensors), block_map, block_map.shape[0], w_dt, g_dt, hyper['lr'], hyper['beta1'], hyper['beta2'],
                    hyper['eps'], hyper['weight_decay'], step, hyper.get('bias_correction', True), hyper.get('adam_mode', False),
                    hyper.get('maximize', False), hyper.get('tensor_scale', True), blocks_per_tensor=chunks,
@@ -197,6 +214,83 @@ def test_fused_step_sparse_gradient_and_zero_state(be):
     for step, kw in ((1, dict()), (1, dict(adam_mode=True)), (3, dict(maximize=True))):
         dev = _fused(be, [t], 5, 6, step, **kw)
         _check(dev[0], t, fp8.E4M3, fp8.E5M2, step, **kw)
+
+
+def _same_state(a, b):
+    bits = lambda t: t.view(torch.int32) if t.dtype == torch.float32 else (t.view(torch.int16) if t.dtype == torch.float16 else t)
+    return all(torch.equal(bits(x), bits(y)) for x, y in zip([a['w'], a['m'], a['v']] + a['wm'] + a['mm'] + a['vm'],
+                                                             [b['w'], b['m'], b['v']] + b['wm'] + b['mm'] + b['vm']))
+
+
+def _next_inputs(t, dev, seed, g_fmt, grad_std=1e-3):
+    """The state a fused step left on the device as the input of the next step, with a fresh gradient."""
+    meta = lambda m: dict(scale=m[0].cpu().reshape(()), scale_inv=m[1].cpu().reshape(()), amax=m[2].cpu())
+    gq, gm = _quant(grad_std * torch.randn(t['w'].numel(), generator=torch.Generator().manual_seed(seed)), g_fmt)
+    return dict(w=dev['w'].cpu(), wm=meta(dev['wm']), g=gq, gm=gm, m=dev['m'].cpu(), mm=meta(dev['mm']), v=dev['v'].cpu(),
+                vm=meta(dev['vm']))
+
+
+@pytest.mark.parametrize('w_fmt,w_dt,g_fmt,g_dt', [(fp8.E4M3, 5, fp8.E5M2, 6), ('f16', 3, fp8.E4M3, 5), (fp8.E5M2, 6, fp8.E4M3, 5)])
+def test_speculative_step_equals_the_in_place_step(be, w_fmt, w_dt, g_fmt, g_dt):
+    """Four steps in a row, each taken both ways from the same state: the one-pass step into separate buffers leaves the
+    bits of the two-pass step, whether its guess (the scales in force) holds or not.  The first step starts from zero
+    moments with scale 1, so every guess is wrong; later steps with gradients of the same size keep their scales; a
+    gradient sixteen times larger moves the moment scales of that step."""
+    sizes = [16384 * 4, 16384 * 2 + 777, 5, 4096 * 1024, 16384]
+    tensors = [_inputs(n, 400 + i, w_fmt, g_fmt, zero_state=True) for i, n in enumerate(sizes)]
+    hits = misses = 0
+    for step in range(1, 5):
+        plain = _fused(be, tensors, w_dt, g_dt, step)
+        spec = _fused(be, tensors, w_dt, g_dt, step, speculative=True)
+        for a, b, t in zip(plain, spec, tensors):
+            assert _same_state(a, b), (step, t['w'].numel())
+            assert b['redo'] in (0, 1)
+            moved = not (same_float(a['wm'][0], t['wm']['scale']) and same_float(a['mm'][0], t['mm']['scale']) and
+                         same_float(a['vm'][0], t['vm']['scale']))
+            assert b['redo'] == int(moved)
+            hits += 1 - b['redo']
+            misses += b['redo']
+        _check(spec[3], tensors[3], w_fmt, g_fmt, step)
+        tensors = [_next_inputs(t, d, 500 + 10 * step + i, g_fmt, grad_std=1.6e-2 if step == 3 else 1e-3)
+                   for i, (t, d) in enumerate(zip(tensors, plain))]
+    assert hits >= 3 and misses >= len(sizes)
+
+
+@pytest.mark.parametrize('kw', [dict(adam_mode=True), dict(maximize=True), dict(bias_correction=False), dict(weight_decay=0.0),
+                                dict(tensor_scale=False), dict(lr=0.5, eps=0.0)])
+def test_speculative_step_variants(be, kw):
+    t = _inputs(16384 * 3 + 100, 7, fp8.E4M3, fp8.E5M2)
+    for step in (2, 3):
+        plain = _fused(be, [t], 5, 6, step, **kw)[0]
+        spec = _fused(be, [t], 5, 6, step, speculative=True, **kw)[0]
+        assert _same_state(plain, spec)
+        _check(spec, t, fp8.E4M3, fp8.E5M2, step, **kw)
+        t = _next_inputs(t, plain, 60 + step, fp8.E5M2)
+
+
+def test_speculative_step_special_values(be):
+    """A NaN second moment (NaN weight amax, scale kept), zero gradients on zero state, and the largest |p'| coming from
+    the update term: same bits as the in-place step in each case."""
+    n = 16384 * 3
+    t = _inputs(n, 56, fp8.E4M3, fp8.E5M2)
+    t['v'].view(torch.int16)[16384 + 4321] = 0x7E00
+    plain, spec = _fused(be, [t], 5, 6, 2)[0], _fused(be, [t], 5, 6, 2, speculative=True)[0]
+    assert torch.isnan(spec['wm'][2][0]).item() and _same_state(plain, spec)
+    t = _inputs(16384 * 5 + 321, 91, fp8.E4M3, fp8.E5M2, zero_state=True)
+    t['g'][torch.rand(t['g'].numel(), generator=torch.Generator().manual_seed(92)) < 0.9] = 0
+    for step, kw in ((1, dict()), (1, dict(adam_mode=True))):
+        assert _same_state(_fused(be, [t], 5, 6, step, **kw)[0], _fused(be, [t], 5, 6, step, speculative=True, **kw)[0])
+    n = 16384 * 6 + 48
+    t = _inputs(n, 55, fp8.E4M3, fp8.E5M2)
+    for idx in (5, 16384 * 2 + 17, n - 3):
+        t['v'][idx] = 0.0
+        t['m'][idx] = 0x7E if idx != 5 else 0xFE
+        t['g'][idx] = 0
+        t['w'][idx] = 0x01
+    for kw in (dict(lr=0.5), dict(lr=0.5, eps=0.0), dict()):
+        spec = _fused(be, [t], 5, 6, 2, speculative=True, **kw)[0]
+        assert _same_state(_fused(be, [t], 5, 6, 2, **kw)[0], spec)
+        _check(spec, t, fp8.E4M3, fp8.E5M2, 2, **kw)
 
 
 def test_fused_step_is_deterministic(be):

@@ -314,6 +314,41 @@ def test_fused_adamw_only_for_weights_under_in_time_scaling(monkeypatch):
     assert torch.allclose(w_fused, w_staged, rtol=0, atol=float(w_fused.abs().max()) * 2e-3)
 
 
+def test_double_buffered_adamw_matches_the_in_place_step():
+    """LBAdamW(double_buffer=True) takes the fused step in one pass into spare buffers and swaps memory afterwards: same
+    weights, moments and metas as double_buffer=False after every step, with the payload tensors staying the objects
+    they were while their addresses alternate."""
+    torch.manual_seed(13)
+    lin = torch.nn.Sequential(torch.nn.Linear(256, 512, bias=False), torch.nn.Linear(512, 128, bias=False)).cuda()
+    x = torch.randn(64, 256, device='cuda')
+    runs = {}
+    for double in (False, True):
+        model_state.clear()
+        model = LinearReplacer.replace(copy.deepcopy(lin), Dtypes.kfloat8_e4m3)
+        opt = LBAdamW(model.parameters(), lr=1e-2, double_buffer=double)
+        values = [p.value for p in model.parameters()]
+        addresses = []
+        history = []
+        for step in range(5):
+            model(x * (1 + step)).square().mean().backward()
+            opt.all_reduce_grads(model)
+            opt.step()
+            opt.zero_grad()
+            addresses.append([p.value.data_ptr() for p in model.parameters()])
+            history.append([(p.value.clone(), p.meta.scale.clone(), opt.state[p]['exp_avg'].value.clone(),
+                             opt.state[p]['exp_avg'].meta.scale.clone(), opt.state[p]['exp_avg_sq'].value.clone(),
+                             opt.state[p]['exp_avg_sq'].meta.scale.clone()) for p in model.parameters()])
+        assert all(p.value is v for p, v in zip(model.parameters(), values))
+        if double:
+            assert addresses[0] != addresses[1] and addresses[0] == addresses[2] and addresses[1] == addresses[3]
+        else:
+            assert all(a == addresses[0] for a in addresses)
+        runs[double] = history
+    for a, b in zip(runs[False], runs[True]):
+        for pa, pb in zip(a, b):
+            assert all(torch.equal(ta, tb) for ta, tb in zip(pa, pb))
+
+
 def test_historical_window_quantization():
     model = LinearReplacer.replace(torch.nn.Linear(4, 8).cuda(), Dtypes.kfloat16)
     opt = LBAdamW(model.parameters())
