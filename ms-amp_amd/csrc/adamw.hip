@@ -183,10 +183,12 @@ __device__ __forceinline__ void prepare(float w_raw, float g_raw, float m_old, f
 // reciprocal, and a bound on its distance from the exactly rounded chain of param_update():
 // the update term is off by at most 13 unit roundoffs, the subtraction adds one rounding on each side.
 // Non-finite inputs make the bound NaN, which every caller treats as "take the exact path".
-__device__ __forceinline__ void estimate(float pj, float m_new, float v_new, const AdamConsts& k, float& p_est,
+// `eps_v` is k.eps held in a vector register (an instruction takes one scalar operand only: with eps in a scalar
+// register next to inv_sbc2 every element would pay for a move).
+__device__ __forceinline__ void estimate(float pj, float m_new, float v_new, const AdamConsts& k, float eps_v, float& p_est,
                                          float& err) {
     const float root = __builtin_amdgcn_sqrtf(v_new);
-    const float den = fmaf(root, k.inv_sbc2, k.eps);
+    const float den = fmaf(root, k.inv_sbc2, eps_v);
     const float r = m_new * __builtin_amdgcn_rcpf(den);
     const float d = k.step_size * r;
     p_est = pj - d;
@@ -362,11 +364,13 @@ __device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t
                                            float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
                                            float ms, float vs, const AdamConsts& k) {
     uint32_t wq[kEPT];
+    float eps_v = k.eps;
+    asm volatile("" : "+v"(eps_v));
 #pragma unroll
     for (int j = 0; j < kEPT; ++j) {
         float pj, g_plain, m_new, v_new, p_est, err;
         prepare<L2>(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
-        estimate(pj, m_new, v_new, k, p_est, err);
+        estimate(pj, m_new, v_new, k, eps_v, p_est, err);
         const float lo = (p_est - err) * ws, hi = (p_est + err) * ws;
         bool same;
         uint32_t code;
@@ -453,22 +457,26 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
 //
 // One lane's 16 elements: as write_step, plus the maxima.  |m'| and |v'| are exact.  For |p'| the estimate gives
 // |p_est| - err <= |p'| <= |p_est| + err; only elements whose upper end reaches the best lower end seen so far are
-// evaluated exactly, and the element that attains the maximum always is.
-template <int WDT, bool L2>
-__device__ __forceinline__ void spec_step(void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i, float* p, const float* g,
+// evaluated exactly, and the element that attains the maximum always is.  Elements that took the exact chain for
+// their code (an estimate too close to a rounding boundary, anything non-finite) have their exact |p'| already.
+template <int WDT, int GDT, bool L2>
+__device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i,
+                                          float* p, const float* g,
                                           float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
                                           float ms, float vs, const AdamConsts& k, float& floor_p, uint32_t& mxp,
                                           float& mxm, float& mxv) {
     uint32_t wq[kEPT];
-    float hi[kEPT], mm[kEPT], vv[kEPT];
-    float lo_max = 0.0f;
+    float hi[kEPT];
+    float lo_max = 0.0f, hi_max = 0.0f;
+    float eps_v = k.eps;
+    asm volatile("" : "+v"(eps_v));
 #pragma unroll
     for (int j = 0; j < kEPT; ++j) {
         float pj, g_plain, m_new, v_new, p_est, err;
         prepare<L2>(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
         mxm = fmaxf(mxm, fabsf(m_new));
         mxv = fmaxf(mxv, fabsf(v_new));
-        estimate(pj, m_new, v_new, k, p_est, err);
+        estimate(pj, m_new, v_new, k, eps_v, p_est, err);
         const float lo = (p_est - err) * ws, up = (p_est + err) * ws;
         bool same;
         uint32_t code;
@@ -480,11 +488,24 @@ __device__ __forceinline__ void spec_step(void* w_out, uint8_t* m_out, uint16_t*
             code = two & 0xffu;
             same = code == ((two >> 8) & 0xffu);
         }
-        if (!(same && err < __uint_as_float(0x7f800000u))) code = quant_weight_exact<WDT>(pj, m_new, v_new, ws, k);
+        float a_hi = fabsf(p_est) + err, a_lo = fabsf(p_est) - err;    // both finite whenever err is
+        if (!(same && err < __uint_as_float(0x7f800000u))) {
+            // the exact chain: its |p'| goes straight into the maximum, and the element leaves the bounds
+            const float pe = param_update(pj, m_new, v_new, k);
+            const uint32_t ab = __float_as_uint(pe) & 0x7fffffffu;
+            mxp = ab > mxp ? ab : mxp;
+            const float scaled = pe * ws;
+            if constexpr (WDT == MSAMP_DT_F16) {
+                code = float_to_f16_bits(scaled);
+            } else {
+                code = quant1<WDT>(scaled);
+            }
+            a_hi = 0.0f, a_lo = 0.0f;
+        }
         wq[j] = code;
-        hi[j] = fabsf(p_est) + err;                       // NaN for anything non-finite: evaluated exactly below
-        lo_max = fmaxf(lo_max, fabsf(p_est) - err);       // fmaxf skips a NaN
-        p[j] = pj, mm[j] = m_new, vv[j] = v_new;
+        hi[j] = a_hi;
+        hi_max = fmaxf(hi_max, a_hi);
+        lo_max = fmaxf(lo_max, a_lo);
         if constexpr (L2) moments(m[j], v[j], g_plain, inv_m, inv_v, k, m_new, v_new);    // stored moments ignore the L2 term
         m[j] = m_new * ms;
         v[j] = v_new * vs;
@@ -505,11 +526,18 @@ __device__ __forceinline__ void spec_step(void* w_out, uint8_t* m_out, uint16_t*
     store_w16<MSAMP_DT_F16>(v_out, i, v);
     floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
     const float skip_below = floor_p * 0.999999f;    // room for the roundings of the bounds themselves
+    if (hi_max >= skip_below) {    // few lanes get here: the ones that hold an element next to the maximum
 #pragma unroll
-    for (int j = 0; j < kEPT; ++j) {
-        if (!(hi[j] < skip_below)) {
-            const uint32_t ab = __float_as_uint(param_update(p[j], mm[j], vv[j], k)) & 0x7fffffffu;
-            mxp = ab > mxp ? ab : mxp;
+        for (int j = 0; j < kEPT; ++j) {
+            if (hi[j] >= skip_below) {
+                // the inputs are still in memory (this pass writes elsewhere): fetching the element again costs less
+                // than keeping 48 more values per lane alive for the few that come here
+                float pj, g_plain, m_new, v_new;
+                prepare<L2>(load_w1<WDT>(d.weight, i + j), load_w1<GDT>(d.grad, i + j), load_w1<MSAMP_DT_E4M3>(d.exp_avg, i + j),
+                            load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i + j), w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+                const uint32_t ab = __float_as_uint(param_update(pj, m_new, v_new, k)) & 0x7fffffffu;
+                mxp = ab > mxp ? ab : mxp;
+            }
         }
     }
 }
@@ -539,7 +567,7 @@ __global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_te
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            spec_step<WDT, L2>(w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p, mxp,
+            spec_step<WDT, GDT, L2>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p, mxp,
                                mxm, mxv);
         }
     } else {
