@@ -343,8 +343,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         // Written as assembly so that the compiler does not see an LDS write it cannot tell apart from
         // the fragment reads: it would otherwise make every LDS read wait for all loads in flight.
         // Completion is tracked by hand with wait_vmcnt<>() before the barriers below.  M0 holds the
-        // wave's LDS destination.
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src + off) : "memory", "m0");
+        // wave's LDS destination.  The address is a scalar base (operand + slice) plus the lane's 32-bit
+        // offset, so no vector instruction is spent on it.
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(off), "s"(src) : "memory", "m0");
     };
 
     // ---- LDS -> fragments of the 16x16x128 MFMA: a lane holds, for row lane % 16 of a 16-row block, the 32 K-bytes
@@ -734,7 +735,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const v4f a = acc[2 * u + h][j];
-                uint8_t* dst = patch + (h * 16 + l16) * kPitch + (j * 16 + g4 * 4) * kEsz;
+                // 8-byte writes of 16 rows at a time: rows r and r + 8 are 8 * (pitch mod 128 bytes) = 128 bytes apart in
+                // bank terms, the same 8-byte slot; the upper eight rows swap each pair of slots (undone when read back)
+                uint8_t* dst = patch + (h * 16 + l16) * kPitch + (((j * 16 + g4 * 4) * kEsz) ^ (kEsz == 2 ? ((l16 >> 3) & 1) << 3 : 0));
                 const float v0 = a[0] * alpha, v1 = a[1] * alpha, v2 = a[2] * alpha, v3 = a[3] * alpha;
                 if constexpr (kEsz == 4) {
                     *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
@@ -753,7 +756,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
             // eight reads in flight together, then the eight stores (named values: an array here ends up in scratch)
             auto rd = [&](int t) {
                 const int pr = (p0 + t) * kRowsPerPass + lane / kChunksPerRow;
-                return *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
+                const uint4 v = *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
+                const bool swapped = kEsz == 2 && (((p0 + t) * kRowsPerPass) >> 3) & 1;    // the same for all lanes of a pass
+                return swapped ? make_uint4(v.z, v.w, v.x, v.y) : v;
             };
             const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3), val4 = rd(4), val5 = rd(5), val6 = rd(6),
                         val7 = rd(7);
