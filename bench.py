@@ -361,8 +361,8 @@ def bench_cast(iters=20):
 
 def bench_grad_side(iters=10):
     """The reducer's compute steps on one bucket of 32 bf16 gradients of [4096,1024] (amax, scales, quantize
-    into the flat E4M3 buffer: 2 B read twice + 1 B written per element), and the per-tensor 2-norms of 64
-    such FP8 gradients (1 B read per element)."""
+    into the flat E4M3 buffer: 2 B read + 1 B written per element when the scales of the round before hold, the
+    input read a second time otherwise), and the per-tensor 2-norms of 64 such FP8 gradients (1 B read per element)."""
     import torch
     from msamp import _backend
     from msamp.nn import GradientBucket
@@ -372,6 +372,10 @@ def bench_grad_side(iters=10):
     out = {}
     ms = _time_gpu(lambda: bucket.quantize(grads, world_size=8), iters)
     out['bucket_quantize_32x4M_bf16'] = {'ms': ms, 'GBps': n * len(grads) * 3 / ms / 1e6}
+    # beside it: without the codes going out during the amax pass (input read twice)
+    bucket = GradientBucket([n] * len(grads), speculate=False)
+    ms = _time_gpu(lambda: bucket.quantize(grads, world_size=8), iters)
+    out['bucket_quantize_32x4M_bf16_two_reads'] = {'ms': ms, 'GBps': n * len(grads) * 3 / ms / 1e6}
     del grads, bucket
     qs = [torch.randint(0, 120, (n,), dtype=torch.uint8, device='cuda') for _ in range(64)]
     sis = [torch.ones((), device='cuda') for _ in qs]
@@ -570,7 +574,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--skip-cpu', action='store_true', help='leave out the CPU-oracle baseline')
     ap.add_argument('--skip-extra', action='store_true', help='leave out the sweep, cast and Adam kernel sections')
-    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'cast', 'adam'), default=None,
+    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'cast', 'adam', 'grad_side'), default=None,
                     help='run one kernel section alone (after the calibration copy), for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -592,6 +596,8 @@ def main():
             out = bench_gemm_sweep(LLAMA_70B, iters=3)
         elif args.only == 'cast':
             out = _round_kernels(bench_cast())
+        elif args.only == 'grad_side':
+            out = _round_kernels(bench_grad_side())
         else:
             out = bench_adam()
         print(json.dumps({'only': args.only, 'result': out}))

@@ -206,7 +206,7 @@ typedef struct msamp_bucket_item {
     float* scale_inv;    /* meta.scale_inv: rewritten                                           */
     uint64_t numel;
     uint32_t acc;        /* scratch                                                             */
-    uint32_t reserved;
+    uint32_t reserved;   /* scratch (zero it once with acc)                                     */
 } msamp_bucket_item;
 
 /* amax[0] = max|src| per item, NaN propagating (distributed.py:156: g.abs().max()); with
@@ -214,6 +214,16 @@ typedef struct msamp_bucket_item {
  * follows ignores NaN). */
 int msamp_bucket_amax(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype,
                       int flags, msamp_stream_t stream);
+
+/* msamp_bucket_amax that also writes, into each item's dst, the FP8 codes of src times the scale the item has NOW (no
+ * counterpart in the reference, which quantizes after the scales are known: distributed.py:163-185).  After a round
+ * of msamp_bucket_cast that scale is rule(amax) * pre_scale of that round, a power of two times a constant that
+ * seldom changes from one round to the next.  msamp_bucket_cast compares the scale it arrives at with the one the
+ * codes were written with and leaves the items where the two agree alone: the bucket is then read once instead of
+ * twice (3 instead of 5 bytes per bf16 element), with the same bytes in the buffer either way.  The codes of an item
+ * are final only after msamp_bucket_cast.  fp8_type must be the one msamp_bucket_cast is then called with. */
+int msamp_bucket_amax_speculative(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks,
+                                  int in_dtype, int fp8_type, int flags, msamp_stream_t stream);
 
 /* scale = rule(amax[0], fallback scale, fp_max, margin) * pre_scale (distributed.py:163-170, pre_scale =
  * 1/sqrt(world size)), dst = FP8 codes of src * scale (distributed.py:179-185), scale_inv = (1/scale) /

@@ -9,7 +9,10 @@ namespace msamp {
 constexpr int kBucketThreads = 256;
 
 // max |x| of one chunk, as the bit pattern of the float (a NaN pattern compares above every number, so it wins)
-template <typename IT>
+// FMT != 0: the chunk is also quantized, with the scale the item has now, into its place in the flat buffer.  That
+// scale is what the previous round's msamp_bucket_cast left there, and it is a power of two times a constant, so it is
+// as a rule the scale this round will arrive at; msamp_bucket_cast then finds its work done (see bucket_scale_kernel).
+template <typename IT, int FMT>
 __global__ __launch_bounds__(kBucketThreads) void bucket_amax_kernel(msamp_bucket_item* __restrict__ items,
                                                                      const int32_t* __restrict__ block_map) {
     constexpr int EPT = In16<IT>::EPT;
@@ -20,21 +23,39 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_amax_kernel(msamp_bucke
     const IT* x = static_cast<const IT*>(d.src);
     const size_t n = d.numel, base = static_cast<size_t>(chunk) * MSAMP_BUCKET_CHUNK;
     uint32_t m = 0;
-    if (base + MSAMP_BUCKET_CHUNK <= n && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    uint8_t* out = d.dst;
+    const float s = FMT != 0 ? *d.scale : 1.0f;
+    const bool vec_out = FMT == 0 || (reinterpret_cast<uintptr_t>(out) & (EPT - 1)) == 0;
+    if (base + MSAMP_BUCKET_CHUNK <= n && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && vec_out) {
         float v[kVecs][EPT];
 #pragma unroll
         for (int u = 0; u < kVecs; ++u) In16<IT>::load(x + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT, v[u]);
 #pragma unroll
-        for (int u = 0; u < kVecs; ++u)
+        for (int u = 0; u < kVecs; ++u) {
 #pragma unroll
             for (int j = 0; j < EPT; ++j) {
                 const uint32_t a = __float_as_uint(v[u][j]) & 0x7fffffffu;
                 m = a > m ? a : m;
             }
+            if constexpr (FMT != 0) {
+                uint32_t w[EPT / 4];
+#pragma unroll
+                for (int j = 0; j < EPT / 4; ++j)
+                    w[j] = quant4<FMT>(v[u][4 * j] * s, v[u][4 * j + 1] * s, v[u][4 * j + 2] * s, v[u][4 * j + 3] * s);
+                uint8_t* o = out + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT;
+                if constexpr (EPT == 4) {
+                    *reinterpret_cast<uint32_t*>(o) = w[0];
+                } else {
+                    *reinterpret_cast<uint2*>(o) = make_uint2(w[0], w[1]);
+                }
+            }
+        }
     } else {
         for (size_t i = base + threadIdx.x; i < n && i < base + MSAMP_BUCKET_CHUNK; i += kBucketThreads) {
-            const uint32_t a = __float_as_uint(Elem<IT>::load(x + i)) & 0x7fffffffu;
+            const float xi = Elem<IT>::load(x + i);
+            const uint32_t a = __float_as_uint(xi) & 0x7fffffffu;
             m = a > m ? a : m;
+            if constexpr (FMT != 0) out[i] = static_cast<uint8_t>(quant1<FMT>(xi * s));
         }
     }
     m = block_max_u32(m, red);
@@ -43,12 +64,17 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_amax_kernel(msamp_bucke
 
 // amax[0] of every tensor from the accumulated pattern (NaN and +Inf become +Inf when asked: the all-reduce that
 // follows in the reducer ignores NaN); the accumulator goes back to zero
-__global__ void bucket_amax_finish_kernel(msamp_bucket_item* items, int n_items, int flags) {
+constexpr uint32_t kBucketDone = 0xffffffffu;    // item.reserved: the buffer already holds this round's codes
+
+__global__ void bucket_amax_finish_kernel(msamp_bucket_item* items, int n_items, int flags, int speculative) {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n_items) return;
     msamp_bucket_item& d = items[t];
     float a = __uint_as_float(d.acc);
     d.acc = 0u;
+    // the scale the codes were written with, if they were (a positive finite one: anything else is no guess)
+    const float guess = *d.scale;
+    d.reserved = (speculative && guess > 0.0f && guess < __uint_as_float(0x7f800000u)) ? __float_as_uint(guess) : 0u;
     if ((flags & MSAMP_FLAG_NAN_TO_INF) && !(a < __uint_as_float(0x7f800000u))) a = __uint_as_float(0x7f800000u);
     *d.amax = a;
 }
@@ -61,6 +87,8 @@ __global__ void bucket_scale_kernel(msamp_bucket_item* items, int n_items, float
     if (t >= n_items) return;
     msamp_bucket_item& d = items[t];
     const float sf = scale_rule(*d.amax, *d.scale, fp_max, margin) * pre_scale;
+    // after msamp_bucket_amax_speculative: did the codes go out with this very scale?
+    if (d.reserved != 0u) d.reserved = (__float_as_uint(sf) == d.reserved) ? kBucketDone : 0u;
     *d.scale = sf;
     const float inv = 1.0f / sf;
     *d.scale_inv = inv / inv_div;
@@ -73,6 +101,7 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp
     constexpr int kVecs = MSAMP_BUCKET_CHUNK / (kBucketThreads * EPT);
     const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
     const msamp_bucket_item& d = items[t];
+    if (d.reserved == kBucketDone) return;    // written by the speculative first pass with the scale that came out
     const IT* x = static_cast<const IT*>(d.src);
     uint8_t* out = d.dst;
     const float s = *d.scale;
@@ -100,6 +129,11 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp
         for (size_t i = base + threadIdx.x; i < n && i < base + MSAMP_BUCKET_CHUNK; i += kBucketThreads)
             out[i] = static_cast<uint8_t>(quant1<FMT>(Elem<IT>::load(x + i) * s));
     }
+}
+
+__global__ void bucket_forget_kernel(msamp_bucket_item* items, int n_items) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n_items) items[t].reserved = 0u;
 }
 
 // ---- norms of FP8 gradients (clip_grad_norm_) ----------------------------------------------------------------
@@ -200,23 +234,43 @@ using namespace msamp;
 
 extern "C" {
 
-int msamp_bucket_amax(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype, int flags,
-                      msamp_stream_t stream) {
-    const int rc = check_bucket_args("msamp_bucket_amax", items, n_items, block_map, n_blocks, in_dtype);
+static int bucket_amax_launch(const char* who, msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks,
+                              int in_dtype, int fp8_type, int flags, msamp_stream_t stream) {
+    const int rc = check_bucket_args(who, items, n_items, block_map, n_blocks, in_dtype);
     if (rc != MSAMP_OK || n_items == 0) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (n_blocks > 0) {
-        if (in_dtype == MSAMP_DT_F32)
-            hipLaunchKernelGGL(bucket_amax_kernel<float>, dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map);
-        else if (in_dtype == MSAMP_DT_F16)
-            hipLaunchKernelGGL(bucket_amax_kernel<f16_t>, dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map);
-        else
-            hipLaunchKernelGGL(bucket_amax_kernel<bf16_t>, dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map);
+#define BUCKET_AMAX(IT)                                                                                                 \
+    do {                                                                                                              \
+        if (fp8_type == MSAMP_DT_E4M3)                                                                                \
+            hipLaunchKernelGGL((bucket_amax_kernel<IT, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+        else if (fp8_type == MSAMP_DT_E5M2)                                                                           \
+            hipLaunchKernelGGL((bucket_amax_kernel<IT, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+        else                                                                                                          \
+            hipLaunchKernelGGL((bucket_amax_kernel<IT, 0>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+    } while (0)
+        if (in_dtype == MSAMP_DT_F32) BUCKET_AMAX(float);
+        else if (in_dtype == MSAMP_DT_F16) BUCKET_AMAX(f16_t);
+        else BUCKET_AMAX(bf16_t);
+#undef BUCKET_AMAX
         MSAMP_CHECK_LAUNCH("bucket_amax_kernel");
     }
-    hipLaunchKernelGGL(bucket_amax_finish_kernel, dim3((n_items + 63) / 64), dim3(64), 0, st, items, n_items, flags);
+    hipLaunchKernelGGL(bucket_amax_finish_kernel, dim3((n_items + 63) / 64), dim3(64), 0, st, items, n_items, flags,
+                       fp8_type != 0 ? 1 : 0);
     MSAMP_CHECK_LAUNCH("bucket_amax_finish_kernel");
     return MSAMP_OK;
+}
+
+int msamp_bucket_amax(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype, int flags,
+                      msamp_stream_t stream) {
+    return bucket_amax_launch("msamp_bucket_amax", items, n_items, block_map, n_blocks, in_dtype, 0, flags, stream);
+}
+
+int msamp_bucket_amax_speculative(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype,
+                                  int fp8_type, int flags, msamp_stream_t stream) {
+    MSAMP_REQUIRE(is_fp8(fp8_type), MSAMP_ERR_DTYPE, "msamp_bucket_amax_speculative: fp8_type %d", fp8_type);
+    return bucket_amax_launch("msamp_bucket_amax_speculative", items, n_items, block_map, n_blocks, in_dtype, fp8_type, flags,
+                              stream);
 }
 
 int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* block_map, int n_blocks, int in_dtype,
@@ -242,6 +296,8 @@ int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* bloc
     else BUCKET_CAST(bf16_t);
 #undef BUCKET_CAST
     MSAMP_CHECK_LAUNCH("bucket_cast_kernel");
+    hipLaunchKernelGGL(bucket_forget_kernel, dim3((n_items + 63) / 64), dim3(64), 0, st, items, n_items);
+    MSAMP_CHECK_LAUNCH("bucket_forget_kernel");
     return MSAMP_OK;
 }
 

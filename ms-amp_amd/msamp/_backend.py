@@ -54,6 +54,7 @@ _SIGNATURES = {
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
     'msamp_fp8_norms': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
     'msamp_bucket_amax': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
+    'msamp_bucket_amax_speculative': ([_vp, _i, _vp, _i, _i, _i, _i, _vp], _i),
     'msamp_bucket_cast': ([_vp, _i, _vp, _i, _i, _i, _f, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
@@ -542,13 +543,21 @@ def bucket_tables(srcs, dsts, amaxs, scales, scale_invs):
     return items, chunk_map([s.numel() for s in srcs], device)
 
 
-def bucket_amax(items, block_map, in_dt, nan_to_inf=True):
-    """amax[0] of every item of the table."""
+def bucket_amax(items, block_map, in_dt, nan_to_inf=True, speculate_fp8_dt=None):
+    """amax[0] of every item of the table.  With speculate_fp8_dt the pass also writes every item's codes with the
+    scale the item has now; bucket_cast then redoes only the items whose scale came out different."""
     lib = load()
     _gpu(items, 'descriptor table')
+    flags = FLAG_NAN_TO_INF if nan_to_inf else 0
+    if speculate_fp8_dt is not None:
+        _check(
+            lib.msamp_bucket_amax_speculative(_ptr(items), items.shape[0], _ptr(block_map), block_map.shape[0], in_dt,
+                                              speculate_fp8_dt, flags, _stream()), 'msamp_bucket_amax_speculative'
+        )
+        return
     _check(
-        lib.msamp_bucket_amax(_ptr(items), items.shape[0], _ptr(block_map), block_map.shape[0], in_dt,
-                              FLAG_NAN_TO_INF if nan_to_inf else 0, _stream()), 'msamp_bucket_amax'
+        lib.msamp_bucket_amax(_ptr(items), items.shape[0], _ptr(block_map), block_map.shape[0], in_dt, flags, _stream()),
+        'msamp_bucket_amax'
     )
 
 

@@ -22,9 +22,10 @@ class GradientBucket:
     its own meta, already divided by the world size the way the reducer leaves it (distributed.py:192),
     so that a SUM all-reduce of `flat` (times the dequantization) yields the average.
     """
-    def __init__(self, numels, device='cuda', qtype=Dtypes.kfloat8_e4m3):
+    def __init__(self, numels, device='cuda', qtype=Dtypes.kfloat8_e4m3, speculate=True):
         if not Dtypes.is_fp8_qtype(qtype):
             raise TypeError('the bucket holds FP8 gradients')
+        self.speculate = speculate    # write the codes during the amax pass, with the scales of the round before
         self.numels = [int(n) for n in numels]
         self.qtype = qtype
         self.flat = torch.zeros(sum(self.numels), dtype=torch.uint8, device=device)
@@ -58,7 +59,10 @@ class GradientBucket:
             raise ValueError('gradients must be contiguous CUDA tensors of one dtype')
         items, block_map = self._get_tables(grads)
         in_dt = _backend._dt(grads[0])
-        _backend.bucket_amax(items, block_map, in_dt, nan_to_inf=True)
+        # The amax pass already writes the codes, with the scales of the round before; the second call then only redoes
+        # the gradients whose scale came out different (same bytes either way).
+        _backend.bucket_amax(items, block_map, in_dt, nan_to_inf=True,
+                             speculate_fp8_dt=int(self.qtype) if self.speculate else None)
         if reduce_amax is not None:
             reduce_amax([m.amax[0:1] for m in self.metas])
         # the division of each finished tensor by the world size (a division of its scale_inv) rides along

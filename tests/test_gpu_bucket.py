@@ -89,6 +89,64 @@ def test_bucket_reuse_and_argument_checks():
     assert GradientBucket([]).quantize([]) == []
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_bucket_speculative_rounds_equal_plain_rounds(dtype):
+    """Five rounds on one bucket, each taken with and without speculation from the same state: same buffer and metas
+    every time.  Round 1 finds scale 1 in the metas (every guess wrong); round 2 has gradients of the same size, so the
+    amax pass alone already leaves the final bytes; in round 3 half of the gradients are 64 times larger (those are
+    done again); round 4 has a NaN in one gradient; round 5 is back to normal."""
+    from msamp import _backend
+    from msamp.nn import GradientBucket
+    sizes = [5, 16384, 3, 16384 * 2 + 777, 1, 4096 * 33, 100, 16384 * 4]
+    world = 2
+    plain, spec = GradientBucket(sizes, speculate=False), GradientBucket(sizes, speculate=True)
+    base = _grads(77, sizes, dtype)
+    for rnd in range(1, 6):
+        noise = torch.Generator().manual_seed(100 + rnd)
+        grads = [(g.float() * (1 + 0.01 * torch.randn(g.shape, generator=noise))).to(dtype) for g in base]
+        if rnd == 3:
+            grads = [g * 64 if i % 2 == 0 else g for i, g in enumerate(grads)]
+        if rnd == 4:
+            grads[3][12345] = float('nan')
+        dev = [g.cuda() for g in grads]
+        before = [m.scale.clone() for m in spec.metas]
+        # what the speculative first pass alone leaves in the buffer
+        items, block_map = spec._get_tables(dev)
+        _backend.bucket_amax(items, block_map, _backend._dt(dev[0]), nan_to_inf=True, speculate_fp8_dt=int(spec.qtype))
+        early = spec.flat.clone()
+        _backend.bucket_cast(items, block_map, _backend._dt(dev[0]), int(spec.qtype), 1.0 / math.sqrt(world), float(world))
+        out_p = plain.quantize(dev, world_size=world)
+        assert torch.equal(spec.flat, plain.flat), rnd
+        for a, b in zip(spec.metas, plain.metas):
+            assert same_float(a.scale, b.scale) and same_float(a.scale_inv, b.scale_inv) and same_float(a.amax[0], b.amax[0])
+        kept = [same_float(m.scale, s) for m, s in zip(spec.metas, before)]
+        for view_offset, n, k in zip(_offsets(sizes), sizes, kept):
+            same_early = torch.equal(early[view_offset:view_offset + n], spec.flat[view_offset:view_offset + n])
+            assert same_early or not k, rnd    # a kept scale means the first pass already wrote the final bytes
+        if rnd == 1:
+            assert not any(kept)
+        if rnd in (2, 5):
+            assert sum(kept) >= len(sizes) - 2 and torch.equal(early, spec.flat) == all(kept)
+        if rnd == 3:
+            assert not any(kept[0::2])
+        _check(plain, out_p, [g.flatten() for g in grads], world, scales=[float(s) for s in before])
+    # and through the class, speculation on by default
+    a, b = GradientBucket(sizes), GradientBucket(sizes, speculate=False)
+    for seed in (1, 1, 2):
+        dev = [g.cuda() for g in _grads(seed, sizes, dtype)]
+        a.quantize(dev, world_size=4)
+        b.quantize(dev, world_size=4)
+        assert torch.equal(a.flat, b.flat)
+
+
+def _offsets(sizes):
+    out, o = [], 0
+    for n in sizes:
+        out.append(o)
+        o += n
+    return out
+
+
 def test_bucket_sum_of_ranks_is_the_average():
     """What the pre-scale and the division are for: with `world` ranks holding the same gradient, adding the ranks'
     dequantized buckets (what the SUM all-reduce of the payloads amounts to) gives the gradient back to FP8
