@@ -234,6 +234,15 @@ __device__ __noinline__ void store_quad_slow(OT* D, int row, int col, int NR, in
 }
 
 
+// 16 bytes of output, stored past the caches (non-temporal).  A round of tiles writes 128 KiB per CU, 4 MiB per XCD: as
+// ordinary stores that is the whole L2, and the operand panels that the next tiles are about to read get evicted for
+// data nobody reads again soon.  Measured on the Llama-7B shapes: 3 to 9 % off the whole GEMM.
+__device__ __forceinline__ void store_out16(void* p, const uint4& v) {
+    typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+    const v4u_t vv = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(vv, static_cast<v4u_t*>(p));
+}
+
 // ---------------------------------------------------------------------------------------------
 // Main kernel: 256 x 256 output tile over 128-byte K slices, four wavefronts each owning a 128 x 128
 // quadrant (8 x 8 accumulators of the 16x16x128 FP8 MFMA = 256 accumulation registers per lane).
@@ -621,7 +630,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 auto st = [&](int t, const uint4& v) {
                     const int grow = row0 + wr * 128 + u * 32 + t * 8 + (lane >> 3);
                     const int gcol = col0 + wc * 128 + (lane & 7) * 16;
-                    *reinterpret_cast<uint4*>(qa.q + static_cast<size_t>(grow) * NC + gcol) = v;
+                    store_out16(qa.q + static_cast<size_t>(grow) * NC + gcol, v);
                 };
                 st(0, val0), st(1, val1), st(2, val2), st(3, val3);
             });
@@ -710,7 +719,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     } else {
                         v = make_uint4(pack_f16(r[0], r[1]), pack_f16(r[2], r[3]), pack_f16(r[4], r[5]), pack_f16(r[6], r[7]));
                     }
-                    if (ok[t]) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
+                    if (ok[t]) store_out16(D + static_cast<size_t>(grow) * NC + gcol, v);
                 }
             });
         });
@@ -767,7 +776,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 const int pc = lane % kChunksPerRow;
                 const int grow = row0 + wr * 128 + u * 32 + pr;
                 const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
-                if (grow < NR && gcol < NC) *reinterpret_cast<uint4*>(D + static_cast<size_t>(grow) * NC + gcol) = v;
+                if (grow < NR && gcol < NC) store_out16(D + static_cast<size_t>(grow) * NC + gcol, v);
             };
             st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
         });
