@@ -243,6 +243,13 @@ __device__ __forceinline__ void store_out16(void* p, const uint4& v) {
     __builtin_nontemporal_store(vv, static_cast<v4u_t*>(p));
 }
 
+// the old output of an accumulating GEMM is read once: past the caches as well
+__device__ __forceinline__ uint4 load_out16(const void* p) {
+    typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+    const v4u_t v = __builtin_nontemporal_load(static_cast<const v4u_t*>(p));
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Main kernel: 256 x 256 output tile over 128-byte K slices, four wavefronts each owning a 128 x 128
 // quadrant (8 x 8 accumulators of the 16x16x128 FP8 MFMA = 256 accumulation registers per lane).
@@ -686,7 +693,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     const int grow = row0 + wr * 128 + u * 32 + (p0 + t) * kRowsPerPass + prl;
                     ok[t] = col_ok && grow < NR;
                     old[t] = make_uint4(0, 0, 0, 0);
-                    if (accumulate && ok[t]) old[t] = *reinterpret_cast<const uint4*>(D + static_cast<size_t>(grow) * NC + gcol);
+                    if (accumulate && ok[t]) old[t] = load_out16(D + static_cast<size_t>(grow) * NC + gcol);
                 }
 #pragma unroll
                 for (int t = 0; t < kGroup; ++t) {
