@@ -306,6 +306,59 @@ __device__ __forceinline__ void round_pair(float a, float b, float& ra, float& r
     }
 }
 
+// ---- the accumulators of the DMA kernel live in fixed AGPRs: block (i, j) of the wave's 8 x 8 in a[4n .. 4n+3], n = i * 8 + j.
+// The register allocator never sees them.  Left to it, they are renumbered between the K loop, its straight-line tail
+// and the epilogue, which costs copies between the MFMAs or spills once all 256 are taken.
+#define MSAMP_A10(p) "a" #p "0", "a" #p "1", "a" #p "2", "a" #p "3", "a" #p "4", "a" #p "5", "a" #p "6", "a" #p "7", "a" #p "8", "a" #p "9"
+#define MSAMP_ALL_AGPRS                                                                                                \
+    "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", MSAMP_A10(1), MSAMP_A10(2), MSAMP_A10(3), MSAMP_A10(4),  \
+        MSAMP_A10(5), MSAMP_A10(6), MSAMP_A10(7), MSAMP_A10(8), MSAMP_A10(9), MSAMP_A10(10), MSAMP_A10(11), MSAMP_A10(12), \
+        MSAMP_A10(13), MSAMP_A10(14), MSAMP_A10(15), MSAMP_A10(16), MSAMP_A10(17), MSAMP_A10(18), MSAMP_A10(19),          \
+        MSAMP_A10(20), MSAMP_A10(21), MSAMP_A10(22), MSAMP_A10(23), MSAMP_A10(24), "a250", "a251", "a252", "a253", "a254", \
+        "a255"
+
+// a[4N .. 4N+3] += srcA x srcB.  No clobber list: the compiler follows a clobbered register with a wait state, one per
+// MFMA.  It learns of the AGPRs from acc_clear() and acc_fence(), which name them all.
+template <int N, int CB, int BL>
+__device__ __forceinline__ void mfma_fixed(const v8i& a, const v8i& b) {
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 a[%2:%3], %0, %1, a[%2:%3] cbsz:%4 blgp:%5"
+                 :
+                 : "v"(a), "v"(b), "n"(N * 4), "n"(N * 4 + 3), "n"(CB), "n"(BL));
+}
+__device__ __forceinline__ void acc_clear() {
+    static_for<64>([&](auto nc) {
+        constexpr int n = decltype(nc)::value;
+        asm volatile("v_accvgpr_write_b32 a[%0], 0\n\tv_accvgpr_write_b32 a[%1], 0\n\tv_accvgpr_write_b32 a[%2], 0\n\t"
+                     "v_accvgpr_write_b32 a[%3], 0"
+                     :
+                     : "n"(n * 4), "n"(n * 4 + 1), "n"(n * 4 + 2), "n"(n * 4 + 3));
+    });
+    asm volatile("s_nop 4" : : : MSAMP_ALL_AGPRS);
+}
+// After the last MFMA: waits out the MFMA pipe (a 16-pass MFMA's result may be read 18 wait states later) and hands out
+// the token that ties the reads below to this point of the program.
+__device__ __forceinline__ uint32_t acc_fence() {
+    uint32_t token;
+    asm volatile("s_nop 15\n\ts_nop 7\n\tv_mov_b32 %0, 0" : "=v"(token) : : MSAMP_ALL_AGPRS);
+    return token;
+}
+__device__ __forceinline__ uint32_t acc_refence(uint32_t token) {
+    asm volatile("" : "+v"(token));
+    return token;
+}
+// Not volatile: the compiler may place the read where it likes after the fence that made the token.
+template <int N>
+__device__ __forceinline__ v4f acc_quad(uint32_t token) {
+    v4f r;
+    float x, y, z, w;
+    asm("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(N * 4), "v"(token));
+    asm("v_accvgpr_read_b32 %0, a[%1]" : "=v"(y) : "n"(N * 4 + 1), "v"(token));
+    asm("v_accvgpr_read_b32 %0, a[%1]" : "=v"(z) : "n"(N * 4 + 2), "v"(token));
+    asm("v_accvgpr_read_b32 %0, a[%1]" : "=v"(w) : "n"(N * 4 + 3), "v"(token));
+    r[0] = x, r[1] = y, r[2] = z, r[3] = w;
+    return r;
+}
+
 template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0, bool ODD_NK = false>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
                                                                      const uint8_t* __restrict__ Y, OT* __restrict__ D,
@@ -398,14 +451,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         }
     };
 
-    typedef float v4f __attribute__((ext_vector_type(4)));
-    v4f acc[8][8];    // acc[i][j]: D rows i * 16 + lane % 16, D columns j * 16 + (lane / 16) * 4 .. + 3 of the quadrant
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+    // accumulator block (i, j): D rows i * 16 + lane % 16, D columns j * 16 + (lane / 16) * 4 .. + 3 of the quadrant
+    acc_clear();
 
     const int nk = K / kBK;
     int fx[2][32], fy[2][32];
@@ -415,22 +462,21 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // of slice ld_kt (ld_first .. ld_first + 7), one every other MFMA.
     // srcA = Y rows (columns of D), srcB = X rows (rows of D): a lane then holds, for D row lane % 16 of a block, four
     // consecutive D columns -- the layout the epilogue wants.
-    auto quarter = [&](int hx, int hy, int* rd_dst, int rd_stage, bool rd_x, int rd_half, bool do_read, int ld_kt,
+    auto quarter = [&](auto hxc, auto hyc, int* rd_dst, int rd_stage, bool rd_x, int rd_half, bool do_read, int ld_kt,
                        int ld_stage, int ld_first, bool do_load) __attribute__((always_inline)) {
         constexpr int cb = (YF == MSAMP_DT_E4M3) ? 0 : 1;
         constexpr int bl = (XF == MSAMP_DT_E4M3) ? 0 : 1;
         const int np = rd_x ? kPX : kPY;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {    // the Y fragment stays for four MFMAs in a row
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int n = j * 4 + i;
+        constexpr int hx = decltype(hxc)::value, hy = decltype(hyc)::value;
+        static_for<4>([&](auto jc) {    // the Y fragment stays for four MFMAs in a row
+            static_for<4>([&](auto ic) {
+                constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
+                constexpr int n = j * 4 + i;
                 const int* cx = fx[hx] + i * 8;
                 const int* cy = fy[hy] + j * 8;
                 const v8i vx = {cx[0], cx[1], cx[2], cx[3], cx[4], cx[5], cx[6], cx[7]};
                 const v8i vy = {cy[0], cy[1], cy[2], cy[3], cy[4], cy[5], cy[6], cy[7]};
-                acc[hx * 4 + i][hy * 4 + j] =
-                    __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(vy, vx, acc[hx * 4 + i][hy * 4 + j], cb, bl, 0, 0, 0, 0);
+                mfma_fixed<(hx * 4 + i) * 8 + hy * 4 + j, cb, bl>(vy, vx);
                 if (do_read) {
 #pragma unroll
                     for (int p = n * np / 16; p < (n + 1) * np / 16; ++p) read_piece(rd_dst, rd_stage, rd_x, rd_half, p);
@@ -440,8 +486,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 // scheduler stretches the fragments' live ranges until the register allocator no longer updates the 64
                 // accumulators in place and copies them around between the MFMAs.
                 __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+            });
+        });
     };
     // Slice kt sits in stage st and slice kt + 1 is on its way into the other stage; X half 0 and Y half 0 of slice
     // kt are in registers.  Quarters 1, 2: X0 x Y0 while Y half 1 arrives, X0 x Y1 while X half 1 arrives -- all of
@@ -449,12 +495,14 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // Quarters 3, 4: X1 x Y0 while X half 0 of slice kt + 1 arrives, X1 x Y1 while its Y half 0 arrives; the stage of
     // slice kt is refilled with slice kt + 2 meanwhile.
     auto slice = [&](int st, bool has_next, int ld_kt, bool do_load) __attribute__((always_inline)) {
-        quarter(0, 0, fy[1], st, false, 1, true, 0, 0, 0, false);
-        quarter(0, 1, fx[1], st, true, 1, true, 0, 0, 0, false);
+        constexpr std::integral_constant<int, 0> c0{};
+        constexpr std::integral_constant<int, 1> c1{};
+        quarter(c0, c0, fy[1], st, false, 1, true, 0, 0, 0, false);
+        quarter(c0, c1, fx[1], st, true, 1, true, 0, 0, 0, false);
         wait_vmcnt<0>();
         __syncthreads();
-        quarter(1, 0, fx[0], st ^ 1, true, 0, has_next, ld_kt, st, 0, do_load);
-        quarter(1, 1, fy[0], st ^ 1, false, 0, has_next, ld_kt, st, 8, do_load);
+        quarter(c1, c0, fx[0], st ^ 1, true, 0, has_next, ld_kt, st, 0, do_load);
+        quarter(c1, c1, fy[0], st ^ 1, false, 0, has_next, ld_kt, st, 8, do_load);
     };
 
     // prologue: slices 0 and 1 (the host sends no problem with fewer than two slices here); wait for slice 0; read
@@ -514,6 +562,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                          : "memory", "m0");
         }
     }
+    const uint32_t acc_token = acc_fence();
     // No barrier here: the last LDS reads of every wave were issued (and awaited) before the barrier of the last
     // slice, and no load is in flight, so each wave may start on its patch as soon as its own MFMAs are done.
 
@@ -527,12 +576,11 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         // max |acc| as an ordered bit pattern: NaN above Inf above everything finite, so a NaN reaches the amax
         // as it does through abs().max()
         uint32_t m = 0;
+        static_for<64>([&](auto nc) {
+            const v4f a = acc_quad<decltype(nc)::value>(acc_token);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) m = umax(m, __float_as_uint(acc[i][j][r]) & 0x7fffffffu);
+            for (int r = 0; r < 4; ++r) m = umax(m, __float_as_uint(a[r]) & 0x7fffffffu);
+        });
         m = block_max_u32(m, q_red);    // valid in lane 0 of wave 0
         const int tid = threadIdx.x;
         if (tid == 0) {
@@ -605,6 +653,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         }
         __syncthreads();    // also: every wave is through with the stages, which the patches below reuse
         const float sc = __uint_as_float(q_scale);
+        const uint32_t acc_token2 = acc_refence(acc_token);    // a second round of reads, not the first one kept alive
         // with a positive finite amax and the scale derived from it nothing leaves the format and nothing is NaN:
         // the clamp and the NaN patch of the general conversion can go
         const bool in_range = __uint_as_float(q_amax) * sc <= qa.fp_max && __uint_as_float(q_amax) > 0.0f;
@@ -616,10 +665,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 constexpr int u = decltype(uc)::value;
                 static_for<2>([&](auto hc) {
                     constexpr int h = decltype(hc)::value;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
+                    static_for<8>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
                         // the outputs as OT would hold them, then scaled
-                        const v4f a = acc[2 * u + h][j];
+                        const v4f a = acc_quad<(2 * u + h) * 8 + j>(acc_token2);
                         float r0, r1, r2, r3;
                         round_pair<OT>(a[0] * alpha, a[1] * alpha, r0, r1);
                         round_pair<OT>(a[2] * alpha, a[3] * alpha, r2, r3);
@@ -627,7 +676,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                         if constexpr (kChecked) w = quant4<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
                         else w = quant4_in_range<QF>(r0 * sc, r1 * sc, r2 * sc, r3 * sc);
                         *reinterpret_cast<uint32_t*>(qpatch + (h * 16 + l16) * kQPitch + j * 16 + g4 * 4) = w;
-                    }
+                    });
                 });
                 // the patch is private to this wave and the LDS serves one wave's requests in order: no waits here
                 auto rd = [&](int t) {
@@ -676,12 +725,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
             constexpr int u = decltype(uc)::value;
             static_for<2>([&](auto hc) {
                 constexpr int h = decltype(hc)::value;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const v4f a = acc[2 * u + h][j];
+                static_for<8>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    const v4f a = acc_quad<(2 * u + h) * 8 + j>(acc_token);
                     *reinterpret_cast<float4*>(fpatch + (h * 16 + l16) * kFPitch + (j * 16 + g4 * 4) * 4) =
                         make_float4(a[0], a[1], a[2], a[3]);
-                }
+                });
             });
             // the patch is private to this wave and the LDS serves one wave's requests in order: no waits needed
             static_for<kPasses / kGroup>([&](auto gc) {
@@ -735,12 +784,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     if (!plain) {
         static_for<8>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const v4f a = acc[i][j];
+            static_for<8>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const v4f a = acc_quad<i * 8 + j>(acc_token);
                 store_quad_slow<OT>(D, row0 + wr * 128 + i * 16 + l16, col0 + wc * 128 + j * 16 + g4 * 4, NR, NC, alpha, a[0], a[1],
                                     a[2], a[3], accumulate, bias, bias_dt);
-            }
+            });
         });
         return;
     }
@@ -748,9 +797,9 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         constexpr int u = decltype(uc)::value;
         static_for<2>([&](auto hc) {
             constexpr int h = decltype(hc)::value;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const v4f a = acc[2 * u + h][j];
+            static_for<8>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const v4f a = acc_quad<(2 * u + h) * 8 + j>(acc_token);
                 // 8-byte writes of 16 rows at a time: rows r and r + 8 are 8 * (pitch mod 128 bytes) = 128 bytes apart in
                 // bank terms, the same 8-byte slot; the upper eight rows swap each pair of slots (undone when read back)
                 uint8_t* dst = patch + (h * 16 + l16) * kPitch + (((j * 16 + g4 * 4) * kEsz) ^ (kEsz == 2 ? ((l16 >> 3) & 1) << 3 : 0));
@@ -762,7 +811,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 } else {
                     *reinterpret_cast<uint2*>(dst) = make_uint2(pack_f16(v0, v1), pack_f16(v2, v3));
                 }
-            }
+            });
         });
         // no wait between the writes above and the reads below, nor before the next unit's writes: the patch is
         // private to this wave and the LDS serves one wave's requests in order
