@@ -99,7 +99,10 @@ __device__ __forceinline__ void tile_of_id(int id, int tiles_r, int tiles_c, boo
     constexpr int kXcd = 8, kGroup = 8;
     const int n_a = by_columns ? tiles_c : tiles_r, n_b = by_columns ? tiles_r : tiles_c;    // a: grouped, b: walked
     const int nt = tiles_r * tiles_c;
-    if (nt % kXcd == 0) id = (id % kXcd) * (nt / kXcd) + id / kXcd;
+    // XCD x runs the workgroups x, x + 8, ...: they get the contiguous ids that start where those of XCDs 0 .. x-1 end
+    // (the first nt % 8 XCDs run one workgroup more than the others)
+    const int x = id % kXcd, extra = nt % kXcd;
+    id = x * (nt / kXcd) + (x < extra ? x : extra) + id / kXcd;
     const int per_group = kGroup * n_b;
     const int g = id / per_group;
     const int first_a = g * kGroup;
