@@ -728,7 +728,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     uint8_t* patch = smem + wave * (32 * kPitch);
     const float alpha = alpha_early;
     const bool vec_ok = (NC % (16 / kEsz) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
-    const bool plain = vec_ok && !accumulate && bias == nullptr;
+    const bool plain = !accumulate && bias == nullptr;    // (rows that 16-byte stores do not fit go out element by element)
+    const bool pairs_ok = (NC % 2 == 0) && ((reinterpret_cast<uintptr_t>(D) & 3) == 0);
     constexpr int kChunksPerRow = 128 * kEsz / 16;      // 16 (2-byte) or 32 (float)
     constexpr int kRowsPerPass = 64 / kChunksPerRow;    // 4 or 2
     constexpr int kElemsPerChunk = 16 / kEsz;           // 8 or 4
@@ -859,7 +860,23 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 const int pc = lane % kChunksPerRow;
                 const int grow = row0 + wr * 128 + u * 32 + pr;
                 const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
-                if (grow < NR && gcol < NC) store_out16(D + static_cast<size_t>(grow) * NC + gcol, v);
+                if (vec_ok) {
+                    if (grow < NR && gcol < NC) store_out16(D + static_cast<size_t>(grow) * NC + gcol, v);
+                } else if (grow < NR) {
+                    // an output whose rows are not 16-byte aligned, or end inside a segment: the lane's segment one element
+                    // at a time (still whole rows side by side: the 64 stores of a wave instruction touch few lines)
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                    OT* out = D + static_cast<size_t>(grow) * NC + gcol;
+                    if (kEsz == 4 || pairs_ok) {    // 4-byte stores: float32, or 2-byte elements in aligned pairs
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (gcol + e * (4 / kEsz) < NC) reinterpret_cast<uint32_t*>(out)[e] = w[e];
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < kElemsPerChunk; ++e)
+                            if (gcol + e < NC) reinterpret_cast<uint16_t*>(out)[e] = static_cast<uint16_t>(w[e >> 1] >> ((e & 1) * 16));
+                    }
+                }
             };
             st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
         });

@@ -96,7 +96,7 @@ def test_accumulate_and_bias(be, out_dtype):
     assert rel_fro(got.float(), want) < (TOL_F32 if out_dtype == torch.float32 else TOL_16)
 
 
-@pytest.mark.parametrize('m,n,k', [(4096, 2048, 256), (4100, 2056, 384), (3001, 2999, 128)])
+@pytest.mark.parametrize('m,n,k', [(4096, 2048, 256), (4100, 2056, 384), (3001, 2999, 128), (4101, 1031, 256)])
 @pytest.mark.parametrize('out_dtype', [torch.bfloat16, torch.float32, torch.float16])
 def test_large_tiles_ragged_edges_accumulate_bias(be, m, n, k, out_dtype):
     """Shapes big enough for the 256x256 direct-to-LDS kernel, with ragged right/bottom edges,
