@@ -821,66 +821,86 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         });
         return;
     }
-    static_for<4>([&](auto uc) {
-        constexpr int u = decltype(uc)::value;
-        static_for<2>([&](auto hc) {
-            constexpr int h = decltype(hc)::value;
-            static_for<8>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                const v4f a = acc_quad<(2 * u + h) * 8 + j>(acc_token);
-                // 8-byte writes of 16 rows at a time: rows r and r + 8 are 8 * (pitch mod 128 bytes) = 128 bytes apart in
-                // bank terms, the same 8-byte slot; the upper eight rows swap each pair of slots (undone when read back)
-                uint8_t* dst = patch + (h * 16 + l16) * kPitch + (((j * 16 + g4 * 4) * kEsz) ^ (kEsz == 2 ? ((l16 >> 3) & 1) << 3 : 0));
-                const float v0 = a[0] * alpha, v1 = a[1] * alpha, v2 = a[2] * alpha, v3 = a[3] * alpha;
-                if constexpr (kEsz == 4) {
-                    *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
-                } else if constexpr (__is_same(OT, bf16_t)) {
-                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(v0, v1), pack_bf16(v2, v3));
-                } else {
-                    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_f16(v0, v1), pack_f16(v2, v3));
-                }
+    // Three copies of the plain epilogue, chosen once per workgroup so that the one that runs is straight-line code:
+    // whole tile with 16-byte row stores (no bounds checks; the address is a scalar row base plus one per-lane offset),
+    // 16-byte row stores with bounds checks (tiles on the right or bottom edge), and rows that 16-byte stores do not fit.
+    // (With the choice made per store, every store dragged three variants and their branches along.)
+    auto emit_plain = [&](auto vec_c, auto inside_c) __attribute__((always_inline)) {
+        constexpr bool kVec = decltype(vec_c)::value, kInside = decltype(inside_c)::value;
+        const int pc = lane % kChunksPerRow, prl = lane / kChunksPerRow;
+        const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
+        // whole tile: byte offset of this lane's segment from the first element of its pass's first row
+        const uint32_t lane_off = (static_cast<uint32_t>(prl) * static_cast<uint32_t>(NC) + static_cast<uint32_t>(pc * kElemsPerChunk)) * kEsz;
+        static_for<4>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            static_for<2>([&](auto hc) {
+                constexpr int h = decltype(hc)::value;
+                static_for<8>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    const v4f a = acc_quad<(2 * u + h) * 8 + j>(acc_token);
+                    // 8-byte writes of 16 rows at a time: rows r and r + 8 are 8 * (pitch mod 128 bytes) = 128 bytes apart in
+                    // bank terms, the same 8-byte slot; the upper eight rows swap each pair of slots (undone when read back)
+                    uint8_t* dst = patch + (h * 16 + l16) * kPitch + (((j * 16 + g4 * 4) * kEsz) ^ (kEsz == 2 ? ((l16 >> 3) & 1) << 3 : 0));
+                    const float v0 = a[0] * alpha, v1 = a[1] * alpha, v2 = a[2] * alpha, v3 = a[3] * alpha;
+                    if constexpr (kEsz == 4) {
+                        *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
+                    } else if constexpr (__is_same(OT, bf16_t)) {
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(v0, v1), pack_bf16(v2, v3));
+                    } else {
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_f16(v0, v1), pack_f16(v2, v3));
+                    }
+                });
+            });
+            // no wait between the writes above and the reads below, nor before the next unit's writes: the patch is
+            // private to this wave and the LDS serves one wave's requests in order
+            constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
+            static_for<kPasses / 8>([&](auto gc) {
+                constexpr int p0 = decltype(gc)::value * 8;
+                // eight reads in flight together, then the eight stores (named values: an array here ends up in scratch)
+                auto rd = [&](int t) {
+                    const int pr = (p0 + t) * kRowsPerPass + prl;
+                    const uint4 v = *reinterpret_cast<const uint4*>(patch + pr * kPitch + pc * 16);
+                    const bool swapped = kEsz == 2 && (((p0 + t) * kRowsPerPass) >> 3) & 1;    // the same for all lanes of a pass
+                    return swapped ? make_uint4(v.z, v.w, v.x, v.y) : v;
+                };
+                const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3), val4 = rd(4), val5 = rd(5), val6 = rd(6),
+                            val7 = rd(7);
+                auto st = [&](int t, const uint4& v) {
+                    const int first_row = row0 + wr * 128 + u * 32 + (p0 + t) * kRowsPerPass;    // wave-uniform
+                    if constexpr (kVec && kInside) {
+                        uint8_t* row_base = reinterpret_cast<uint8_t*>(D + static_cast<size_t>(first_row) * NC + (col0 + wc * 128));
+                        store_out16(row_base + lane_off, v);
+                    } else if constexpr (kVec) {
+                        const int grow = first_row + prl;
+                        if (grow < NR && gcol < NC) store_out16(D + static_cast<size_t>(grow) * NC + gcol, v);
+                    } else {
+                        // an output whose rows are not 16-byte aligned, or end inside a segment: the lane's segment one
+                        // element at a time (still whole rows side by side: the 64 stores of a wave instruction touch few lines)
+                        const int grow = first_row + prl;
+                        if (grow < NR) {
+                            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                            OT* out = D + static_cast<size_t>(grow) * NC + gcol;
+                            if (kEsz == 4 || pairs_ok) {    // 4-byte stores: float32, or 2-byte elements in aligned pairs
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    if (gcol + e * (4 / kEsz) < NC) reinterpret_cast<uint32_t*>(out)[e] = w[e];
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < kElemsPerChunk; ++e)
+                                    if (gcol + e < NC) reinterpret_cast<uint16_t*>(out)[e] = static_cast<uint16_t>(w[e >> 1] >> ((e & 1) * 16));
+                            }
+                        }
+                    }
+                };
+                st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
             });
         });
-        // no wait between the writes above and the reads below, nor before the next unit's writes: the patch is
-        // private to this wave and the LDS serves one wave's requests in order
-        constexpr int kPasses = 32 / kRowsPerPass;    // 8 or 16
-        static_for<kPasses / 8>([&](auto gc) {
-            constexpr int p0 = decltype(gc)::value * 8;
-            // eight reads in flight together, then the eight stores (named values: an array here ends up in scratch)
-            auto rd = [&](int t) {
-                const int pr = (p0 + t) * kRowsPerPass + lane / kChunksPerRow;
-                const uint4 v = *reinterpret_cast<const uint4*>(patch + pr * kPitch + (lane % kChunksPerRow) * 16);
-                const bool swapped = kEsz == 2 && (((p0 + t) * kRowsPerPass) >> 3) & 1;    // the same for all lanes of a pass
-                return swapped ? make_uint4(v.z, v.w, v.x, v.y) : v;
-            };
-            const uint4 val0 = rd(0), val1 = rd(1), val2 = rd(2), val3 = rd(3), val4 = rd(4), val5 = rd(5), val6 = rd(6),
-                        val7 = rd(7);
-            auto st = [&](int t, const uint4& v) {
-                const int pr = (p0 + t) * kRowsPerPass + lane / kChunksPerRow;
-                const int pc = lane % kChunksPerRow;
-                const int grow = row0 + wr * 128 + u * 32 + pr;
-                const int gcol = col0 + wc * 128 + pc * kElemsPerChunk;
-                if (vec_ok) {
-                    if (grow < NR && gcol < NC) store_out16(D + static_cast<size_t>(grow) * NC + gcol, v);
-                } else if (grow < NR) {
-                    // an output whose rows are not 16-byte aligned, or end inside a segment: the lane's segment one element
-                    // at a time (still whole rows side by side: the 64 stores of a wave instruction touch few lines)
-                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-                    OT* out = D + static_cast<size_t>(grow) * NC + gcol;
-                    if (kEsz == 4 || pairs_ok) {    // 4-byte stores: float32, or 2-byte elements in aligned pairs
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (gcol + e * (4 / kEsz) < NC) reinterpret_cast<uint32_t*>(out)[e] = w[e];
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < kElemsPerChunk; ++e)
-                            if (gcol + e < NC) reinterpret_cast<uint16_t*>(out)[e] = static_cast<uint16_t>(w[e >> 1] >> ((e & 1) * 16));
-                    }
-                }
-            };
-            st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
-        });
-    });
+    };
+    const bool inside = row0 + kDmaTile <= NR && col0 + kDmaTile <= NC;
+    // (the per-lane offset of the whole-tile form is 32 bits: four rows of the output)
+    if (vec_ok && inside && static_cast<unsigned long long>(NC) * kEsz * 4 < (1ull << 31)) emit_plain(std::true_type{}, std::true_type{});
+    else if (vec_ok) emit_plain(std::true_type{}, std::false_type{});
+    else emit_plain(std::false_type{}, std::false_type{});
 }
 
 // The kernel is built once for an even and once for an odd number of K slices (its last slices are straight-line
