@@ -87,8 +87,9 @@ __global__ void bucket_scale_kernel(msamp_bucket_item* items, int n_items, float
     if (t >= n_items) return;
     msamp_bucket_item& d = items[t];
     const float sf = scale_rule(*d.amax, *d.scale, fp_max, margin) * pre_scale;
-    // after msamp_bucket_amax_speculative: did the codes go out with this very scale?
-    if (d.reserved != 0u) d.reserved = (__float_as_uint(sf) == d.reserved) ? kBucketDone : 0u;
+    // after msamp_bucket_amax_speculative: did the codes go out with this very scale?  (A mark left by an earlier cast
+    // of the same round is no guess: a second cast without a new amax pass writes the codes again.)
+    if (d.reserved != 0u) d.reserved = (d.reserved != kBucketDone && __float_as_uint(sf) == d.reserved) ? kBucketDone : 0u;
     *d.scale = sf;
     const float inv = 1.0f / sf;
     *d.scale_inv = inv / inv_div;
@@ -129,11 +130,6 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp
         for (size_t i = base + threadIdx.x; i < n && i < base + MSAMP_BUCKET_CHUNK; i += kBucketThreads)
             out[i] = static_cast<uint8_t>(quant1<FMT>(Elem<IT>::load(x + i) * s));
     }
-}
-
-__global__ void bucket_forget_kernel(msamp_bucket_item* items, int n_items) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t < n_items) items[t].reserved = 0u;
 }
 
 // ---- norms of FP8 gradients (clip_grad_norm_) ----------------------------------------------------------------
@@ -296,8 +292,6 @@ int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* bloc
     else BUCKET_CAST(bf16_t);
 #undef BUCKET_CAST
     MSAMP_CHECK_LAUNCH("bucket_cast_kernel");
-    hipLaunchKernelGGL(bucket_forget_kernel, dim3((n_items + 63) / 64), dim3(64), 0, st, items, n_items);
-    MSAMP_CHECK_LAUNCH("bucket_forget_kernel");
     return MSAMP_OK;
 }
 
