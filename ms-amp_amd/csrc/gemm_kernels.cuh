@@ -95,7 +95,7 @@ __device__ __forceinline__ float load_bias(const void* bias, int dt, int i) {
 // workgroup id -> tile, keeping the workgroups of one XCD on adjacent tiles and walking groups of `kGroup` tile rows
 // column by column (or, with `by_columns`, groups of tile columns row by row): the 32 CUs of an XCD then work on an
 // 8 x 4 patch of tiles and share its 12 operand panels through that L2.
-__device__ __forceinline__ void tile_of_id(int id, int tiles_r, int tiles_c, bool by_columns, int& tr, int& tc) {
+__device__ __forceinline__ void tile_of_id(int id, int tiles_r, int tiles_c, bool by_columns, bool wide, int& tr, int& tc) {
     constexpr int kXcd = 8, kGroup = 8;
     const int n_a = by_columns ? tiles_c : tiles_r, n_b = by_columns ? tiles_r : tiles_c;    // a: grouped, b: walked
     const int nt = tiles_r * tiles_c;
@@ -108,12 +108,20 @@ __device__ __forceinline__ void tile_of_id(int id, int tiles_r, int tiles_c, boo
     const int first_a = g * kGroup;
     const int here = (n_a - first_a) < kGroup ? (n_a - first_a) : kGroup;
     const int in_g = id - g * per_group;
-    const int a = first_a + in_g % here, b = in_g / here;
+    int a = first_a + in_g % here, b = in_g / here;
+    if (wide && here == kGroup) {
+        // the patch of an XCD the other way round: 32 consecutive ids are 4 of the grouped dimension x 8 of the walked one
+        const int blk = in_g / (8 * kGroup), r = in_g % (8 * kGroup);
+        if ((blk + 1) * 8 <= n_b) {
+            a = first_a + (r / 32) * 4 + (r % 4);
+            b = blk * 8 + (r % 32) / 4;
+        }
+    }
     tr = by_columns ? b : a;
     tc = by_columns ? a : b;
 }
 __device__ __forceinline__ void tile_of_block(int tiles_r, int tiles_c, int& tr, int& tc) {
-    tile_of_id(blockIdx.x, tiles_r, tiles_c, false, tr, tc);
+    tile_of_id(blockIdx.x, tiles_r, tiles_c, false, false, tr, tc);
 }
 
 // Which operand the walk of 256 x 256 tiles groups.  The panels of the grouped operand (eight per group, one group per
@@ -397,7 +405,17 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     const int tiles_r = (NR + kDmaTile - 1) / kDmaTile, tiles_c = (NC + kDmaTile - 1) / kDmaTile;
     const bool by_columns = walk_by_columns(tiles_r, tiles_c, K);
     int tr, tc;
-    tile_of_id(blockIdx.x, tiles_r, tiles_c, by_columns, tr, tc);
+    // Which way round the 32 tiles of an XCD lie.  A K-major operand with a long leading dimension that is a multiple
+    // of 4 KiB is hard on that XCD's L2: the 128 k-rows of a tile's 256-byte strip lie a multiple of 4 KiB apart, L2
+    // misses double (TCC_MISS, FETCH_SIZE x 2.4 on 8192 x 28672 x 16384 with Y as [K, 28672]) and the CUs that share
+    // the strip all wait.  Eight such strips shared by four CUs each then beat four shared by eight: the patch is turned
+    // so that this operand gets the eight (that shape: 2.82 -> 3.07 PFLOP/s; with X K-major as well 2.73 -> 3.09;
+    // 28672 x 8192 x 16384, both K-major: 2.88 -> 3.02).  Measured only where it is applied: K of 16384 and more, one
+    // such operand (with two, or at K = 8192, turning the patch lost 1 to 7 %).
+    auto strips = [](int n) { return n % 4096 == 0 && n >= 12288; };
+    const bool strips_x = XT && strips(NR), strips_y = YT && strips(NC);
+    const bool wide = K >= 16384 && strips_x != strips_y && (strips_y ? !by_columns : by_columns);
+    tile_of_id(blockIdx.x, tiles_r, tiles_c, by_columns, wide, tr, tc);
     const int row0 = tr * kDmaTile, col0 = tc * kDmaTile;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wr = wave >> 1, wc = wave & 1;
@@ -569,7 +587,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         const int nid = blockIdx.x + 256;
         if (nid < tiles_r * tiles_c) {
             int ntr, ntc;
-            tile_of_id(nid, tiles_r, tiles_c, by_columns, ntr, ntc);
+            tile_of_id(nid, tiles_r, tiles_c, by_columns, wide, ntr, ntc);
             const int nr0 = ntr * kDmaTile, nc0 = ntc * kDmaTile;
             // line L of an operand's 512: row-major, half L % 2 of row L / 2 (clamped like the tile loads); K-major (whole
             // tiles only), half L % 2 of the tile's 256 bytes in k-row L / 2 (K >= 256 here)
