@@ -485,3 +485,34 @@ def test_random_small_ragged_problems_with_bias_and_accumulation(be):
         got = _run(be, a, a_dt, a_si, b, b_dt, b_si, out_dtype=od, accumulate=base is not None, bias=bias,
                    out=None if base is None else base.clone().cuda())
         assert rel_fro(got.float(), ref) < (TOL_F32 if od == torch.float32 else TOL_16), (it, m, n, k, od, mode)
+
+
+@pytest.mark.parametrize('nr,nc,k,a_kmajor,b_kmajor', [
+    (28672, 8192, 16384, True, True),      # tile columns grouped, the XCD patch turned for X
+    (8192, 28672, 16384, True, True),      # tile rows grouped, the patch turned for Y
+    (8192, 28672, 16384, True, False),     # the same with only Y K-major
+    (8192, 12288, 16384, False, False),    # row-major: the patch as it was
+    (16384, 4096, 4096, False, False),     # tall, everything cached: rows grouped
+    (4096, 16384, 4096, False, False),     # wide: columns grouped
+    (28928, 8448, 256, False, False),      # 113 x 33 tiles: a count that 8 does not divide
+    (1280, 2304, 256, True, True),         # 5 x 9 tiles, fewer than one round
+])
+def test_every_tile_is_written_whatever_the_walk(be, nr, nc, k, a_kmajor, b_kmajor):
+    """The tile walk (groups of tile rows or columns, XCD-contiguous ids, the patch of an XCD turned or not) is chosen
+    from the shape and the operand layouts.  Operands that are constant along K make the whole output predictable,
+    D[r, c] = K * x[r] * y[c] with powers of two (exact in bf16), so a tile that the walk skipped, or wrote twice with
+    another tile's data, shows."""
+    g = torch.Generator(device='cuda').manual_seed(nr + nc)
+    # E4M3 codes of 2^-2 .. 2^1: exponent field 5 .. 8, mantissa 0
+    ex = torch.randint(5, 9, (nr, ), device='cuda', generator=g, dtype=torch.int32)
+    ey = torch.randint(5, 9, (nc, ), device='cuda', generator=g, dtype=torch.int32)
+    xs = (ex << 3).to(torch.uint8)
+    ys = (ey << 3).to(torch.uint8)
+    x = xs.view(1, nr).expand(k, nr).contiguous() if b_kmajor else xs.view(nr, 1).expand(nr, k).contiguous()
+    y = ys.view(1, nc).expand(k, nc).contiguous() if a_kmajor else ys.view(nc, 1).expand(nc, k).contiguous()
+    out = torch.full((nr, nc), float('nan'), dtype=torch.bfloat16, device='cuda')
+    one = torch.ones((), device='cuda')
+    be.fp8_gemm(y, 5, one, x, 5, one, out, a_kmajor=a_kmajor, b_kmajor=b_kmajor)
+    want = (float(k) * torch.exp2((ex - 7).float()).view(nr, 1) * torch.exp2((ey - 7).float()).view(1, nc)).to(torch.bfloat16)
+    bad = (out != want) | out.isnan()
+    assert not bool(bad.any()), f'{int(bad.sum())} wrong outputs, first at {bad.nonzero()[0].tolist()}'
