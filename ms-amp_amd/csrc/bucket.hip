@@ -14,7 +14,7 @@ constexpr int kBucketThreads = 256;
 // as a rule the scale this round will arrive at; msamp_bucket_cast then finds its work done (see bucket_scale_kernel).
 template <typename IT, int FMT>
 __global__ __launch_bounds__(kBucketThreads) void bucket_amax_kernel(msamp_bucket_item* __restrict__ items,
-                                                                     const int32_t* __restrict__ block_map) {
+                                                                     const int32_t* __restrict__ block_map, int stream) {
     constexpr int EPT = In16<IT>::EPT;
     constexpr int kVecs = MSAMP_BUCKET_CHUNK / (kBucketThreads * EPT);    // 16 (fp32) or 8 (16-bit)
     __shared__ uint32_t red[kBucketThreads / kWave];
@@ -29,7 +29,8 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_amax_kernel(msamp_bucke
     if (base + MSAMP_BUCKET_CHUNK <= n && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && vec_out) {
         float v[kVecs][EPT];
 #pragma unroll
-        for (int u = 0; u < kVecs; ++u) In16<IT>::load(x + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT, v[u]);
+        for (int u = 0; u < kVecs; ++u)
+            In16<IT>::load(x + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT, v[u], stream != 0);
 #pragma unroll
         for (int u = 0; u < kVecs; ++u) {
 #pragma unroll
@@ -97,7 +98,7 @@ __global__ void bucket_scale_kernel(msamp_bucket_item* items, int n_items, float
 
 template <typename IT, int FMT>
 __global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp_bucket_item* __restrict__ items,
-                                                                     const int32_t* __restrict__ block_map) {
+                                                                     const int32_t* __restrict__ block_map, int stream) {
     constexpr int EPT = In16<IT>::EPT;
     constexpr int kVecs = MSAMP_BUCKET_CHUNK / (kBucketThreads * EPT);
     const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
@@ -112,7 +113,8 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp
     if (base + MSAMP_BUCKET_CHUNK <= n && vec) {
         float v[kVecs][EPT];
 #pragma unroll
-        for (int u = 0; u < kVecs; ++u) In16<IT>::load(x + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT, v[u]);
+        for (int u = 0; u < kVecs; ++u)
+            In16<IT>::load(x + base + (static_cast<size_t>(u) * kBucketThreads + threadIdx.x) * EPT, v[u], stream != 0);
 #pragma unroll
         for (int u = 0; u < kVecs; ++u) {
             uint32_t w[EPT / 4];
@@ -235,15 +237,18 @@ static int bucket_amax_launch(const char* who, msamp_bucket_item* items, int n_i
     const int rc = check_bucket_args(who, items, n_items, block_map, n_blocks, in_dtype);
     if (rc != MSAMP_OK || n_items == 0) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // more bytes than the caches keep: read them as a stream
+    const int in_size = in_dtype == MSAMP_DT_F32 ? 4 : 2;
+    const int streams = static_cast<size_t>(n_blocks) * MSAMP_BUCKET_CHUNK * in_size >= kStreamBytes ? 1 : 0;
     if (n_blocks > 0) {
 #define BUCKET_AMAX(IT)                                                                                                 \
     do {                                                                                                              \
         if (fp8_type == MSAMP_DT_E4M3)                                                                                \
-            hipLaunchKernelGGL((bucket_amax_kernel<IT, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+            hipLaunchKernelGGL((bucket_amax_kernel<IT, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map, streams); \
         else if (fp8_type == MSAMP_DT_E5M2)                                                                           \
-            hipLaunchKernelGGL((bucket_amax_kernel<IT, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+            hipLaunchKernelGGL((bucket_amax_kernel<IT, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map, streams); \
         else                                                                                                          \
-            hipLaunchKernelGGL((bucket_amax_kernel<IT, 0>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+            hipLaunchKernelGGL((bucket_amax_kernel<IT, 0>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map, streams); \
     } while (0)
         if (in_dtype == MSAMP_DT_F32) BUCKET_AMAX(float);
         else if (in_dtype == MSAMP_DT_F16) BUCKET_AMAX(f16_t);
@@ -280,12 +285,14 @@ int msamp_bucket_cast(msamp_bucket_item* items, int n_items, const int32_t* bloc
                        margin, pre_scale, scale_inv_div);
     MSAMP_CHECK_LAUNCH("bucket_scale_kernel");
     if (n_blocks == 0) return MSAMP_OK;
+    const int in_size = in_dtype == MSAMP_DT_F32 ? 4 : 2;
+    const int streams = static_cast<size_t>(n_blocks) * MSAMP_BUCKET_CHUNK * in_size >= kStreamBytes ? 1 : 0;
 #define BUCKET_CAST(IT)                                                                                                  \
     do {                                                                                                               \
         if (fp8_type == MSAMP_DT_E4M3)                                                                                 \
-            hipLaunchKernelGGL((bucket_cast_kernel<IT, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+            hipLaunchKernelGGL((bucket_cast_kernel<IT, MSAMP_DT_E4M3>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map, streams); \
         else                                                                                                           \
-            hipLaunchKernelGGL((bucket_cast_kernel<IT, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map); \
+            hipLaunchKernelGGL((bucket_cast_kernel<IT, MSAMP_DT_E5M2>), dim3(n_blocks), dim3(kBucketThreads), 0, st, items, block_map, streams); \
     } while (0)
     if (in_dtype == MSAMP_DT_F32) BUCKET_CAST(float);
     else if (in_dtype == MSAMP_DT_F16) BUCKET_CAST(f16_t);
