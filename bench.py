@@ -372,6 +372,17 @@ def bench_grad_side(iters=10):
     out = {}
     ms = _time_gpu(lambda: bucket.quantize(grads, world_size=8), iters)
     out['bucket_quantize_32x4M_bf16'] = {'ms': ms, 'GBps': n * len(grads) * 3 / ms / 1e6}
+    # the same through the two C entry points alone, tables built once (what the launches cost without the Python around them)
+    import math
+    items, block_map = bucket._get_tables(grads)
+    in_dt = _backend._dt(grads[0])
+
+    def two_calls():
+        _backend.bucket_amax(items, block_map, in_dt, nan_to_inf=True, speculate_fp8_dt=int(bucket.qtype))
+        _backend.bucket_cast(items, block_map, in_dt, int(bucket.qtype), 1.0 / math.sqrt(8), 8.0)
+
+    ms = _time_gpu(two_calls, iters)
+    out['bucket_quantize_32x4M_bf16_entry_points_only'] = {'ms': ms, 'GBps': n * len(grads) * 3 / ms / 1e6}
     # beside it: without the codes going out during the amax pass (input read twice)
     bucket = GradientBucket([n] * len(grads), speculate=False)
     ms = _time_gpu(lambda: bucket.quantize(grads, world_size=8), iters)
