@@ -491,6 +491,7 @@ def test_random_small_ragged_problems_with_bias_and_accumulation(be):
     (28672, 8192, 16384, True, True),      # tile columns grouped, the XCD patch turned for X
     (8192, 28672, 16384, True, True),      # tile rows grouped, the patch turned for Y
     (8192, 28672, 16384, True, False),     # the same with only Y K-major
+    (9216, 28672, 16384, True, False),     # the same with a last group of four tile rows
     (8192, 12288, 16384, False, False),    # row-major: the patch as it was
     (16384, 4096, 4096, False, False),     # tall, everything cached: rows grouped
     (4096, 16384, 4096, False, False),     # wide: columns grouped
