@@ -94,7 +94,7 @@ struct In16;    // one 16-byte load = EPT elements as float
 // once.  Plain streaming reads of 2 GiB reach 6.4 TB/s on this part with ordinary loads and 7.1 TB/s with the mark; on
 // data that a cache still holds the mark costs (the transposes, 64 MiB casts: 6 to 25 % slower), so the callers set it
 // by size.
-constexpr size_t kStreamBytes = 192ull << 20;
+constexpr size_t kStreamBytes = 96ull << 20;
 __device__ __forceinline__ uint4 ld16(const void* p, bool stream = false) {
     if (stream) {
         typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
