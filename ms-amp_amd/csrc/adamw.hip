@@ -319,13 +319,6 @@ __global__ void fused_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, 
     *d.v_amax = av;
 }
 
-// The new payloads are not read again before the next step, by when no cache holds them: they are stored past the
-// caches (1.77 -> 1.73 ms for 1.0e9 parameters in the one-pass step; the same mark on the loads cost 1.5 %).
-__device__ __forceinline__ void st16(void* p, const uint4& v) {
-    typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
-    const v4u_t t = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(t, static_cast<v4u_t*>(p));
-}
 template <int WDT>
 __device__ __forceinline__ void store_w16(void* base, size_t i, const float* f) {
     if constexpr (WDT == MSAMP_DT_F16) {
@@ -333,15 +326,15 @@ __device__ __forceinline__ void store_w16(void* base, size_t i, const float* f) 
 #pragma unroll
         for (int j = 0; j < 8; ++j) w[j] = float_to_f16_bits(f[2 * j]) | (float_to_f16_bits(f[2 * j + 1]) << 16);
         uint4* p = reinterpret_cast<uint4*>(static_cast<uint16_t*>(base) + i);
-        st16(p, make_uint4(w[0], w[1], w[2], w[3]));
-        st16(p + 1, make_uint4(w[4], w[5], w[6], w[7]));
+        p[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        p[1] = make_uint4(w[4], w[5], w[6], w[7]);
     } else {
         uint4 o;
         o.x = quant4<WDT>(f[0], f[1], f[2], f[3]);
         o.y = quant4<WDT>(f[4], f[5], f[6], f[7]);
         o.z = quant4<WDT>(f[8], f[9], f[10], f[11]);
         o.w = quant4<WDT>(f[12], f[13], f[14], f[15]);
-        st16(static_cast<uint8_t*>(base) + i, o);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(base) + i) = o;
     }
 }
 
@@ -397,15 +390,15 @@ __device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t
     }
     if constexpr (WDT == MSAMP_DT_F16) {
         uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
-        st16(o, make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16)));
-        st16(o + 1, make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16)));
+        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
+        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
     } else {
         uint4 o;
         o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
         o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
         o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-        st16(static_cast<uint8_t*>(w_out) + i, o);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
     }
     store_w16<MSAMP_DT_E4M3>(m_out, i, m);
     store_w16<MSAMP_DT_F16>(v_out, i, v);
@@ -519,15 +512,15 @@ __device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_o
     }
     if constexpr (WDT == MSAMP_DT_F16) {
         uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
-        st16(o, make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16)));
-        st16(o + 1, make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16)));
+        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
+        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
     } else {
         uint4 o;
         o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
         o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
         o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-        st16(static_cast<uint8_t*>(w_out) + i, o);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
     }
     store_w16<MSAMP_DT_E4M3>(m_out, i, m);
     store_w16<MSAMP_DT_F16>(v_out, i, v);
