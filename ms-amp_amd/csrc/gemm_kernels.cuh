@@ -528,9 +528,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     for (int p = n * np / 16; p < (n + 1) * np / 16; ++p) read_piece(rd_dst, rd_stage, rd_x, rd_half, p);
                 }
                 if (do_load && (n & 1)) dma(ld_kt, ld_stage, ld_first + (n >> 1));
-                // Nothing moves across: one MFMA, then the reads and the load that go with it.  Left a free hand, the
-                // scheduler stretches the fragments' live ranges until the register allocator no longer updates the 64
-                // accumulators in place and copies them around between the MFMAs.
+                // Nothing moves across: one MFMA, then the reads and the load that go with it, so that the LDS reads and
+                // the tile loads stay spread evenly between the MFMAs as written.
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
@@ -564,8 +563,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
 #pragma unroll
     for (int p = 0; p < kPY; ++p) read_piece(fy[0], 0, false, 0, p);
     // Two slices per turn of the loop (stage 0, stage 1).  What is left afterwards -- two slices when the slice count is
-    // even, three when it is odd (ODD_NK, chosen by the host) -- follows as straight-line code, so that no branch sits
-    // between the MFMAs (another thing that makes the compiler shuffle the accumulators between registers).
+    // even, three when it is odd (ODD_NK, chosen by the host) -- follows as straight-line code: the last slices load
+    // nothing and the last one reads no fragments for a successor, which the compiler then knows.
     int kt = 0;
     for (; kt + 3 < nk; kt += 2) {
         slice(0, true, kt + 2, true);
