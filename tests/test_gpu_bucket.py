@@ -236,3 +236,26 @@ def test_clip_grad_norm_uses_the_codes():
         for p, old in zip(params, before):
             assert torch.allclose(p.grad.float(), old * coef, rtol=1e-5, atol=0)
         assert all(torch.equal(c, p.grad.value) for c, p in zip(codes, [p for p in params if hasattr(p.grad, 'value')]))
+
+
+@pytest.mark.parametrize('speculate', [True, False])
+def test_bucket_larger_than_the_caches_equals_its_tensors_one_by_one(speculate):
+    """A bucket whose gradients add up to 128 MiB is read as a stream; the same gradients in buckets of one (32 MiB each)
+    are not.  Same codes, scales and amax either way, on a first round (fresh metas) and a second one (the scales of
+    the first are guessed and mostly hold)."""
+    from msamp.nn import GradientBucket
+    n = 16 * 1024 * 1024
+    g = torch.Generator(device='cuda').manual_seed(9)
+    grads = [(torch.randn(n, device='cuda', generator=g) * 10.0 ** (i - 3)).bfloat16() for i in range(4)]
+    big = GradientBucket([n] * 4, speculate=speculate)
+    small = [GradientBucket([n], speculate=speculate) for _ in range(4)]
+    for rnd in range(2):
+        if rnd == 1:
+            grads = [x * 1.01 for x in grads]
+        out_big = big.quantize(grads, world_size=4)
+        for i, b in enumerate(small):
+            out = b.quantize([grads[i]], world_size=4)[0]
+            assert torch.equal(b.flat, big.flat[i * n:(i + 1) * n]), (rnd, i)
+            for name in ('scale', 'scale_inv'):
+                assert same_float(getattr(out.meta, name), getattr(out_big[i].meta, name)), (rnd, i, name)
+            assert same_float(out.meta.amax[0], out_big[i].meta.amax[0])
