@@ -135,7 +135,8 @@ __global__ __launch_bounds__(kBucketThreads) void bucket_cast_kernel(const msamp
 }
 
 // ---- norms of FP8 gradients (clip_grad_norm_) ----------------------------------------------------------------
-// sum |q|^p (p = 1, 2) or max |q| over the codes of each tensor, accumulated in double: the dequantization factor
+// sum |q|^p (p = 1, 2) or max |q| over the codes of each tensor, accumulated in double (four elements at a time are
+// summed in float32 first): the dequantization factor
 // is constant per tensor and is applied once at the end, so a tensor is read at one byte per element and never
 // expanded to float32 in memory.
 template <int FMT, int KIND>    // KIND: 1, 2, or 0 for the maximum
@@ -170,7 +171,16 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_norm_kernel(msamp_norm_ite
             for (int j = 0; j < 4; ++j) {
                 float a, b, c, e;
                 dequant4<FMT>(words[j], a, b, c, e);
-                take(a), take(b), take(c), take(e);
+                if constexpr (KIND == 0) {
+                    take(a), take(b), take(c), take(e);
+                } else if constexpr (KIND == 1) {
+                    // four values at a time in float32 (three roundings of 2^-24 each), then into the double sum: a
+                    // double conversion and addition per element kept the vector units busier than the memory
+                    acc += static_cast<double>((fabsf(a) + fabsf(b)) + (fabsf(c) + fabsf(e)));
+                } else {
+                    // the square of an FP8 value is exact in float32
+                    acc += static_cast<double>(fmaf(a, a, b * b) + fmaf(c, c, e * e));
+                }
             }
         }
     } else {
