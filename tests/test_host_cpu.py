@@ -247,3 +247,38 @@ def test_chunk_map_rows_and_cache():
     assert m.tolist() == [[0, 0], [0, 1], [0, 2], [2, 0]]
     assert _backend.chunk_map([2 * c + 1, 0, c], 'cpu') is m
     assert _backend.chunk_map([], 'cpu').shape[0] == 0
+
+
+def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(tmp_path):
+    """The accumulators of fp8_gemm_dma_kernel live in fixed AGPRs behind the compiler's back (inline-assembly MFMAs).
+    That holds only while the compiler itself uses no AGPR in those kernels (it would, to spill VGPRs) and no scratch
+    memory: compile the kernels of one format pair to assembly and look.  Cross-compiles without a GPU."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which('hipcc') or '/opt/rocm/bin/hipcc'
+    if not os.path.exists(hipcc):
+        pytest.skip('no hipcc here')
+    src = os.path.join(os.path.dirname(_backend.__file__), '..', 'csrc')
+    out = str(tmp_path / 'gemm_inst.s')
+    cmd = [hipcc, '--offload-arch=gfx950', '-O3', '-std=c++17', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+           '-Wno-unused-command-line-argument', '-Wno-inline-asm', '-DMSAMP_XF=5', '-DMSAMP_YF=5', '--cuda-device-only', '-S',
+           '-o', out, os.path.join(src, 'gemm_inst.hip')]
+    subprocess.run(cmd, check=True, capture_output=True, cwd=src)
+    kernel, in_asm, found = None, False, {}
+    for line in open(out):
+        m = re.match(r'^(_Z\w+):', line)
+        if m:
+            kernel = m.group(1)
+        elif '#ASMSTART' in line:
+            in_asm = True
+        elif '#ASMEND' in line:
+            in_asm = False
+        elif kernel and 'fp8_gemm_dma_kernel' in kernel:
+            c = found.setdefault(kernel, [0, 0, 0])
+            if 'v_accvgpr' in line:
+                c[0 if in_asm else 1] += 1
+            if re.search(r'scratch_(load|store)', line):
+                c[2] += 1
+    assert len(found) >= 10    # bf16 / f16 / float outputs, row- and K-major operands, both parities, the fused cast
+    for name, (ours, compilers, scratch) in found.items():
+        assert ours >= 512 and compilers == 0 and scratch == 0, (name, ours, compilers, scratch)
