@@ -91,10 +91,10 @@ def test_bucket_reuse_and_argument_checks():
 
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 def test_bucket_speculative_rounds_equal_plain_rounds(dtype):
-    """Five rounds on one bucket, each taken with and without speculation from the same state: same buffer and metas
-    every time.  Round 1 finds scale 1 in the metas (every guess wrong); round 2 has gradients of the same size, so the
-    amax pass alone already leaves the final bytes; in round 3 half of the gradients are 64 times larger (those are
-    done again); round 4 has a NaN in one gradient; round 5 is back to normal."""
+    """Five reductions on one bucket, each taken with and without speculation from the same state: same buffer and
+    metas every time.  The first finds scale 1 in the metas (every guess wrong); the second has gradients of the same
+    size, so the amax pass alone already leaves the final bytes; in the third half of the gradients are 64 times larger
+    (those are done again); the fourth has a NaN in one gradient; the fifth is back to normal."""
     from msamp import _backend
     from msamp.nn import GradientBucket
     sizes = [5, 16384, 3, 16384 * 2 + 777, 1, 4096 * 33, 100, 16384 * 4]
