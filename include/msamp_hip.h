@@ -268,19 +268,27 @@ int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv
 
 /* The weight-gradient GEMM of a linear layer followed by its cast to FP8 (nn/functional.py:100-111 followed by
  * :121-123 of the reference: `wgrad = Gemm.fp8_gemm(...)`, then `wgrad.cast(Dtypes.kfloat8_e4m3, meta=..., sync=True)`)
- * as ONE launch: q = FP8 codes of round_to_d_dtype(D) * scale, with *amax = max |round_to_d_dtype(D)|, *scale from the
- * pow-2 rule of that amax (fallback: the old *scale) and *scale_inv = 1 / *scale -- bit for bit what
- * msamp_fp8_gemm_kmajor into a d_dtype buffer followed by msamp_cast_to_fp8_intime of that buffer gives, without the
- * buffer.  flags and workspace as for msamp_cast_to_fp8_intime.
- * Returns MSAMP_NOT_FUSED (1), having done nothing, when the fused form does not apply and the caller has to take
- * the two steps: it needs m and n multiples of 256, k a multiple of 128 and at least 256, at most one 256 x 256 output tile per
- * compute unit (its workgroups wait for each other), q_type E4M3, both operands K-major or neither, a stream on which
- * such kernels are allowed (not capturing, the device's first), and no MSAMP_FLAG_TWO_PASS. */
+ * without the second trip over the product: q = FP8 codes of round_to_d_dtype(D) * scale, with
+ * *amax = max |round_to_d_dtype(D)|, *scale from the pow-2 rule of that amax (fallback: the old *scale) and
+ * *scale_inv = 1 / *scale -- bit for bit what msamp_fp8_gemm_kmajor into a d_dtype buffer followed by
+ * msamp_cast_to_fp8_intime of that buffer gives.  flags and workspace as for msamp_cast_to_fp8_intime.  Two forms:
+ *  - one launch, the product never leaves the chip: at most one 256 x 256 output tile per compute unit (the workgroups
+ *    wait for each other), accumulate == 0, a stream on which such kernels are allowed (not capturing, no other stream
+ *    of the device busy with them), no MSAMP_FLAG_TWO_PASS;
+ *  - on speculation, any number of tiles, any stream, also under capture: needs d, a buffer of n x m d_dtype elements
+ *    (16-byte aligned).  The GEMM stores the product there as msamp_fp8_gemm_kmajor would (added to what d holds if
+ *    accumulate != 0: gradient accumulation, functional.py:100-111) and beside it the codes for the scale the meta
+ *    holds before the call; the workgroup that finishes last applies the rule, and only if the rule arrives at another
+ *    scale does a second launch read d again and rewrite the codes.  On return d holds the (accumulated) product.
+ *    Not taken with MSAMP_FLAG_NO_SPECULATION, nor for d_dtype float32.
+ * Both need m and n multiples of 256, k a multiple of 128 and at least 256, q_type E4M3, both operands K-major or
+ * neither.  d may be null: then only the first form is considered.
+ * Returns MSAMP_NOT_FUSED (1), having done nothing, when neither form applies and the caller has to take the two steps. */
 #define MSAMP_NOT_FUSED 1
 int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b, int b_type,
-                        const float* b_scale_inv, int b_kmajor, int d_dtype, uint8_t* q, int q_type, float* scale,
-                        float* amax, float* scale_inv, int m, int n, int k, int margin, int flags, void* workspace,
-                        msamp_stream_t stream);
+                        const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int accumulate, uint8_t* q, int q_type,
+                        float* scale, float* amax, float* scale_inv, int m, int n, int k, int margin, int flags,
+                        void* workspace, msamp_stream_t stream);
 
 /* msamp_adamw.adamw_fp8_stage1_compute (adamw.cu:99-127): fp32 param/grad, quantized moments;
  * updates param in place and atomically maxes |m'|, |v'| into the two amax cells.

@@ -2,6 +2,7 @@
 // amax-window update.  All bandwidth-bound: 16-byte lane-contiguous loads, packed FP8 converters,
 // wavefront shuffle reductions, one atomic per block.
 #include "common.cuh"
+#include "gemm_call.h"
 
 #include <atomic>
 #include <mutex>
@@ -54,7 +55,8 @@ struct Gate {
 __device__ __forceinline__ bool gate_closed(const Gate& g) { return g.counter != nullptr && *g.counter >= g.window; }
 
 // where cast_to_fp8_kernel takes its scale from
-enum ScaleSource { kGivenScale = 0, kInTime = 1, kRescale = 2 };
+// (kGivenIfFlagged: as kGivenScale, but the launch does nothing unless the word it.ws points at is non-zero)
+enum ScaleSource { kGivenScale = 0, kInTime = 1, kRescale = 2, kGivenIfFlagged = 3 };
 
 // every workgroup of the second pass derives the same amax and scale from the partial maxima
 __device__ __forceinline__ float resolve_in_time_scale(const InTimeArgs& a, uint32_t* red, float* scale_inv) {
@@ -112,6 +114,9 @@ __global__ __launch_bounds__(THREADS) void cast_to_fp8_kernel(const IT* __restri
         if (blockIdx.x == 0 && it.amax_copy != nullptr) {
             for (int j = threadIdx.x; j < it.window; j += blockDim.x) it.amax_copy[j] = it.known_amax[j];
         }
+    } else if constexpr (INTIME == kGivenIfFlagged) {
+        if (*it.ws == 0u) return;    // the codes written on speculation stand
+        s = *scale_p;
     } else {
         s = *scale_p;
     }
@@ -1019,6 +1024,26 @@ static int launch_amax(const IT* x, size_t n, uint32_t* ws, const float* scale, 
     return MSAMP_OK;
 }
 
+template <typename IT>
+static int launch_cast_if_flagged(const IT* d, size_t n, const float* scale, uint8_t* q, int q_type, const uint32_t* redo,
+                                  hipStream_t st) {
+    constexpr int EPT = In16<IT>::EPT;
+    const int vec_ok = (aligned(d, 16) && aligned(q, EPT) ? 1 : 0) | (n * sizeof(IT) >= kStreamBytes ? 2 : 0);
+    // as a rule every workgroup returns at once: few of them, grid-stride
+    int grid = grid_for(n, static_cast<size_t>(kCastThreads) * EPT * kCastUnroll);
+    const int cap = cu_count() * 4;
+    grid = grid < cap ? grid : cap;
+    const InTimeArgs flag = {redo, nullptr, nullptr, 0.0f, 0, 0, nullptr, nullptr, nullptr, 0, nullptr, 0};
+    if (q_type == MSAMP_DT_E4M3)
+        hipLaunchKernelGGL((cast_to_fp8_kernel<IT, MSAMP_DT_E4M3, false, kGivenIfFlagged>), dim3(grid), dim3(kCastThreads), 0, st, d, q, n,
+                           scale, static_cast<float*>(nullptr), static_cast<float*>(nullptr), vec_ok, 0, flag);
+    else
+        hipLaunchKernelGGL((cast_to_fp8_kernel<IT, MSAMP_DT_E5M2, false, kGivenIfFlagged>), dim3(grid), dim3(kCastThreads), 0, st, d, q, n,
+                           scale, static_cast<float*>(nullptr), static_cast<float*>(nullptr), vec_ok, 0, flag);
+    MSAMP_CHECK_LAUNCH("cast_to_fp8_kernel (if flagged)");
+    return MSAMP_OK;
+}
+
 // first pass: partial maxima of |x| into the workspace (plus the scale in force, for the rule's fallback)
 constexpr Gate kNoGate = {nullptr, 0};
 
@@ -1039,23 +1064,16 @@ static int dispatch_amax(const void* x, int dtype, size_t n, void* ws, const flo
     return MSAMP_ERR_DTYPE;
 }
 
-// true if the runtime confirms kResBlocksPerCu workgroups of this kernel fit one CU (asked once per kernel)
-static bool fits_resident(const void* fn) {
-    static std::mutex mu;
-    static const void* known[32];
-    static bool fits[32];
-    static int n_known = 0;
-    std::lock_guard<std::mutex> lock(mu);
-    for (int i = 0; i < n_known; ++i)
-        if (known[i] == fn) return fits[i];
-    int blocks = 0;
-    const bool ok = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, fn, kResThreads, 0) == hipSuccess &&
-                    blocks >= kResBlocksPerCu;
-    if (n_known < 32) {
-        known[n_known] = fn;
-        fits[n_known++] = ok;
+// true if the runtime confirms kResBlocksPerCu workgroups of this kernel fit one CU; `state` is the caller's
+// function-local cache for one instantiation (-1 = not asked yet)
+static bool fits_resident(const void* fn, std::atomic<int>& state) {
+    int fits = state.load(std::memory_order_acquire);
+    if (fits < 0) {
+        int blocks = 0;
+        fits = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, fn, kResThreads, 0) == hipSuccess && blocks >= kResBlocksPerCu;
+        state.store(fits, std::memory_order_release);
     }
-    return ok;
+    return fits != 0;
 }
 
 // One-pass (register-resident) in-time cast; returns 1 if it does not apply and the two-pass path must run.
@@ -1084,7 +1102,8 @@ static int launch_resident(const IT* x, size_t n, float* scale, float* amax, flo
     bool fits = true;
 #define LAUNCH(FMT, R) \
     do { \
-        fits = fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, FMT, R, SPEC>)); \
+        static std::atomic<int> fits_state{-1}; \
+        fits = fits_resident(reinterpret_cast<const void*>(&cast_intime_resident_kernel<IT, FMT, R, SPEC>), fits_state); \
         if (fits) hipLaunchKernelGGL((cast_intime_resident_kernel<IT, FMT, R, SPEC>), dim3(static_cast<unsigned>(g)), dim3(kResThreads), 0, st, x, out, n, scale, amax, scale_inv, slots, fp_max, margin, flags, rounds, token, spin_limit, error_word); \
     } while (0)
 #define LAUNCH_R(FMT) \
@@ -1347,25 +1366,39 @@ static int launch_add_to_fp8(uint8_t* q, int fp8_type, const IT* other, size_t n
 // only the address hipGetSymbolAddress reports for the device that is current.
 static __device__ __align__(256) __attribute__((used)) unsigned char scratch[MSAMP_WORKSPACE_BYTES];
 
-static int static_workspace(void** ws) {
+int static_workspace(void** ws) {
     static std::mutex mu;
     static void* ptrs[64];
     static bool known[64];
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
-    MSAMP_REQUIRE(dev >= 0 && dev < 64, MSAMP_ERR_SHAPE, "msamp_cast_to_fp8_intime_static: device index %d", dev);
+    MSAMP_REQUIRE(dev >= 0 && dev < 64, MSAMP_ERR_SHAPE, "static workspace: device index %d", dev);
     std::lock_guard<std::mutex> lock(mu);
     if (!known[dev]) {
         void* p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
-        MSAMP_REQUIRE(p != nullptr, MSAMP_ERR_WORKSPACE, "msamp_cast_to_fp8_intime_static: no address for the static workspace");
+        MSAMP_REQUIRE(p != nullptr, MSAMP_ERR_WORKSPACE, "no address for the static workspace");
         ptrs[dev] = p;
         known[dev] = true;
     }
     *ws = ptrs[dev];
     return MSAMP_OK;
+}
+
+int cast_again_if_flagged(const void* d, int d_dtype, size_t n, const float* scale, uint8_t* q, int q_type, const uint32_t* redo,
+                          hipStream_t st) {
+    switch (d_dtype) {
+        case MSAMP_DT_F32:
+            return launch_cast_if_flagged(static_cast<const float*>(d), n, scale, q, q_type, redo, st);
+        case MSAMP_DT_F16:
+            return launch_cast_if_flagged(static_cast<const f16_t*>(d), n, scale, q, q_type, redo, st);
+        case MSAMP_DT_BF16:
+            return launch_cast_if_flagged(static_cast<const bf16_t*>(d), n, scale, q, q_type, redo, st);
+    }
+    set_error("unsupported dtype %d", d_dtype);
+    return MSAMP_ERR_DTYPE;
 }
 
 }    // namespace msamp

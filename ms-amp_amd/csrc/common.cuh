@@ -20,6 +20,8 @@ int hip_fail(hipError_t e, const char* what);
 bool waiting_kernels_allowed(hipStream_t st);
 // `count` consecutive non-zero tokens, unique in this process
 uint32_t next_tokens(uint32_t count);
+// device address of the library's own workspace (the one msamp_cast_to_fp8_intime_static uses) on the current device
+int static_workspace(void** ws);
 // how many times the collecting workgroup of a waiting kernel polls before it gives up (msamp_set_spin_limit)
 uint32_t collector_spin_limit();
 

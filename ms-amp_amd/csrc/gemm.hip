@@ -23,36 +23,53 @@ static bool kmajor_shape_ok(int NR, int NC, int K, bool xt, bool yt) {
 
 using namespace msamp;
 
+// words of the workspace that the speculative form of msamp_fp8_gemm_cast uses: running maximum, ticket counter (both
+// left at zero by every call) and the flag its second launch reads
+constexpr int kWsGemmSpec = 10;
+
 extern "C" int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
-                                   int b_type, const float* b_scale_inv, int b_kmajor, int d_dtype, uint8_t* q, int q_type,
-                                   float* scale, float* amax, float* scale_inv, int m, int n, int k, int margin, int flags,
-                                   void* workspace, msamp_stream_t stream) {
+                                   int b_type, const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int accumulate,
+                                   uint8_t* q, int q_type, float* scale, float* amax, float* scale_inv, int m, int n, int k,
+                                   int margin, int flags, void* workspace, msamp_stream_t stream) {
     MSAMP_REQUIRE(is_fp8(a_type) && is_fp8(b_type) && is_fp8(q_type), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_cast: types %d, %d -> %d",
                   a_type, b_type, q_type);
     MSAMP_REQUIRE(is_hp(d_dtype), MSAMP_ERR_DTYPE, "msamp_fp8_gemm_cast: intermediate dtype %d", d_dtype);
     MSAMP_REQUIRE(m > 0 && n > 0 && k > 0, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_cast: m=%d n=%d k=%d", m, n, k);
     MSAMP_REQUIRE(a && b && q && a_scale_inv && b_scale_inv && scale && amax && scale_inv, MSAMP_ERR_NULL,
                   "msamp_fp8_gemm_cast: null pointer");
-    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(q, 16), MSAMP_ERR_ALIGNMENT,
-                  "msamp_fp8_gemm_cast: operands and output must be 16-byte aligned");
+    MSAMP_REQUIRE(!accumulate || d != nullptr, MSAMP_ERR_NULL, "msamp_fp8_gemm_cast: accumulate needs d");
+    MSAMP_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(q, 16) && aligned(d, 16), MSAMP_ERR_ALIGNMENT,
+                  "msamp_fp8_gemm_cast: operands and outputs must be 16-byte aligned");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool both = a_kmajor && b_kmajor, neither = !a_kmajor && !b_kmajor;
     const long tiles = static_cast<long>(n / kDmaTile) * (m / kDmaTile);
     const bool fits32 = static_cast<unsigned long long>(n) * k < (1ull << 32) && static_cast<unsigned long long>(m) * k < (1ull << 32);
     if (q_type != MSAMP_DT_E4M3 || !(both || neither) || m % kDmaTile || n % kDmaTile || k % kBK || k < 2 * kBK || !fits32 ||
-        tiles > cu_count() || tiles > kMaxSlots || workspace == nullptr || (flags & MSAMP_FLAG_TWO_PASS))
+        workspace == nullptr)
         return MSAMP_NOT_FUSED;
-    if (!waiting_kernels_allowed(st)) return MSAMP_NOT_FUSED;
-    QuantArgs qa;
+    QuantArgs qa = {};
     qa.q = q, qa.scale = scale, qa.amax = amax, qa.scale_inv = scale_inv;
     qa.slots = reinterpret_cast<uint64_t*>(static_cast<char*>(workspace) + kWsSlotBytes);
     qa.fp_max = fp8_max(q_type), qa.margin = margin, qa.flags = flags;
-    qa.token = next_tokens(1);
-    qa.spin_limit = collector_spin_limit();
     qa.error_word = static_cast<uint32_t*>(workspace) + kWsErrorWord;
-    // X = b (rows of D), Y = a (columns of D)
-    const GemmCall c = {b, a, nullptr, d_dtype, n, m, k, b_scale_inv, a_scale_inv, 0, nullptr, 0, both, both, &qa, st};
-    return dispatch_pair(b_type, a_type, c);
+    qa.spec_words = static_cast<uint32_t*>(workspace) + kWsGemmSpec;
+    // one launch, D never stored: at most one tile per compute unit, on a stream that may run waiting kernels
+    if (!accumulate && tiles <= cu_count() && tiles <= kMaxSlots && !(flags & MSAMP_FLAG_TWO_PASS) && waiting_kernels_allowed(st)) {
+        qa.token = next_tokens(1);
+        qa.spin_limit = collector_spin_limit();
+        // X = b (rows of D), Y = a (columns of D)
+        const GemmCall c = {b, a, nullptr, d_dtype, n, m, k, b_scale_inv, a_scale_inv, 0, nullptr, 0, both, both, &qa, st};
+        const int rc = dispatch_pair(b_type, a_type, c);
+        if (rc != MSAMP_NOT_FUSED) return rc;
+    }
+    if (d == nullptr || (flags & MSAMP_FLAG_NO_SPECULATION)) return MSAMP_NOT_FUSED;
+    // on speculation: D and the codes for the scale in force side by side, then (only if the rule arrives at another
+    // scale) the cast of D again
+    GemmCall c = {b, a, d, d_dtype, n, m, k, b_scale_inv, a_scale_inv, accumulate, nullptr, 0, both, both, &qa, st};
+    c.qspec = true;
+    const int rc = dispatch_pair(b_type, a_type, c);
+    if (rc != MSAMP_OK) return rc;
+    return cast_again_if_flagged(d, d_dtype, static_cast<size_t>(n) * m, scale, q, q_type, qa.spec_words + 2, st);
 }
 
 extern "C" int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,

@@ -20,10 +20,12 @@ struct QuantArgs {
     uint32_t token;
     uint32_t spin_limit;
     uint32_t* error_word;    // sticky: set when a bounded wait runs out
+    uint32_t* spec_words;    // speculative form: [0] running maximum, [1] ticket counter (both zero between calls), [2] out: 1 = cast again
 };
 
 // One product D[NR][NC] = X[NR][K] . Y[NC][K]^T * *xs * *ys.  xt / yt: that operand is handed over K-major.
-// qa != nullptr: the output is cast on to FP8 in the same launch and D is not written.
+// qa != nullptr: the output is cast on to FP8 in the same launch; D is not written, unless `qspec` asks for the
+// speculative form, which stores D as usual and the codes of D times the scale in force next to it.
 struct GemmCall {
     const uint8_t* X;
     const uint8_t* Y;
@@ -38,10 +40,15 @@ struct GemmCall {
     bool xt, yt;
     const QuantArgs* qa;
     hipStream_t st;
+    bool qspec = false;
 };
 
 template <int XF, int YF>
 int run_gemm_pair(const GemmCall& c);
+
+// Implemented with the cast kernels: q = FP8(d * *scale) over n elements, unless *redo is zero (then nothing is done).
+int cast_again_if_flagged(const void* d, int d_dtype, size_t n, const float* scale, uint8_t* q, int q_type, const uint32_t* redo,
+                          hipStream_t st);
 
 extern template int run_gemm_pair<MSAMP_DT_E4M3, MSAMP_DT_E4M3>(const GemmCall&);
 extern template int run_gemm_pair<MSAMP_DT_E4M3, MSAMP_DT_E5M2>(const GemmCall&);

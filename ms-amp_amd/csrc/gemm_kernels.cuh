@@ -323,7 +323,14 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 //    bit what the two steps give, without D's trip through memory.  Every workgroup holds its tile in registers
 //    while the maxima meet (slots in the workspace, as in the one-pass in-time cast), so the launch must have all
 //    its workgroups on the chip at once: the host only takes this path for at most one tile per CU.
-// QuantArgs (the meta pointers and meeting slots of the fused cast) is declared in gemm_call.h
+//  * QSPEC: the cast to FP8 rides along on speculation instead, for any number of tiles.  The output is stored in OT as
+//    usual and, next to it, the codes of the rounded output times the scale the meta holds before the call; every
+//    workgroup folds the maximum of its rounded outputs into one word of the workspace, and the workgroup that
+//    finishes last (a ticket counter tells) applies the scale rule, rewrites the meta and leaves a flag that says
+//    whether the rule arrived at another scale than the one used.  Only then does the caller's next kernel read the
+//    stored output again and cast it with the new scale; otherwise the codes stand, bit for bit what the two steps
+//    give, and the stored output is never read back.  No workgroup waits for another.
+// QuantArgs (the meta pointers, meeting slots and workspace words of the fused casts) is declared in gemm_call.h
 
 // a * b rounded to OT (as the plain epilogue stores it) and widened again
 template <typename OT>
@@ -338,6 +345,12 @@ __device__ __forceinline__ void round_pair(float a, float b, float& ra, float& r
         const f16x2 h = __builtin_convertvector(v, f16x2);
         ra = static_cast<float>(h[0]), rb = static_cast<float>(h[1]);
     }
+}
+
+// element-wise unsigned maximum of two packed 16-bit pairs
+__device__ __forceinline__ uint32_t pk_umax16(uint32_t a, uint32_t b) {
+    typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2, a), __builtin_bit_cast(u16x2, b)));
 }
 
 // ---- the accumulators of the DMA kernel live in fixed AGPRs: block (i, j) of the wave's 8 x 8 in a[4n .. 4n+3], n = i * 8 + j.
@@ -393,7 +406,7 @@ __device__ __forceinline__ v4f acc_quad(uint32_t token) {
     return r;
 }
 
-template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0, bool ODD_NK = false>
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0, bool ODD_NK = false, bool QSPEC = false>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
                                                                      const uint8_t* __restrict__ Y, OT* __restrict__ D,
                                                                      int NR, int NC, int K,
@@ -422,6 +435,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // the output factor is fetched now: left to the epilogue, the two scalar loads sit on its critical path
     float alpha_early = (*x_scale_inv) * (*y_scale_inv);
     asm volatile("" : "+v"(alpha_early));
+    // QSPEC: the scale the codes are written with, as the meta holds it now (the last workgroup rewrites the meta)
+    float guess = 1.0f;
+    if constexpr (QSPEC) {
+        guess = *qa.scale;
+        asm volatile("" : "+v"(guess));
+    }
 
     // ---- global -> LDS.  A stage holds 256 X rows then 256 Y rows, 128 bytes per row.  One wave
     // instruction fills 8 rows (1 KiB, lane-contiguous): lane l lands in row l/8, 16-byte position l%8,
@@ -750,7 +769,21 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     constexpr int kChunksPerRow = 128 * kEsz / 16;      // 16 (2-byte) or 32 (float)
     constexpr int kRowsPerPass = 64 / kChunksPerRow;    // 4 or 2
     constexpr int kElemsPerChunk = 16 / kEsz;           // 8 or 4
-    if (!plain && vec_ok) {
+    // QSPEC: the codes of a unit leave through a second per-wave patch, behind the room of the four largest (float32)
+    // output patches; spec_max is the running maximum of the rounded outputs' magnitudes, as float32 bit patterns or
+    // as two packed 16-bit patterns (NaN patterns compare above Inf, so a NaN reaches the amax as through abs().max())
+    constexpr int kCPitch = 128 + 16;
+    uint8_t* cpatch = smem + 4 * (32 * (128 * 4 + 16)) + wave * (32 * kCPitch);
+    uint32_t spec_max = 0;
+    // the values a packed pair of 16-bit outputs stands for
+    auto widen_pair = [&](uint32_t pk, float& lo, float& hi) __attribute__((always_inline)) {
+        if constexpr (__is_same(OT, bf16_t)) {
+            lo = __uint_as_float(pk << 16), hi = __uint_as_float(pk & 0xffff0000u);
+        } else {
+            lo = f16_bits_to_float(pk & 0xffffu), hi = f16_bits_to_float(pk >> 16);
+        }
+    };
+    auto emit_fused_rows = [&]() __attribute__((always_inline)) {
         // ---- bias and / or accumulation with 16-byte row accesses: the raw float32 accumulators of a 32-row unit go
         // through a per-wave float32 patch, each lane picks up one 16-byte segment of an output row, reads the old
         // output there if it is to be added, and stores fma(acc, alpha, bias) (+ old) rounded once -- the expression of
@@ -821,12 +854,40 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                         v = make_uint4(pack_f16(r[0], r[1]), pack_f16(r[2], r[3]), pack_f16(r[4], r[5]), pack_f16(r[6], r[7]));
                     }
                     if (ok[t]) store_out16(D + static_cast<size_t>(grow) * NC + gcol, v);
+                    if constexpr (QSPEC) {
+                        // the codes of the eight (four) outputs just rounded: 8 (4) bytes of a row of q per lane
+                        float rr[kElemsPerChunk];
+                        if constexpr (kEsz == 4) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) rr[e] = r[e], spec_max = umax(spec_max, __float_as_uint(r[e]) & 0x7fffffffu);
+                        } else {
+                            const uint32_t pk[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                spec_max = pk_umax16(spec_max, pk[e] & 0x7fff7fffu);
+                                widen_pair(pk[e], rr[2 * e], rr[2 * e + 1]);
+                            }
+                        }
+                        uint8_t* qo = qa.q + static_cast<size_t>(grow) * NC + gcol;
+                        const uint32_t c0 = quant4<MSAMP_DT_E4M3>(rr[0] * guess, rr[1] * guess, rr[2] * guess, rr[3] * guess);
+                        if constexpr (kEsz == 4) {
+                            if (ok[t]) __builtin_nontemporal_store(c0, reinterpret_cast<uint32_t*>(qo));
+                        } else {
+                            const uint32_t c1 = quant4<MSAMP_DT_E4M3>(rr[4] * guess, rr[5] * guess, rr[6] * guess, rr[7] * guess);
+                            typedef uint32_t v2u_t __attribute__((ext_vector_type(2)));
+                            const v2u_t cc = {c0, c1};
+                            if (ok[t]) __builtin_nontemporal_store(cc, reinterpret_cast<v2u_t*>(qo));
+                        }
+                    }
                 }
             });
         });
+    };
+    if (!QSPEC && !plain && vec_ok) {
+        emit_fused_rows();
         return;
     }
-    if (!plain) {
+    if (!QSPEC && !plain) {
         static_for<8>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             static_for<8>([&](auto jc) {
@@ -859,13 +920,27 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     // bank terms, the same 8-byte slot; the upper eight rows swap each pair of slots (undone when read back)
                     uint8_t* dst = patch + (h * 16 + l16) * kPitch + (((j * 16 + g4 * 4) * kEsz) ^ (kEsz == 2 ? ((l16 >> 3) & 1) << 3 : 0));
                     const float v0 = a[0] * alpha, v1 = a[1] * alpha, v2 = a[2] * alpha, v3 = a[3] * alpha;
+                    float r0 = v0, r1 = v1, r2 = v2, r3 = v3;    // QSPEC: the outputs as OT holds them
                     if constexpr (kEsz == 4) {
                         *reinterpret_cast<float4*>(dst) = make_float4(v0, v1, v2, v3);
-                    } else if constexpr (__is_same(OT, bf16_t)) {
-                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(v0, v1), pack_bf16(v2, v3));
+                        if constexpr (QSPEC)
+                            spec_max = umax(umax(spec_max, __float_as_uint(v0) & 0x7fffffffu),
+                                            umax(umax(__float_as_uint(v1) & 0x7fffffffu, __float_as_uint(v2) & 0x7fffffffu),
+                                                 __float_as_uint(v3) & 0x7fffffffu));
                     } else {
-                        *reinterpret_cast<uint2*>(dst) = make_uint2(pack_f16(v0, v1), pack_f16(v2, v3));
+                        uint32_t p01, p23;
+                        if constexpr (__is_same(OT, bf16_t)) p01 = pack_bf16(v0, v1), p23 = pack_bf16(v2, v3);
+                        else p01 = pack_f16(v0, v1), p23 = pack_f16(v2, v3);
+                        *reinterpret_cast<uint2*>(dst) = make_uint2(p01, p23);
+                        if constexpr (QSPEC) {
+                            spec_max = pk_umax16(spec_max, pk_umax16(p01 & 0x7fff7fffu, p23 & 0x7fff7fffu));
+                            widen_pair(p01, r0, r1);
+                            widen_pair(p23, r2, r3);
+                        }
                     }
+                    if constexpr (QSPEC)
+                        *reinterpret_cast<uint32_t*>(cpatch + (h * 16 + l16) * kCPitch + j * 16 + g4 * 4) =
+                            quant4<MSAMP_DT_E4M3>(r0 * guess, r1 * guess, r2 * guess, r3 * guess);
                 });
             });
             // no wait between the writes above and the reads below, nor before the next unit's writes: the patch is
@@ -911,8 +986,55 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                 };
                 st(0, val0), st(1, val1), st(2, val2), st(3, val3), st(4, val4), st(5, val5), st(6, val6), st(7, val7);
             });
+            if constexpr (QSPEC) {
+                // the unit's codes: 32 rows of 128 bytes, eight rows per pass, 16 bytes per lane (whole tiles only)
+                auto crd = [&](int t) {
+                    return *reinterpret_cast<const uint4*>(cpatch + (t * 8 + (lane >> 3)) * kCPitch + (lane & 7) * 16);
+                };
+                const uint4 c0 = crd(0), c1 = crd(1), c2 = crd(2), c3 = crd(3);
+                auto cst = [&](int t, const uint4& v) {
+                    const int grow = row0 + wr * 128 + u * 32 + t * 8 + (lane >> 3);
+                    const int gcol = col0 + wc * 128 + (lane & 7) * 16;
+                    store_out16(qa.q + static_cast<size_t>(grow) * NC + gcol, v);
+                };
+                cst(0, c0), cst(1, c1), cst(2, c2), cst(3, c3);
+            }
         });
     };
+    if constexpr (QSPEC) {
+        // whole tiles and 16-byte rows only, no bias (the host sees to that): the output in OT and its codes side by side
+        if (accumulate) emit_fused_rows();
+        else emit_plain(std::true_type{}, std::true_type{});
+        uint32_t m = spec_max;
+        if constexpr (kEsz == 2) {
+            m = umax(m & 0xffffu, m >> 16);
+            if constexpr (__is_same(OT, bf16_t)) m <<= 16;
+            else m = __float_as_uint(f16_bits_to_float(m));
+        }
+        __shared__ uint32_t spec_red[kGemmThreads / kWave];
+        m = block_max_u32(m, spec_red);    // valid in lane 0 of wave 0
+        if (threadIdx.x == 0) {
+            // fold into the call's one word; the fence puts that before the ticket, and whoever draws the last ticket
+            // therefore sees every workgroup's maximum
+            uint32_t* w = qa.spec_words;
+            if (m > __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(w, m);
+            __threadfence();
+            const uint32_t ticket = atomicAdd(w + 1, 1u);
+            if (ticket == gridDim.x - 1) {
+                __threadfence();
+                const uint32_t mm = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                w[0] = 0u, w[1] = 0u;    // ready for the next call
+                float am = __uint_as_float(mm);
+                if ((qa.flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
+                const float sc = scale_rule(am, guess, qa.fp_max, qa.margin);
+                *qa.amax = am;
+                *qa.scale = sc;
+                *qa.scale_inv = 1.0f / sc;
+                w[2] = __float_as_uint(sc) != __float_as_uint(guess) ? 1u : 0u;    // the codes must be written again
+            }
+        }
+        return;
+    }
     const bool inside = row0 + kDmaTile <= NR && col0 + kDmaTile <= NC;
     // (the per-lane offset of the whole-tile form is 32 bits: four rows of the output)
     if (vec_ok && inside && static_cast<unsigned long long>(NC) * kEsz * 4 < (1ull << 31)) emit_plain(std::true_type{}, std::true_type{});
@@ -981,6 +1103,32 @@ static int launch_gemm_dma_quant(const uint8_t* X, const uint8_t* Y, int NR, int
                                  const QuantArgs& qa, hipStream_t st) {
     if ((K / kBK) & 1) return launch_gemm_dma_quant_parity<XF, YF, OT, XT, YT, QF, true>(X, Y, NR, NC, K, xs, ys, qa, st);
     return launch_gemm_dma_quant_parity<XF, YF, OT, XT, YT, QF, false>(X, Y, NR, NC, K, xs, ys, qa, st);
+}
+
+// the same kernel with the cast to FP8 riding along on speculation (see QSPEC above); the caller has checked the shape
+template <int XF, int YF, typename OT, bool XT, bool YT, bool ODD>
+static int launch_gemm_dma_spec_parity(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                                       const float* ys, int accumulate, const QuantArgs& qa, hipStream_t st) {
+    constexpr int smem = 2 * kDmaStage;
+    static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, 0, ODD, true>;
+    if (!configured.load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel, speculative cast)");
+        configured.store(true, std::memory_order_release);
+    }
+    const int tiles = (NR / kDmaTile) * (NC / kDmaTile);
+    hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys, accumulate,
+                       static_cast<const void*>(nullptr), 0, qa);
+    MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel (speculative cast)");
+    return MSAMP_OK;
+}
+
+template <int XF, int YF, typename OT, bool XT, bool YT>
+static int launch_gemm_dma_spec(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
+                                const float* ys, int accumulate, const QuantArgs& qa, hipStream_t st) {
+    if ((K / kBK) & 1) return launch_gemm_dma_spec_parity<XF, YF, OT, XT, YT, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, qa, st);
+    return launch_gemm_dma_spec_parity<XF, YF, OT, XT, YT, false>(X, Y, D, NR, NC, K, xs, ys, accumulate, qa, st);
 }
 
 template <int BR, int BC, int XF, int YF, typename OT, bool KGUARD>
@@ -1059,11 +1207,29 @@ static int pick_out_quant(const uint8_t* X, const uint8_t* Y, int d_dtype, int N
     }
 }
 
+template <int XF, int YF, bool T>
+static int pick_out_spec(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, int NR, int NC, int K, const float* xs,
+                         const float* ys, int accumulate, const QuantArgs& qa, hipStream_t st) {
+    switch (d_dtype) {
+        case MSAMP_DT_F32:
+            // a float32 product takes the two steps: with four-byte outputs the epilogue that also emits codes does not
+            // fit the vector registers left beside the accumulators
+            return MSAMP_NOT_FUSED;
+        case MSAMP_DT_F16:
+            return launch_gemm_dma_spec<XF, YF, f16_t, T, T>(X, Y, D, NR, NC, K, xs, ys, accumulate, qa, st);
+        default:
+            return launch_gemm_dma_spec<XF, YF, bf16_t, T, T>(X, Y, D, NR, NC, K, xs, ys, accumulate, qa, st);
+    }
+}
 
 // Everything behind the C entry points for one pair of operand formats.  gemm_inst.hip instantiates it once per
 // pair (four translation units, so that they compile side by side).
 template <int XF, int YF>
 int run_gemm_pair(const GemmCall& c) {
+    if (c.qa != nullptr && c.qspec) {
+        if (c.xt) return pick_out_spec<XF, YF, true>(c.X, c.Y, c.D, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, c.accumulate, *c.qa, c.st);
+        return pick_out_spec<XF, YF, false>(c.X, c.Y, c.D, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, c.accumulate, *c.qa, c.st);
+    }
     if (c.qa != nullptr) {
         if (c.xt) return pick_out_quant<XF, YF, true>(c.X, c.Y, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, *c.qa, c.st);
         return pick_out_quant<XF, YF, false>(c.X, c.Y, c.d_dtype, c.NR, c.NC, c.K, c.xs, c.ys, *c.qa, c.st);

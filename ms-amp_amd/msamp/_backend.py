@@ -10,6 +10,7 @@ import ctypes
 import os
 
 import torch
+import torch.distributed as _dist
 
 _LIB_NAME = 'libmsamp_hip.so'
 _LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), 'lib', _LIB_NAME)
@@ -50,7 +51,7 @@ _SIGNATURES = {
     'msamp_cast_transpose_gated': ([_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp], _i),
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
-    'msamp_fp8_gemm_cast': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp], _i),
+    'msamp_fp8_gemm_cast': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp], _i),
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
     'msamp_fp8_norms': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
     'msamp_bucket_amax': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
@@ -134,6 +135,7 @@ ERR_TIMEOUT = -5
 WS_ERROR_BYTE = 32    # byte offset of the sticky error word in a workspace
 _force_two_pass = False
 _pending_error_reads = {}
+_static_workspace_streams = set()    # (device index, raw stream) pairs that ran msamp_cast_to_fp8_intime_static
 
 
 class WaitExpiredError(RuntimeError):
@@ -149,17 +151,27 @@ def check_async_error(block=True):
     in-time cast, the fused GEMM + cast).  Such a failure cannot be seen by the call that enqueued the kernel; the
     kernel leaves a sticky word in the workspace instead.
 
-    block=True reads the word of every workspace of this process now (synchronises their streams' work up to here).
+    block=True reads the word of every workspace of this process now (synchronises their streams' work up to here),
+    including the library's own workspace on every device where cast_to_fp8_intime_static was called.
     block=False never waits: it looks at the copies of the words requested by the previous call -- if they have
     arrived -- and requests new ones, so a training loop that calls it once per step learns of a failure a step or
-    two late without ever synchronising.  Either way a failure raises WaitExpiredError, after switching this
-    process to the two-pass kernels for good (same results, no waiting): the tensors and metas the failed kernel
-    wrote are invalid and the step must be repeated."""
+    two late without ever synchronising (the library's own workspace has no tensor to copy from and is left to the
+    blocking form).  Either way a failure raises WaitExpiredError, after switching this process to the two-pass
+    kernels for good (same results, no waiting).  The tensors and metas the failed kernel wrote are invalid, and so
+    is whatever was computed from them since: go back to the last good state (a checkpoint)."""
     global _force_two_pass
     lib = load()
     failed = None
     if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
         return    # nothing here can be recorded into a graph, and the waiting kernels stay out of captured streams anyway
+    if block:
+        for dev, stream in sorted(_static_workspace_streams):
+            with torch.cuda.device(dev):
+                rc = lib.msamp_check_async_error(None, stream)
+            if rc == ERR_TIMEOUT:
+                failed = lib.msamp_last_error().decode(errors='replace')
+            elif rc != 0:
+                _check(rc, 'msamp_check_async_error')
     for key, ws in list(_workspaces.items()):
         if not ws.is_cuda:
             continue
@@ -187,8 +199,12 @@ def check_async_error(block=True):
             entry['in_flight'] = True
     if failed is not None:
         _force_two_pass = True
-        raise WaitExpiredError(failed + '; the tensors and metas it wrote are invalid. The process now uses the two-pass '
-                               'kernels only: repeat the step.')
+        # copies of the words requested before they were cleared still carry the old code: forget them, so that
+        # the failure is reported once
+        _pending_error_reads.clear()
+        raise WaitExpiredError(failed + '; the tensors and metas it wrote are invalid, and so is everything computed from '
+                               'them since. The process now uses the two-pass kernels only: restore the last good state '
+                               'and go on from there.')
 
 
 def set_spin_limit(polls):
@@ -275,11 +291,25 @@ def cast_to_fp8(x, scale, amax_cell, scale_inv, fp8_dt):
     return out
 
 
+_world_seen = (None, False)
+
+
+def _default_group():
+    """The default process group, or None while torch.distributed is not initialised."""
+    return _dist.GroupMember.WORLD if _dist.is_available() else None
+
+
 def _shared_device():
     """True when other kernels may hold part of the GPU for long (a process group with peers keeps RCCL kernels
-    resident beside the compute stream): kernels whose workgroups wait for each other then stay off."""
-    import torch.distributed as dist
-    return dist.is_available() and dist.is_initialized() and dist.get_world_size() > 1
+    resident beside the compute stream): kernels whose workgroups wait for each other then stay off.  The answer
+    is kept per default process group, so a cast pays one attribute read for it."""
+    global _world_seen
+    world = _default_group()
+    if world is None:
+        return False
+    if world is not _world_seen[0]:
+        _world_seen = (world, _dist.get_world_size() > 1)
+    return _world_seen[1]
 
 
 def cast_to_fp8_intime(x, scale, amax_cell, scale_inv, fp8_dt, margin=0, nan_to_inf=False, two_pass=False, speculate=True):
@@ -312,6 +342,7 @@ def cast_to_fp8_intime_static(x, scale, amax_cell, scale_inv, out, fp8_dt, margi
     _gpu(out, 'output')
     if out.dtype != torch.uint8 or out.numel() != x.numel() or not out.is_contiguous():
         raise ValueError('out must be a contiguous uint8 tensor with as many elements as the input')
+    _static_workspace_streams.add((x.device.index if x.device.index is not None else torch.cuda.current_device(), _stream()))
     _check(
         lib.msamp_cast_to_fp8_intime_static(
             _ptr(x), _dt(x), x.numel(), _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), _ptr(out), fp8_dt, margin,
@@ -482,10 +513,14 @@ NOT_FUSED = 1
 
 
 def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, scale, amax_cell, scale_inv, margin=0,
-                  nan_to_inf=False, a_kmajor=False, b_kmajor=False):
+                  nan_to_inf=False, a_kmajor=False, b_kmajor=False, hp_out=None, accumulate=False, speculate=True):
     """The product of fp8_gemm, rounded to hp_dtype and cast on to FP8 with in-time scaling (amax_cell[0], scale and
-    scale_inv are updated) in one launch.  Returns the uint8 payload [N, M], or None when the fused form does not apply
-    to this problem or stream (nothing has been touched then): take fp8_gemm and cast_to_fp8_intime instead."""
+    scale_inv are updated), without a second trip over the product.  Small problems (at most one tile per compute unit)
+    take one launch and never store the product; any other problem stores it in `hp_out` (allocated here if not given;
+    with `accumulate` it must be given and the product is added to what it holds) together with the codes for the scale in
+    force, and reads it again only when the scale rule arrives at another scale.  Returns the uint8 payload [N, M], or
+    None when neither form applies to this problem (nothing has been touched then): take fp8_gemm and cast_to_fp8_intime
+    instead."""
     lib = load()
     _gpu(a, 'mat_a')
     _gpu(b, 'mat_b')
@@ -495,11 +530,19 @@ def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, sc
         raise ValueError(f'shape mismatch: a {tuple(a.shape)}, b {tuple(b.shape)}')
     if hp_dtype not in _TORCH_TO_DT:
         raise TypeError(f'unsupported intermediate dtype {hp_dtype}')
+    if accumulate and hp_out is None:
+        raise ValueError('accumulate needs hp_out')
+    if hp_out is not None and (hp_out.dtype != hp_dtype or tuple(hp_out.shape) != (n, m) or not hp_out.is_contiguous()):
+        raise ValueError(f'hp_out must be a contiguous {hp_dtype} tensor of shape {(n, m)}')
+    if hp_out is None and speculate and m % 256 == 0 and n % 256 == 0 and (n // 256) * (m // 256) > 0:
+        hp_out = torch.empty(n, m, dtype=hp_dtype, device=a.device)
     out = torch.empty(n, m, dtype=torch.uint8, device=a.device)
     rc = lib.msamp_fp8_gemm_cast(
         _ptr(a), a_dt, _ptr(a_scale_inv), 1 if a_kmajor else 0, _ptr(b), b_dt, _ptr(b_scale_inv), 1 if b_kmajor else 0,
-        _TORCH_TO_DT[hp_dtype], _ptr(out), q_dt, _ptr(scale), _ptr(amax_cell), _ptr(scale_inv), m, n, k, margin,
-        (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _two_pass_only() else 0), _ptr(workspace(a.device)), _stream()
+        _ptr(hp_out), _TORCH_TO_DT[hp_dtype], 1 if accumulate else 0, _ptr(out), q_dt, _ptr(scale), _ptr(amax_cell),
+        _ptr(scale_inv), m, n, k, margin,
+        (FLAG_NAN_TO_INF if nan_to_inf else 0) | (FLAG_TWO_PASS if _two_pass_only() else 0) |
+        (0 if speculate else FLAG_NO_SPECULATION), _ptr(workspace(a.device)), _stream()
     )
     if rc == NOT_FUSED:
         return None

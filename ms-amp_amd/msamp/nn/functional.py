@@ -67,23 +67,29 @@ class _FP8GemmFunction(torch.autograd.Function):
             else:
                 mat_a, mat_b, layout = ctx.input_fp8.fp8_transpose(), ograd_fp8_t, {}
             wgrad = None
-            if ctx.weight.grad is None and not model_state.use_fp8_ddp:
-                # GEMM and cast in one launch where the kernel takes the problem (same bits as the two steps below)
-                wgrad = Gemm.fp8_gemm_cast(mat_a, mat_b, ctx.output_qtype, metas['wgrad'], sync=True, **layout)
+            old_wgrad = None
+            if ctx.weight.grad is not None:
+                # gradient accumulation: add into the dequantized previous gradient
+                old_wgrad = ctx.weight.grad.to(ctx.output_dtype)
+            if not model_state.use_fp8_ddp:
+                # GEMM and cast without reading the product back, where the kernel takes the problem (same bits as the
+                # two steps below)
+                wgrad = Gemm.fp8_gemm_cast(
+                    mat_a, mat_b, ctx.output_qtype, metas['wgrad'], sync=True, accumulate=old_wgrad is not None, out=old_wgrad,
+                    **layout
+                )
             if wgrad is None:
-                if ctx.weight.grad is None:
+                if old_wgrad is None:
                     wgrad = Gemm.fp8_gemm(mat_a, mat_b, ctx.output_qtype, use_split_accumulator=True, **layout)
                 else:
-                    # gradient accumulation: add into the dequantized previous gradient
-                    old_wgrad = ctx.weight.grad.to(ctx.output_dtype)
                     wgrad = Gemm.fp8_gemm(
                         mat_a, mat_b, ctx.output_qtype, accumulate=True, out=old_wgrad, use_split_accumulator=True, **layout
                     )
-                    del old_wgrad
                 if model_state.use_fp8_ddp:
                     wgrad.meta = metas['wgrad']
                 else:
                     wgrad = wgrad.cast(Dtypes.kfloat8_e4m3, meta=metas['wgrad'], sync=True)
+            del old_wgrad
             ctx.weight.backward_grad_update(wgrad)
 
         bias_grad = output_grad.sum(0).to(ctx.bias_dtype) if ctx.need_bias_grad else None

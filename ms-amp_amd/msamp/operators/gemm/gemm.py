@@ -31,21 +31,28 @@ class Gemm:
 
     @classmethod
     @torch.no_grad()
-    def fp8_gemm_cast(cls, mat_a, mat_b, out_qtype, meta, sync=False, a_kmajor=False, b_kmajor=False):
-        """fp8_gemm(mat_a, mat_b, out_qtype).cast(meta.qtype, meta=meta, sync=sync) for a meta with in-time scaling,
-        as one kernel launch (not in the reference, which takes the two steps: nn/functional.py:100-123).  Returns the
-        FP8 ScalingTensor, or None if the fused kernel does not take this problem -- the caller then takes the two
-        steps itself; the result is the same bit for bit."""
+    def fp8_gemm_cast(cls, mat_a, mat_b, out_qtype, meta, sync=False, a_kmajor=False, b_kmajor=False, accumulate=False,
+                      out=None):
+        """fp8_gemm(mat_a, mat_b, out_qtype, accumulate=accumulate, out=out).cast(meta.qtype, meta=meta, sync=sync) for a
+        meta with in-time scaling, without reading the product back (not in the reference, which takes the two steps:
+        nn/functional.py:100-123).  Small products take one launch and are never stored; larger ones are stored in
+        `out` (a scratch tensor if not given) next to the codes for the scale the meta holds, and are read again only
+        when the scale rule moves the scale.  Returns the FP8 ScalingTensor, or None if the kernel does not take this
+        problem -- the caller then takes the two steps itself; the result is the same bit for bit."""
         assert isinstance(mat_a, ScalingTensor) and isinstance(mat_b, ScalingTensor)
         assert mat_a.is_cuda and mat_a.is_contiguous() and mat_b.is_cuda and mat_b.is_contiguous()
         assert Dtypes.is_fp8_qtype(mat_a.qtype) and Dtypes.is_fp8_qtype(mat_b.qtype) and Dtypes.is_fp8_qtype(meta.qtype)
         if meta.scaling_mode() != 'in_time' or (a_kmajor != b_kmajor):
             return None
+        out_dtype = Dtypes.get_dtype_from_qtype(out_qtype)
+        if out is not None:
+            assert out.is_cuda and out.is_contiguous() and out.dtype == out_dtype
+        else:
+            assert not accumulate, 'accumulate needs an output tensor'
         payload = _backend.fp8_gemm_cast(
             cls._aligned(mat_a.value), int(mat_a.qtype), mat_a.meta.scale_inv, cls._aligned(mat_b.value), int(mat_b.qtype),
-            mat_b.meta.scale_inv,
-            Dtypes.get_dtype_from_qtype(out_qtype), int(meta.qtype), meta.scale, meta.amax[0:1], meta.scale_inv,
-            nan_to_inf=sync, a_kmajor=a_kmajor, b_kmajor=b_kmajor
+            mat_b.meta.scale_inv, out_dtype, int(meta.qtype), meta.scale, meta.amax[0:1], meta.scale_inv,
+            nan_to_inf=sync, a_kmajor=a_kmajor, b_kmajor=b_kmajor, hp_out=out, accumulate=accumulate
         )
         return None if payload is None else ScalingTensor(payload, meta)
 

@@ -294,6 +294,49 @@ def test_llama_layer_shapes_sampled(be, tokens, d_out, d_in):
     assert rel_fro(dw[cols.cuda()][:, cin.cuda()], want) < TOL_F32
 
 
+def _strip(n):
+    """One index per block of 256 (one per tile of the kernel), at an offset that moves through the tile: whole rows and
+    columns of the output at these indices pass through every tile, every wave quadrant and every 16-row block."""
+    return torch.tensor([min(256 * i + (37 * i + 5) % 256, n - 1) for i in range((n + 255) // 256)])
+
+
+@pytest.mark.parametrize('tokens,d_out,d_in', [(16384, 11008, 4096), (16384, 4096, 11008), (16384, 12288, 4096),
+                                               (16384, 4096, 4096), (16384, 8192, 28672), (16384, 10240, 8192),
+                                               (16384, 28672, 8192), (16384, 8192, 8192)])
+def test_llama_layer_shapes_whole_rows_and_columns(be, tokens, d_out, d_in):
+    """The same 24 GEMMs, each checked on whole output rows and whole output columns -- one row through every row of
+    tiles, one column through every column of tiles, so every tile and each of its four wave quadrants is crossed --
+    against a float32 matmul on the CPU of the operands as torch's own float8 types decode them."""
+    x = _gpu_codes((tokens, d_in), 5, 11)
+    w = _gpu_codes((d_out, d_in), 5, 12)
+    dy = _gpu_codes((tokens, d_out), 6, 13)
+    xs, ws, dys = 2.0**-7, 2.0**-9, 2.0**-14
+    one = lambda v: torch.tensor(v, device='cuda')
+    xf = (x.view(torch.float8_e4m3fn).float() * xs).cpu()
+    wf = (w.view(torch.float8_e4m3fn).float() * ws).cpu()
+    dyf = (dy.view(torch.float8_e5m2).float() * dys).cpu()
+    rt, ro, ri = _strip(tokens), _strip(d_out), _strip(d_in)
+
+    def check(out, want_rows, r, want_cols, c, tol):
+        assert rel_fro(out[r.cuda()].float().cpu(), want_rows) < tol
+        assert rel_fro(out[:, c.cuda()].float().cpu(), want_cols) < tol
+        # and nothing in the strips is far off on its own (a slip confined to a few elements hides in a norm)
+        scale = want_rows.abs().max().item()
+        assert (out[r.cuda()].float().cpu() - want_rows).abs().max().item() < 0.05 * scale
+
+    y = torch.empty(tokens, d_out, dtype=torch.bfloat16, device='cuda')
+    be.fp8_gemm(w, 5, one(ws), x, 5, one(xs), y)
+    check(y, xf[rt] @ wf.t(), rt, xf @ wf[ro].t(), ro, TOL_16)
+    del y
+    dx = torch.empty(tokens, d_in, dtype=torch.bfloat16, device='cuda')
+    be.fp8_gemm(w, 5, one(ws), dy, 6, one(dys), dx, a_kmajor=True)
+    check(dx, dyf[rt] @ wf, rt, dyf @ wf[:, ri], ri, TOL_16)
+    del dx
+    dw = torch.empty(d_out, d_in, dtype=torch.float32, device='cuda')
+    be.fp8_gemm(x, 5, one(xs), dy, 6, one(dys), dw, a_kmajor=True, b_kmajor=True)
+    check(dw, dyf[:, ro].t() @ xf, ro, dyf.t() @ xf[:, ri], ri, TOL_F32)
+
+
 def test_operand_beyond_4_gib(be):
     """An operand of 70 016 x 65 536 bytes (4.6 GB): its 32-bit byte offsets would wrap, so the library has to route
     it to the kernel with 64-bit addressing.  Rows below and above the 4 GiB mark against the oracle."""
@@ -363,7 +406,7 @@ def test_gemm_with_fused_cast_special_values(be, nan_to_inf, poison):
 
 
 def test_gemm_with_fused_cast_declines_what_it_cannot_take(be):
-    """Ragged shapes, mixed layouts, more tiles than compute units, a capturing stream: None, and nothing written."""
+    """Ragged shapes, mixed layouts, more tiles than compute units without speculation: None, and nothing written."""
     one = torch.ones((), device='cuda')
 
     def call(m, n, k, **kw):
@@ -378,12 +421,114 @@ def test_gemm_with_fused_cast_declines_what_it_cannot_take(be):
     assert call(256, 256, 128) == (None, 2.0, 3.0, 5.0)    # a single slice of K
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     side = 256 * (int(cus ** 0.5) + 1)
-    assert call(side, side, 256) == (None, 2.0, 3.0, 5.0)
+    assert call(side, side, 256, speculate=False) == (None, 2.0, 3.0, 5.0)    # more tiles than compute units wait for nobody
     assert call(256, 256, 256, q_dt=6) == (None, 2.0, 3.0, 5.0)
     assert call(256, 256, 256, a_kmajor=True) == (None, 2.0, 3.0, 5.0)    # mixed layouts
     for layout in (dict(), dict(a_kmajor=True, b_kmajor=True)):
         got, *_ = call(256, 256, 256, **layout)
         assert got is not None
+
+
+def _spec_case(be, a, a_dt, sa, b, b_dt, sb, hp, kmajor, meta, old=None):
+    """One call of the speculative form on `meta` = (scale, scale_inv, amax) against the two steps from the same meta
+    values; returns the codes.  `old`: previous gradient to accumulate into."""
+    k, m = a.shape if kmajor else a.shape[::-1]
+    n = b.shape[1] if kmajor else b.shape[0]
+    s, si, am = meta
+    s2, si2, am2 = s.clone(), si.clone(), am.clone()
+    d2 = old.clone() if old is not None else torch.empty(n, m, dtype=hp, device='cuda')
+    be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, d2, accumulate=old is not None, a_kmajor=kmajor, b_kmajor=kmajor)
+    want = be.cast_to_fp8_intime(d2, s2, am2, si2, 5, nan_to_inf=True, two_pass=True, speculate=False)
+    d = old.clone() if old is not None else torch.full((n, m), float('nan'), dtype=hp, device='cuda')
+    got = be.fp8_gemm_cast(a, a_dt, sa, b, b_dt, sb, hp, 5, s, am, si, nan_to_inf=True, a_kmajor=kmajor, b_kmajor=kmajor,
+                           hp_out=d, accumulate=old is not None)
+    assert got is not None, 'the speculative form should take this problem'
+    assert torch.equal(d.view(torch.int16), d2.view(torch.int16)), 'the stored product differs from the plain GEMM'
+    assert torch.equal(got, want)
+    assert same_float(am, am2) and same_float(s, s2) and same_float(si, si2)
+    return got
+
+
+@pytest.mark.parametrize('a_dt,b_dt', [(5, 6), (5, 5)])
+@pytest.mark.parametrize('m,n,k', [(4352, 4096, 256), (4096, 11008, 384), (8192, 28672, 256), (512, 256, 640)])
+@pytest.mark.parametrize('hp', [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('kmajor', [True, False])
+def test_gemm_with_speculative_cast_matches_the_two_steps(be, a_dt, b_dt, m, n, k, hp, kmajor):
+    """More output tiles than compute units (272, 688 and 3584 tiles; the small case is sent the same way by keeping
+    the waiting kernels off): the GEMM stores the product and, beside it, the codes for the scale the meta holds.  A
+    fresh meta (scale 1: the rule moves it, the product is cast again), the same operands again (the scale stands:
+    nothing is read back), operands four times larger (the scale moves again), then accumulation into the previous
+    product: codes, amax, scale, scale_inv and the stored product equal the two steps, bit for bit, every time."""
+    a = _gpu_codes((k, m) if kmajor else (m, k), a_dt, 3 * m + k)
+    b = _gpu_codes((k, n) if kmajor else (n, k), b_dt, 5 * n + k)
+    # (the codes are uniformly random, E5M2 ones reach 14336: factors that keep the float16 products finite)
+    sa, sb = (torch.tensor(v, device='cuda') for v in ((0.125, 0.5) if hp == torch.bfloat16 else (2.0 ** -12, 2.0 ** -10)))
+    meta = (torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda'))
+    small = (m // 256) * (n // 256) <= torch.cuda.get_device_properties(0).multi_processor_count
+    saved = be._force_two_pass
+    be._force_two_pass = be._force_two_pass or small
+    try:
+        _spec_case(be, a, a_dt, sa, b, b_dt, sb, hp, kmajor, meta)
+        first_scale = meta[0].clone()
+        assert float(first_scale) != 1.0
+        _spec_case(be, a, a_dt, sa, b, b_dt, sb, hp, kmajor, meta)
+        assert same_float(meta[0], first_scale)
+        _spec_case(be, a, a_dt, sa * 4, b, b_dt, sb, hp, kmajor, meta)
+        assert float(meta[0]) == float(first_scale) / 4
+        g = torch.Generator(device='cuda').manual_seed(m + n)
+        old = (torch.randn(n, m, device='cuda', generator=g) * float(meta[2][0]) * 0.3).to(hp)
+        _spec_case(be, a, a_dt, sa * 4, b, b_dt, sb, hp, kmajor, meta, old=old)
+    finally:
+        be._force_two_pass = saved
+
+
+@pytest.mark.parametrize('poison', ['nan', 'inf', 'zero'])
+def test_gemm_with_speculative_cast_special_values(be, poison):
+    """A NaN or an Inf in the product, or an all-zero product, through the speculative form (272 tiles)."""
+    m, n, k = 4352, 4096, 256
+    a = _gpu_codes((k, m), 6, 1)
+    b = _gpu_codes((k, n), 6, 2)
+    if poison == 'nan':
+        a[7, 5] = 0x7f
+    elif poison == 'inf':
+        a[7, 5] = 0x7c
+    else:
+        a.zero_()
+    one = torch.ones((), device='cuda')
+    meta = (torch.full((), 4.0, device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda'))
+    _spec_case(be, a, 6, one, b, 6, one, torch.bfloat16, True, meta)
+    _spec_case(be, a, 6, one, b, 6, one, torch.bfloat16, True, meta)
+
+
+def test_gemm_with_speculative_cast_replays_from_a_graph(be):
+    """The speculative form waits for nobody and takes its decisions on the GPU, so it can be captured: replays over
+    operands whose scale stands and whose scale moves, each against the eager two steps, with eager work in between."""
+    m, n, k = 4352, 4096, 256
+    a = _gpu_codes((k, m), 5, 11)
+    b = _gpu_codes((k, n), 6, 12)
+    sb = torch.tensor(0.5, device='cuda')
+    sa = torch.tensor(0.125, device='cuda')
+    s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+    d = torch.empty(n, m, dtype=torch.bfloat16, device='cuda')
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        be.fp8_gemm_cast(a, 5, sa, b, 6, sb, torch.bfloat16, 5, s, am, si, nan_to_inf=True, a_kmajor=True, b_kmajor=True, hp_out=d)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        q = be.fp8_gemm_cast(a, 5, sa, b, 6, sb, torch.bfloat16, 5, s, am, si, nan_to_inf=True, a_kmajor=True, b_kmajor=True, hp_out=d)
+    assert q is not None
+    for factor in (0.125, 0.125, 1.0, 1.0, 0.03125, 0.125):
+        sa.fill_(factor)
+        s0, si0, am0 = s.clone(), si.clone(), am.clone()
+        graph.replay()
+        d2 = be.fp8_gemm(a, 5, sa, b, 6, sb, torch.empty_like(d), a_kmajor=True, b_kmajor=True)
+        want = be.cast_to_fp8_intime(d2, s0, am0, si0, 5, nan_to_inf=True, two_pass=True, speculate=False)
+        torch.cuda.synchronize()
+        assert torch.equal(q, want) and torch.equal(d.view(torch.int16), d2.view(torch.int16)), factor
+        assert same_float(am, am0) and same_float(s, s0) and same_float(si, si0), factor
 
 
 def test_fp8linear_weight_gradient_uses_the_fused_kernel_and_matches():

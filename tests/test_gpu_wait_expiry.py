@@ -98,3 +98,49 @@ def test_expired_wait_of_the_fused_gemm_cast_is_reported(be):
     q2 = be.cast_to_fp8_intime(d, s2, am2[0:1], si2, be.DT_E4M3, two_pass=True)
     assert q1 is not None and torch.equal(q1, q2) and same_float(am1, am2) and same_float(s1, s2)
     assert lib.msamp_check_async_error(ws.data_ptr(), stream) == 0
+
+
+def test_waiting_kernels_follow_the_stream_that_is_in_use(be):
+    """The one-pass kernels are kept to one stream per device at a time, but a stream that has gone idle does not
+    keep them: after a warm-up on a side stream the main stream gets them back (seen through the spin limit of zero,
+    which only a one-pass kernel reacts to)."""
+    x = torch.randn(2 * 1024 * 1024, device='cuda')
+
+    def one_pass_ran():
+        s, si, am = make_meta(scale=4.0)
+        be.set_spin_limit(0)
+        try:
+            be.cast_to_fp8_intime(x, s, am[0:1], si, be.DT_E4M3)
+            torch.cuda.synchronize()
+        finally:
+            be.set_spin_limit(1 << 20)
+        gave_up = bool(torch.isnan(am[0]).item())
+        if gave_up:
+            with pytest.raises(be.WaitExpiredError):
+                be.check_async_error(block=True)
+            be._force_two_pass = False
+        return gave_up
+
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        assert one_pass_ran()        # the side stream takes the device over from the idle main stream
+    assert one_pass_ran()            # and the main stream takes it back once the side stream is idle
+    with torch.cuda.stream(side):
+        # while the main stream is busy the side stream is refused and takes the two-pass kernels: right bytes, no NaN
+        big = torch.randn(64 * 1024 * 1024, device='cuda')
+        torch.cuda.current_stream().wait_stream(torch.cuda.default_stream())
+    s0, si0, am0 = make_meta()
+    for _ in range(40):
+        be.cast_to_fp8_intime(big, s0, am0[0:1], si0, be.DT_E4M3)    # main stream: busy for a few milliseconds
+    with torch.cuda.stream(side):
+        s, si, am = make_meta(scale=4.0)
+        be.set_spin_limit(0)
+        try:
+            be.cast_to_fp8_intime(x, s, am[0:1], si, be.DT_E4M3)
+        finally:
+            be.set_spin_limit(1 << 20)
+        side.synchronize()
+        assert not torch.isnan(am[0]).item()
+    torch.cuda.synchronize()
+    be.check_async_error(block=True)

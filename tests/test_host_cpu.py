@@ -226,14 +226,19 @@ def test_scale_group_layout_matches_header():
 
 
 def test_one_pass_kernels_stay_off_under_a_process_group(monkeypatch):
-    """Kernels whose workgroups wait for each other are only asked for when no other rank exists."""
+    """Kernels whose workgroups wait for each other are only asked for when no other rank exists; the answer is kept
+    per default process group."""
     import torch.distributed as dist
     from msamp import _backend
     assert _backend._shared_device() is False
-    monkeypatch.setattr(dist, 'is_initialized', lambda: True)
+    monkeypatch.setattr(_backend, '_default_group', lambda group=object(): group)
     monkeypatch.setattr(dist, 'get_world_size', lambda group=None: 2)
     assert _backend._shared_device() is True
     monkeypatch.setattr(dist, 'get_world_size', lambda group=None: 1)
+    assert _backend._shared_device() is True    # same group: not asked again
+    monkeypatch.setattr(_backend, '_default_group', lambda group=object(): group)    # another group: asked again
+    assert _backend._shared_device() is False
+    monkeypatch.setattr(_backend, '_default_group', lambda: None)
     assert _backend._shared_device() is False
 
 
@@ -249,23 +254,42 @@ def test_chunk_map_rows_and_cache():
     assert _backend.chunk_map([], 'cpu').shape[0] == 0
 
 
-def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(tmp_path):
-    """The accumulators of fp8_gemm_dma_kernel live in fixed AGPRs behind the compiler's back (inline-assembly MFMAs).
-    That holds only while the compiler itself uses no AGPR in those kernels (it would, to spill VGPRs) and no scratch
-    memory: compile the kernels of one format pair to assembly and look.  Cross-compiles without a GPU."""
+GEMM_PAIRS = ((5, 5), (5, 6), (6, 5), (6, 6))    # the four translation units of the Makefile: E4M3 / E5M2 operands
+
+
+@pytest.fixture(scope='module')
+def gemm_assembly(tmp_path_factory):
+    """The GEMM kernels of every operand-format pair compiled to assembly, side by side (cross-compiles without a GPU)."""
     import shutil
     import subprocess
     hipcc = shutil.which('hipcc') or '/opt/rocm/bin/hipcc'
     if not os.path.exists(hipcc):
         pytest.skip('no hipcc here')
     src = os.path.join(os.path.dirname(_backend.__file__), '..', 'csrc')
-    out = str(tmp_path / 'gemm_inst.s')
-    cmd = [hipcc, '--offload-arch=gfx950', '-O3', '-std=c++17', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
-           '-Wno-unused-command-line-argument', '-Wno-inline-asm', '-DMSAMP_XF=5', '-DMSAMP_YF=5', '--cuda-device-only', '-S',
-           '-o', out, os.path.join(src, 'gemm_inst.hip')]
-    subprocess.run(cmd, check=True, capture_output=True, cwd=src)
+    tmp = tmp_path_factory.mktemp('gemm_asm')
+    procs = {}
+    for xf, yf in GEMM_PAIRS:
+        out = str(tmp / f'gemm_inst_{xf}{yf}.s')
+        cmd = [hipcc, '--offload-arch=gfx950', '-O3', '-std=c++17', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+               '-Wno-unused-command-line-argument', '-Wno-inline-asm', f'-DMSAMP_XF={xf}', f'-DMSAMP_YF={yf}',
+               '--cuda-device-only', '-S', '-o', out, os.path.join(src, 'gemm_inst.hip')]
+        procs[(xf, yf)] = (out, subprocess.Popen(cmd, cwd=src, stdout=subprocess.PIPE, stderr=subprocess.STDOUT))
+    paths = {}
+    for pair, (out, proc) in procs.items():
+        log = proc.communicate()[0]
+        assert proc.returncode == 0, log.decode(errors='replace')[-2000:]
+        paths[pair] = out
+    return paths
+
+
+@pytest.mark.parametrize('pair', GEMM_PAIRS)
+def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(gemm_assembly, pair):
+    """The accumulators of fp8_gemm_dma_kernel live in fixed AGPRs behind the compiler's back (inline-assembly MFMAs).
+    That holds only while the compiler itself uses no AGPR in those kernels (it would, to spill VGPRs) and no scratch
+    memory.  Each pair of operand formats is a translation unit of its own with its own register allocation: look at
+    the assembly of all four."""
     kernel, in_asm, found = None, False, {}
-    for line in open(out):
+    for line in open(gemm_assembly[pair]):
         m = re.match(r'^(_Z\w+):', line)
         if m:
             kernel = m.group(1)
@@ -279,6 +303,7 @@ def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(tmp_pa
                 c[0 if in_asm else 1] += 1
             if re.search(r'scratch_(load|store)', line):
                 c[2] += 1
-    assert len(found) >= 10    # bf16 / f16 / float outputs, row- and K-major operands, both parities, the fused cast
+    # bf16 / f16 / float outputs, row- and K-major operands, both parities, the fused and the speculative cast
+    assert len(found) >= 40
     for name, (ours, compilers, scratch) in found.items():
         assert ours >= 512 and compilers == 0 and scratch == 0, (name, ours, compilers, scratch)

@@ -70,3 +70,29 @@ def test_static_workspace_rejects_oversize_and_bad_arguments(be):
                                                be.DT_E4M3, 0, 0, None) == -3
     assert lib.msamp_cast_to_fp8_intime_static(*args(0)) == 0
     torch.cuda.synchronize()
+
+
+def test_static_workspace_reports_a_wait_that_ran_out(be):
+    """With the spin limit forced to zero every wait of the one-pass kernel gives up at once (every kernel still runs
+    to its end); the sticky word then sits in the library's own workspace, which a null workspace pointer stands for."""
+    lib = be.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.msamp_check_async_error(None, stream) == 0
+    x = torch.randn(3 * 1024 * 1024 + 11, device='cuda')
+    s, si, am = _meta()
+    out = torch.empty(x.numel(), dtype=torch.uint8, device='cuda')
+    be.set_spin_limit(0)
+    try:
+        be.cast_to_fp8_intime_static(x, s, am, si, out, be.DT_E4M3)
+        torch.cuda.synchronize()
+    finally:
+        be.set_spin_limit(1 << 20)
+    assert torch.isnan(am[0]).item() and s.item() == 3.0
+    try:
+        with pytest.raises(be.WaitExpiredError):
+            be.check_async_error(block=True)
+        assert be._force_two_pass
+    finally:
+        be._force_two_pass = False
+    assert lib.msamp_check_async_error(None, stream) == 0    # reported once, then clear
+    _pair(be, x, be.DT_E4M3, False)    # and the static array is as good as before
