@@ -373,6 +373,30 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
                                       double weight_decay, int step, int bias_correction, int adam_mode, int maximize,
                                       int tensor_scale, msamp_stream_t stream);
 
+/* The one-pass step of msamp_adamw_fp8_fused_speculative without the second set of buffers (not in the reference,
+ * whose optimizer is LBAdamW.adamw_fn, adamw.py:148-199).  The caller keeps the payloads of all n_tensors tensors
+ * back to back, in the order of `block_map`, each padded to whole chunks of MSAMP_ADAMW_CHUNK elements, in three arenas
+ * (weights, exp_avg, exp_avg_sq) that have |shift_elems| elements of room at one end; the descriptors point at the
+ * payloads where they are now.  The call writes every tensor's new payloads shift_elems elements away from the old
+ * ones (the same element offset in all three arenas): with a negative shift it walks the chunks front to back, with a
+ * positive one back to front, so that the room is always ahead of the walk, and it sees to it that a chunk is
+ * overwritten only once its tensor's scales are known and, where they came out different from the ones used, the
+ * chunk has been done again from its inputs.  The caller alternates the sign from step to step (with descriptors that
+ * point at the new places).  No tensor may have more chunks than the room holds (sticky error word otherwise, see
+ * below); for the workgroups never to wait for each other in practice, make the room a few thousand chunks larger
+ * than the largest tensor.  Results, metas and `redo` as for msamp_adamw_fp8_fused_speculative: the same bits that
+ * msamp_adamw_fp8_fused leaves in place.  `posts`: DEVICE array of MSAMP_ADAMW_POST_WORDS 8-byte words per tensor,
+ * zeroed once by the caller, through which the workgroups of a call tell each other how a tensor came out.  The
+ * descriptors' acc and reserved words must be zero before the first call (the library leaves them at zero).  `workspace`: the MSAMP_WORKSPACE_BYTES buffer of the other entry points; a wait that
+ * runs out (msamp_set_spin_limit) or a layout that breaks the rule above sets its sticky error word, reported by
+ * msamp_check_async_error: the state is then partly updated and must be restored from a copy. */
+#define MSAMP_ADAMW_POST_WORDS 8
+int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, uint64_t* posts, int n_tensors,
+                                const int32_t* block_map, int n_blocks, long long shift_elems, int weight_dtype, int grad_dtype,
+                                double lr, double beta1,
+                                double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
+                                int maximize, int tensor_scale, void* workspace, msamp_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

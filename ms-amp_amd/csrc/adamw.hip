@@ -319,31 +319,54 @@ __global__ void fused_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, 
     *d.v_amax = av;
 }
 
-template <int WDT>
+// Stores of the fused kernels' outputs.  THRU: written through to where every compute unit of the GPU sees them (the
+// `sc1` stores that an agent-scope atomic store is made of), which the shifting step needs: there a chunk may be
+// written twice, by workgroups on different dies with an L2 each, and a line left dirty in one of them would be
+// written back over the later store.  The stores are assembly because no builtin makes a 16-byte one; the kernel
+// waits for them by hand (s_waitcnt) where their completion matters.
+template <bool THRU>
+__device__ __forceinline__ void put16(void* p, const uint4& v) {
+    if constexpr (THRU) {
+        typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+        const v4u_t vv = {v.x, v.y, v.z, v.w};
+        // (the wait states after it: a store of more than 8 bytes reads its data registers over several cycles, and the
+        // compiler, which does not know this is one, would not keep the next instruction off them)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(vv) : "memory");
+    } else {
+        *static_cast<uint4*>(p) = v;
+    }
+}
+template <bool THRU, typename T>
+__device__ __forceinline__ void put1(T* p, T v) {
+    if constexpr (THRU) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
+template <int WDT, bool THRU = false>
 __device__ __forceinline__ void store_w16(void* base, size_t i, const float* f) {
     if constexpr (WDT == MSAMP_DT_F16) {
         uint32_t w[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) w[j] = float_to_f16_bits(f[2 * j]) | (float_to_f16_bits(f[2 * j + 1]) << 16);
         uint4* p = reinterpret_cast<uint4*>(static_cast<uint16_t*>(base) + i);
-        p[0] = make_uint4(w[0], w[1], w[2], w[3]);
-        p[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        put16<THRU>(p, make_uint4(w[0], w[1], w[2], w[3]));
+        put16<THRU>(p + 1, make_uint4(w[4], w[5], w[6], w[7]));
     } else {
         uint4 o;
         o.x = quant4<WDT>(f[0], f[1], f[2], f[3]);
         o.y = quant4<WDT>(f[4], f[5], f[6], f[7]);
         o.z = quant4<WDT>(f[8], f[9], f[10], f[11]);
         o.w = quant4<WDT>(f[12], f[13], f[14], f[15]);
-        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(base) + i) = o;
+        put16<THRU>(static_cast<uint8_t*>(base) + i, o);
     }
 }
 
-template <int WDT>
+template <int WDT, bool THRU = false>
 __device__ __forceinline__ void store_w1(void* base, size_t i, float f) {
     if constexpr (WDT == MSAMP_DT_F16) {
-        static_cast<uint16_t*>(base)[i] = static_cast<uint16_t>(float_to_f16_bits(f));
+        put1<THRU>(static_cast<uint16_t*>(base) + i, static_cast<uint16_t>(float_to_f16_bits(f)));
     } else {
-        static_cast<uint8_t*>(base)[i] = static_cast<uint8_t>(quant1<WDT>(f));
+        put1<THRU>(static_cast<uint8_t*>(base) + i, static_cast<uint8_t>(quant1<WDT>(f)));
     }
 }
 
@@ -359,7 +382,7 @@ __device__ __forceinline__ uint32_t quant_weight_exact(float pj, float m_new, fl
 }
 
 // One lane's 16 elements of the second pass: requantized weight, exp_avg and exp_avg_sq are stored at element i.
-template <int WDT, bool L2>
+template <int WDT, bool L2, bool THRU = false>
 __device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i, float* p, const float* g,
                                            float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
                                            float ms, float vs, const AdamConsts& k) {
@@ -390,18 +413,51 @@ __device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t
     }
     if constexpr (WDT == MSAMP_DT_F16) {
         uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
-        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
-        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
+        put16<THRU>(o, make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16)));
+        put16<THRU>(o + 1, make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16)));
     } else {
         uint4 o;
         o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
         o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
         o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
+        put16<THRU>(static_cast<uint8_t*>(w_out) + i, o);
     }
-    store_w16<MSAMP_DT_E4M3>(m_out, i, m);
-    store_w16<MSAMP_DT_F16>(v_out, i, v);
+    store_w16<MSAMP_DT_E4M3, THRU>(m_out, i, m);
+    store_w16<MSAMP_DT_F16, THRU>(v_out, i, v);
+}
+
+// Second pass: recompute m', v' exactly and requantize them; for the weight, quantize both ends of the
+// estimate's error interval -- when they give the same code (rounding is monotonic) that code is the
+// exact answer, otherwise (or for anything non-finite) the element takes the exact chain.
+// One chunk of the second pass: the tensor's inputs at d.weight / d.grad / d.exp_avg / d.exp_avg_sq, requantized with
+// the given scales into w_out / m_out / v_out (which may be the inputs' own places).
+template <int WDT, int GDT, bool L2, bool THRU = false>
+__device__ __forceinline__ void write_chunk(const msamp_adamw_tensor& d, int chunk, void* w_out, uint8_t* m_out, uint16_t* v_out,
+                                            float w_si, float g_si, float inv_m, float inv_v, float ws, float ms, float vs,
+                                            const AdamConsts& k) {
+    const size_t n = d.numel;
+    const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
+    if (base + MSAMP_ADAMW_CHUNK <= n) {
+#pragma unroll 1
+        for (int s = 0; s < kSteps; ++s) {
+            const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
+            float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
+            load16<WDT, GDT>(d, i, p, g, m, v);
+            write_step<WDT, L2, THRU>(w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
+        }
+    } else {
+        for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
+            const float m_old = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v_old = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
+            float pj, g_plain, m_new, v_new;
+            prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
+                    g_plain, m_new, v_new);
+            store_w1<WDT, THRU>(w_out, i, param_update(pj, m_new, v_new, k) * ws);
+            if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
+            store_w1<MSAMP_DT_E4M3, THRU>(m_out, i, m_new * ms);
+            store_w1<MSAMP_DT_F16, THRU>(v_out, i, v_new * vs);
+        }
+    }
 }
 
 // Second pass: recompute m', v' exactly and requantize them; for the weight, quantize both ends of the
@@ -422,30 +478,9 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
     void* w_out = outs ? outs[t].weight : d.weight;
     uint8_t* m_out = outs ? outs[t].exp_avg : d.exp_avg;
     uint16_t* v_out = outs ? outs[t].exp_avg_sq : d.exp_avg_sq;
-    const size_t n = d.numel;
-    const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
     const float w_si = d.saved[0], g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv, inv_m = d.saved[1], inv_v = d.saved[2];
     const float ws = *d.w_scale, ms = *d.m_scale, vs = *d.v_scale;
-    if (base + MSAMP_ADAMW_CHUNK <= n) {
-#pragma unroll 1
-        for (int s = 0; s < kSteps; ++s) {
-            const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
-            float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
-            load16<WDT, GDT>(d, i, p, g, m, v);
-            write_step<WDT, L2>(w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
-        }
-    } else {
-        for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
-            const float m_old = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v_old = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
-            float pj, g_plain, m_new, v_new;
-            prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
-                    g_plain, m_new, v_new);
-            store_w1<WDT>(w_out, i, param_update(pj, m_new, v_new, k) * ws);
-            if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
-            store_w1<MSAMP_DT_E4M3>(m_out, i, m_new * ms);
-            store_w1<MSAMP_DT_F16>(v_out, i, v_new * vs);
-        }
-    }
+    write_chunk<WDT, GDT, L2>(d, chunk, w_out, m_out, v_out, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
 }
 
 // ---- speculative single pass -------------------------------------------------------------------
@@ -459,7 +494,7 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
 // |p_est| - err <= |p'| <= |p_est| + err; only elements whose upper end reaches the best lower end seen so far are
 // evaluated exactly, and the element that attains the maximum always is.  Elements that took the exact chain for
 // their code (an estimate too close to a rounding boundary, anything non-finite) have their exact |p'| already.
-template <int WDT, int GDT, bool L2>
+template <int WDT, int GDT, bool L2, bool THRU = false>
 __device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i,
                                           float* p, const float* g,
                                           float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
@@ -512,18 +547,18 @@ __device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_o
     }
     if constexpr (WDT == MSAMP_DT_F16) {
         uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
-        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
-        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
+        put16<THRU>(o, make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16)));
+        put16<THRU>(o + 1, make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16)));
     } else {
         uint4 o;
         o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
         o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
         o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
+        put16<THRU>(static_cast<uint8_t*>(w_out) + i, o);
     }
-    store_w16<MSAMP_DT_E4M3>(m_out, i, m);
-    store_w16<MSAMP_DT_F16>(v_out, i, v);
+    store_w16<MSAMP_DT_E4M3, THRU>(m_out, i, m);
+    store_w16<MSAMP_DT_F16, THRU>(v_out, i, v);
     floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
     const float skip_below = floor_p * 0.999999f;    // room for the roundings of the bounds themselves
     if (hi_max >= skip_below) {    // few lanes get here: the ones that hold an element next to the maximum
@@ -542,16 +577,11 @@ __device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_o
     }
 }
 
-template <int WDT, int GDT, bool L2>
-__global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_tensor* __restrict__ tensors,
-                                                                   const int32_t* __restrict__ block_map, AdamConsts k,
-                                                                   const msamp_adamw_buffers* __restrict__ outs) {
-    __shared__ uint32_t red[kAdamThreads / kWave];
-    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
-    msamp_adamw_tensor& d = tensors[t];
-    void* w_out = outs[t].weight;
-    uint8_t* m_out = outs[t].exp_avg;
-    uint16_t* v_out = outs[t].exp_avg_sq;
+// One chunk of the speculative pass: outputs quantized with the scales in force, the chunk's three maxima handed back
+// (valid in the workgroup's first lane).
+template <int WDT, int GDT, bool L2, bool THRU = false>
+__device__ __forceinline__ void spec_chunk(msamp_adamw_tensor& d, int chunk, void* w_out, uint8_t* m_out, uint16_t* v_out,
+                                           const AdamConsts& k, uint32_t* red, uint32_t& max_p, uint32_t& max_m, uint32_t& max_v) {
     const size_t n = d.numel;
     const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
     const float w_si = *d.w_scale_inv, g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv;
@@ -567,8 +597,8 @@ __global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_te
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            spec_step<WDT, GDT, L2>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p, mxp,
-                               mxm, mxv);
+            spec_step<WDT, GDT, L2, THRU>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p,
+                                          mxp, mxm, mxv);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
@@ -581,20 +611,218 @@ __global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_te
             mxp = ab > mxp ? ab : mxp;
             mxm = fmaxf(mxm, fabsf(m_new));
             mxv = fmaxf(mxv, fabsf(v_new));
-            store_w1<WDT>(w_out, i, pn * ws);
+            store_w1<WDT, THRU>(w_out, i, pn * ws);
             if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
-            store_w1<MSAMP_DT_E4M3>(m_out, i, m_new * ms);
-            store_w1<MSAMP_DT_F16>(v_out, i, v_new * vs);
+            store_w1<MSAMP_DT_E4M3, THRU>(m_out, i, m_new * ms);
+            store_w1<MSAMP_DT_F16, THRU>(v_out, i, v_new * vs);
         }
     }
-    const uint32_t a = block_max_u32(mxp, red);
-    const uint32_t b = block_max_u32(__float_as_uint(mxm), red);
-    const uint32_t c = block_max_u32(__float_as_uint(mxv), red);
+    // THRU: every wave's stores have arrived before the workgroup's barrier, hence before anything its first lane
+    // publishes afterwards
+    if constexpr (THRU) __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0)
+    max_p = block_max_u32(mxp, red);
+    max_m = block_max_u32(__float_as_uint(mxm), red);
+    max_v = block_max_u32(__float_as_uint(mxv), red);
+}
+
+template <int WDT, int GDT, bool L2>
+__global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_tensor* __restrict__ tensors,
+                                                                   const int32_t* __restrict__ block_map, AdamConsts k,
+                                                                   const msamp_adamw_buffers* __restrict__ outs) {
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
+    msamp_adamw_tensor& d = tensors[t];
+    uint32_t a, b, c;
+    spec_chunk<WDT, GDT, L2>(d, chunk, outs[t].weight, outs[t].exp_avg, outs[t].exp_avg_sq, k, red, a, b, c);
     if (threadIdx.x == 0) {
         if (a) atomicMax(&d.acc[0], a);
         if (b) atomicMax(&d.acc[1], b);
         if (c) atomicMax(&d.acc[2], c);
     }
+}
+
+// ---- the one-pass step inside shifting arenas -------------------------------------------------------------
+// The speculative pass needs its outputs away from its inputs (a tensor whose scales it guessed wrong is done again
+// from the inputs), but not a whole second set of buffers.  Here the payloads of all tensors lie back to back in one
+// arena per kind (weights, exp_avg, exp_avg_sq), each tensor padded to whole chunks, with `slack` chunks of room at
+// one end, and a step moves everything by `slack` chunks towards the room: the workgroup of chunk j writes where the
+// chunk `slack` positions earlier in the walk used to be.  That earlier chunk's tensor must be through by then: every
+// workgroup bumps its tensor's counter when its chunk is stored, the one that bumps it last applies the scale rule
+// (what fused_scales_kernel does for the other forms) and posts the outcome in the tensor's post words.  A workgroup
+// about to overwrite a chunk first waits for that post -- only ever for tensors that lie wholly earlier in the walk,
+// whose workgroups the hardware started earlier, so nobody waits for a workgroup that cannot run -- and, if the post
+// says the tensor takes another round, does that chunk again first, from the inputs it is about to overwrite.  The
+// chunks at the end of the walk, which nobody overwrites, are seen to by fused_shift_tail_kernel.  The next step walks
+// the other way and moves everything back.  Extra memory: `slack` chunks per arena instead of a second copy.
+//
+// What crosses between workgroups, and how, without a fence (a release or acquire at agent scope writes back or
+// invalidates a whole L2 on this part, which one workgroup in sixty thousand can afford and every workgroup cannot):
+//  * the maxima and the counter are agent-scope atomics; the counter's increment takes the returned old maxima as an
+//    operand, so it is issued only when those atomics have been performed;
+//  * a post is one 8-byte agent-scope store of {token, value}: whoever reads this call's token beside a value reads
+//    that value;
+//  * payload stores are written through (put16 / put1 with THRU) and every wave waits for its own before the
+//    workgroup's barrier, so a chunk is in memory before its workgroup counts it -- and before any workgroup that then
+//    writes the same places a second time (the other round, possibly from another die) issues its stores;
+//  * inputs are read with ordinary loads: nothing writes them during the launch until their own overwriting.
+struct ShiftArgs {
+    long long shift;        // output element = input element + shift (its sign is the direction of the walk)
+    int slack;              // |shift| in chunks
+    int n_chunks;
+    uint32_t token;
+    uint32_t spin_limit;
+    uint32_t* error_word;
+    int32_t* redo;
+    uint64_t* posts;        // kShiftPostWords words per tensor
+    float w_fp_max;
+    int tensor_scale;
+};
+constexpr uint32_t kErrShiftGaveUp = 4, kErrShiftLayout = 8;
+// post words of a tensor: [0] 1 = another round; then the factors that round needs: the old weight scale_inv, the old
+// reciprocal moment scales, the new weight and moment scales
+constexpr int kShiftPostWords = MSAMP_ADAMW_POST_WORDS;
+
+__device__ __forceinline__ void post_word(uint64_t* p, uint32_t token, uint32_t value) {
+    __hip_atomic_store(p, (static_cast<uint64_t>(token) << 32) | value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// the value posted beside this call's token; `ok` is cleared if it does not show up within the limit
+__device__ __forceinline__ uint32_t await_post(const uint64_t* p, const ShiftArgs& a, bool& ok) {
+    for (uint32_t spins = 0; ok; ++spins) {
+        const uint64_t w = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (static_cast<uint32_t>(w >> 32) == a.token) return static_cast<uint32_t>(w);
+        // the limit, or somebody else has given up already: nobody waits any longer
+        if (spins >= a.spin_limit || __hip_atomic_load(a.error_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) ok = false;
+        else __builtin_amdgcn_s_sleep(8);
+    }
+    return 0u;
+}
+
+template <int WDT>
+__device__ __forceinline__ void* shifted_weight(void* p, long long shift) {
+    if constexpr (WDT == MSAMP_DT_F16) return static_cast<uint16_t*>(p) + shift;
+    else return static_cast<uint8_t*>(p) + shift;
+}
+
+// what fused_scales_kernel does, for one tensor, by the workgroup that stored the tensor's last chunk
+__device__ __forceinline__ void decide_tensor(msamp_adamw_tensor& d, int t, const ShiftArgs& a) {
+    const float ap = __uint_as_float(__hip_atomic_load(&d.acc[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    const float am = __uint_as_float(__hip_atomic_load(&d.acc[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    const float av = __uint_as_float(__hip_atomic_load(&d.acc[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    // left at zero for the next step (atomic stores: the words are only ever touched at that level)
+    __hip_atomic_store(&d.acc[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&d.acc[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&d.acc[2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&d.reserved[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float old_ws = *d.w_scale, old_ms = *d.m_scale, old_vs = *d.v_scale;
+    const float old_wsi = *d.w_scale_inv, old_inv_m = 1.0f / old_ms, old_inv_v = 1.0f / old_vs;
+    d.saved[0] = old_wsi, d.saved[1] = old_inv_m, d.saved[2] = old_inv_v;
+    const float ws = scale_rule(ap, old_ws, a.w_fp_max, 0);
+    const float ms = a.tensor_scale ? scale_rule(am, 1.0f, 448.0f, 0) : 1.0f;
+    const float vs = a.tensor_scale ? scale_rule(av, 1.0f, 65504.0f, 0) : 1.0f;
+    const uint32_t again = (__float_as_uint(ws) != __float_as_uint(old_ws) || __float_as_uint(ms) != __float_as_uint(old_ms) ||
+                            __float_as_uint(vs) != __float_as_uint(old_vs))
+                               ? 1u
+                               : 0u;
+    // for the kernels and the host that come after this launch
+    a.redo[t] = static_cast<int32_t>(again);
+    *d.w_scale = ws;
+    *d.w_scale_inv = 1.0f / ws;
+    *d.w_amax = ap;
+    *d.m_scale = ms;
+    *d.m_scale_inv = 1.0f / ms;
+    *d.m_amax = am;
+    *d.v_scale = vs;
+    *d.v_scale_inv = 1.0f / vs;
+    *d.v_amax = av;
+    // for the workgroups of this launch that will overwrite this tensor's chunks
+    uint64_t* post = a.posts + static_cast<size_t>(t) * kShiftPostWords;
+    if (again) {
+        post_word(post + 1, a.token, __float_as_uint(old_wsi));
+        post_word(post + 2, a.token, __float_as_uint(old_inv_m));
+        post_word(post + 3, a.token, __float_as_uint(old_inv_v));
+        post_word(post + 4, a.token, __float_as_uint(ws));
+        post_word(post + 5, a.token, __float_as_uint(ms));
+        post_word(post + 6, a.token, __float_as_uint(vs));
+    }
+    post_word(post, a.token, again);
+}
+
+template <int WDT, int GDT, bool L2>
+__global__ __launch_bounds__(kAdamThreads) void fused_shift_kernel(msamp_adamw_tensor* __restrict__ tensors,
+                                                                    const int32_t* __restrict__ block_map, AdamConsts k,
+                                                                    ShiftArgs a) {
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    __shared__ int s_verdict;
+    __shared__ float s_factor[6];
+    const int b = blockIdx.x;
+    const bool up = a.shift > 0;    // moving up: walk from the top, so that the room is always ahead
+    const int j = up ? a.n_chunks - 1 - b : b;
+    const int t = block_map[2 * j], chunk = block_map[2 * j + 1];
+    if (b >= a.slack) {
+        // the chunk that lies where this one's outputs go
+        const int jv = up ? j + a.slack : j - a.slack;
+        const int tv = block_map[2 * jv], cv = block_map[2 * jv + 1];
+        if (threadIdx.x == 0) {
+            int verdict = -1;
+            if (tv == t) {
+                // a tensor longer than the room: the layout is not what this kernel needs
+                report_wait_expired(a.error_word, kErrShiftLayout);
+            } else {
+                const uint64_t* post = a.posts + static_cast<size_t>(tv) * kShiftPostWords;
+                bool ok = true;
+                const uint32_t again = await_post(post, a, ok);
+                if (ok && again) {
+#pragma unroll
+                    for (int i = 0; i < 6; ++i) s_factor[i] = __uint_as_float(await_post(post + 1 + i, a, ok));
+                }
+                if (ok) verdict = static_cast<int>(again);
+                else report_wait_expired(a.error_word, kErrShiftGaveUp);
+            }
+            s_verdict = verdict;
+        }
+        __syncthreads();
+        // gave up: this chunk is left as it was (the call has failed; the error word says so)
+        if (s_verdict < 0) return;
+        if (s_verdict > 0) {
+            msamp_adamw_tensor& dv = tensors[tv];
+            const float g_si0 = *dv.g_scale_inv, g_si = k.maximize ? -g_si0 : g_si0;
+            write_chunk<WDT, GDT, L2, true>(dv, cv, shifted_weight<WDT>(dv.weight, a.shift), dv.exp_avg + a.shift,
+                                            dv.exp_avg_sq + a.shift, s_factor[0], g_si, s_factor[1], s_factor[2], s_factor[3],
+                                            s_factor[4], s_factor[5], k);
+            // its loads are through (they fed its stores) before this chunk's outputs land on what they read
+            __syncthreads();
+        }
+    }
+    msamp_adamw_tensor& d = tensors[t];
+    uint32_t mp, mm, mv;
+    spec_chunk<WDT, GDT, L2, true>(d, chunk, shifted_weight<WDT>(d.weight, a.shift), d.exp_avg + a.shift, d.exp_avg_sq + a.shift, k,
+                                   red, mp, mm, mv);
+    if (threadIdx.x == 0) {
+        const uint32_t chunks = static_cast<uint32_t>((d.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK);
+        // the maxima first; their returned values are an operand of the count, which is therefore issued after them
+        const uint32_t o0 = atomicMax(&d.acc[0], mp), o1 = atomicMax(&d.acc[1], mm), o2 = atomicMax(&d.acc[2], mv);
+        uint32_t one = 1u;
+        asm volatile("" : "+v"(one) : "v"(o0), "v"(o1), "v"(o2));
+        const uint32_t count = atomicAdd(&d.reserved[0], one);
+        if (count == chunks - 1) decide_tensor(d, t, a);
+    }
+}
+
+// the last `slack` chunks of the walk: nothing is written over them, so nobody has looked at their tensors' marks
+// (a launch of its own: everything the first one stored is in memory by now, ordinary loads do)
+template <int WDT, int GDT, bool L2>
+__global__ __launch_bounds__(kAdamThreads) void fused_shift_tail_kernel(msamp_adamw_tensor* __restrict__ tensors,
+                                                                         const int32_t* __restrict__ block_map, AdamConsts k,
+                                                                         ShiftArgs a) {
+    const int first = a.n_chunks > a.slack ? a.n_chunks - a.slack : 0;
+    const int b = first + blockIdx.x;    // position in the walk
+    const int j = a.shift > 0 ? a.n_chunks - 1 - b : b;
+    const int t = block_map[2 * j], chunk = block_map[2 * j + 1];
+    if (a.redo[t] == 0) return;
+    msamp_adamw_tensor& d = tensors[t];
+    const float g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv;
+    write_chunk<WDT, GDT, L2>(d, chunk, shifted_weight<WDT>(d.weight, a.shift), d.exp_avg + a.shift, d.exp_avg_sq + a.shift,
+                              d.saved[0], g_si, d.saved[1], d.saved[2], *d.w_scale, *d.m_scale, *d.v_scale, k);
 }
 
 static int adam_grid(size_t n) {
@@ -799,6 +1027,39 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
     const int32_t* redo_in = redo;
     FUSED_LAUNCH(fused_write_kernel, n_blocks, tensors, block_map, k, outputs, redo_in);
     MSAMP_CHECK_LAUNCH("fused_write_kernel");
+    return MSAMP_OK;
+}
+int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, uint64_t* posts, int n_tensors,
+                                const int32_t* block_map, int n_blocks, long long shift_elems, int weight_dtype, int grad_dtype,
+                                double lr, double beta1, double beta2, double eps, double weight_decay, int step,
+                                int bias_correction, int adam_mode, int maximize, int tensor_scale, void* workspace,
+                                msamp_stream_t stream) {
+    const int rc = fused_args_ok("msamp_adamw_fp8_fused_shift", tensors, n_tensors, block_map, n_blocks, weight_dtype, grad_dtype);
+    if (rc != MSAMP_OK || n_tensors == 0 || n_blocks == 0) return rc;
+    MSAMP_REQUIRE(redo != nullptr && posts != nullptr, MSAMP_ERR_NULL, "msamp_adamw_fp8_fused_shift: null redo or posts");
+    MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_adamw_fp8_fused_shift: workspace required");
+    const long long mag = shift_elems < 0 ? -shift_elems : shift_elems;
+    MSAMP_REQUIRE(mag > 0 && mag % MSAMP_ADAMW_CHUNK == 0 && mag / MSAMP_ADAMW_CHUNK <= 0x7fffffffLL, MSAMP_ERR_SHAPE,
+                  "msamp_adamw_fp8_fused_shift: shift_elems=%lld must be a non-zero multiple of %d", shift_elems, MSAMP_ADAMW_CHUNK);
+    AdamConsts k;
+    const bool l2 = fused_consts(lr, beta1, beta2, eps, weight_decay, step, bias_correction, adam_mode, maximize, k);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    ShiftArgs a;
+    a.shift = shift_elems;
+    a.slack = static_cast<int>(mag / MSAMP_ADAMW_CHUNK);
+    a.n_chunks = n_blocks;
+    a.token = next_tokens(1);
+    a.spin_limit = collector_spin_limit();
+    a.error_word = static_cast<uint32_t*>(workspace) + kWsErrorWord;
+    a.redo = redo;
+    a.posts = posts;
+    a.w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
+    a.tensor_scale = tensor_scale;
+    FUSED_LAUNCH(fused_shift_kernel, n_blocks, tensors, block_map, k, a);
+    MSAMP_CHECK_LAUNCH("fused_shift_kernel");
+    const int tail = n_blocks < a.slack ? n_blocks : a.slack;
+    FUSED_LAUNCH(fused_shift_tail_kernel, tail, tensors, block_map, k, a);
+    MSAMP_CHECK_LAUNCH("fused_shift_tail_kernel");
     return MSAMP_OK;
 }
 #undef FUSED_LAUNCH

@@ -60,6 +60,7 @@ _SIGNATURES = {
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_adamw_fp8_fused_shift': ([_vp, _vp, _vp, _i, _vp, _i, ctypes.c_longlong, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _vp], _i),
     'msamp_adamw_fp8_fused_speculative': ([_vp, _vp, _vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
 }
 
@@ -720,4 +721,30 @@ def adamw_fused_speculative(desc, outputs, redo, n_tensors, block_map, n_blocks,
             eps, weight_decay, step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0,
             1 if tensor_scale else 0, _stream()
         ), 'msamp_adamw_fp8_fused_speculative'
+    )
+
+
+ADAMW_POST_WORDS = 8
+
+
+def adamw_fused_shift(desc, redo, posts, n_tensors, block_map, n_blocks, shift_elems, weight_dt, grad_dt, lr, beta1, beta2, eps,
+                      weight_decay, step, bias_correction, adam_mode, maximize, tensor_scale):
+    """The fused step in one pass inside shifting arenas: every tensor's new payloads land `shift_elems` elements away
+    from the old ones (see msamp_adamw_fp8_fused_shift for the layout this needs).  `redo`: int32 device tensor
+    [n_tensors], set by the call where a tensor took the second round; `posts`: int64 device tensor [n_tensors,
+    ADAMW_POST_WORDS], zeroed once, the kernels' own."""
+    lib = load()
+    _gpu(desc, 'descriptor table')
+    _gpu(redo, 'redo flags')
+    if redo.dtype != torch.int32 or redo.numel() != n_tensors or not redo.is_contiguous():
+        raise ValueError('redo must be a contiguous int32 tensor of n_tensors flags')
+    _gpu(posts, 'post words')
+    if posts.dtype != torch.int64 or posts.numel() != n_tensors * ADAMW_POST_WORDS or not posts.is_contiguous():
+        raise ValueError('posts must be a contiguous int64 tensor of n_tensors x %d words' % ADAMW_POST_WORDS)
+    _check(
+        lib.msamp_adamw_fp8_fused_shift(
+            _ptr(desc), _ptr(redo), _ptr(posts), n_tensors, _ptr(block_map), n_blocks, int(shift_elems), weight_dt, grad_dt, lr, beta1, beta2,
+            eps, weight_decay, step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0,
+            1 if tensor_scale else 0, _ptr(workspace(desc.device)), _stream()
+        ), 'msamp_adamw_fp8_fused_shift'
     )

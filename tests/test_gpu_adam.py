@@ -293,6 +293,127 @@ def test_speculative_step_special_values(be):
         _check(spec, t, fp8.E4M3, fp8.E5M2, 2, **kw)
 
 
+def _fused_shift(be, tensors, w_dt, g_dt, step, slack, up, check_clean=True, **kw):
+    """msamp_adamw_fp8_fused_shift on a list of tensor dicts: the payloads are laid out back to back, padded to whole
+    chunks, in three arenas with `slack` chunks of room (below the data when the step moves down, above it when it moves
+    up); returns device copies of everything, the new payloads read from where the step put them."""
+    ch = be.ADAMW_CHUNK
+    chunks = [(t['w'].numel() + ch - 1) // ch for t in tensors]
+    pos = np.concatenate([[0], np.cumsum(chunks)]).tolist()
+    total = pos[-1]
+    wsz = 2 if w_dt == 3 else 1
+    arenas = {k: torch.full(((total + slack) * ch * sz, ), 0x55, dtype=torch.uint8, device='cuda')
+              for k, sz in (('w', wsz), ('m', 1), ('v', 2))}
+    size = dict(w=wsz, m=1, v=2)
+    src, dst = (0, slack) if up else (slack, 0)
+
+    def view(kind, t_idx, off, like):
+        first = (pos[t_idx] + off) * ch * size[kind]
+        return arenas[kind][first:first + like.numel() * size[kind]].view(like.dtype)
+
+    dev, rows = [], []
+    for i, t in enumerate(tensors):
+        d = dict(g=t['g'].cuda(), wm=_dev_meta(t['wm']), gsi=t['gm']['scale_inv'].clone().cuda().reshape(()),
+                 mm=_dev_meta(t['mm']), vm=_dev_meta(t['vm']))
+        for kind in 'wmv':
+            d[kind] = view(kind, i, src, t[kind])
+            d[kind].copy_(t[kind])
+        dev.append(d)
+        rows.append((d['w'].data_ptr(), d['g'].data_ptr(), d['m'].data_ptr(), d['v'].data_ptr(),
+                     d['wm'][0].data_ptr(), d['wm'][1].data_ptr(), d['wm'][2].data_ptr(), d['gsi'].data_ptr(),
+                     d['mm'][0].data_ptr(), d['mm'][1].data_ptr(), d['mm'][2].data_ptr(),
+                     d['vm'][0].data_ptr(), d['vm'][1].data_ptr(), d['vm'][2].data_ptr(), d['w'].numel(), 0, 0, 0, 0))
+    desc = torch.from_numpy(np.asarray(rows, dtype=np.int64)).cuda()
+    bm = np.stack([np.repeat(np.arange(len(tensors), dtype=np.int32), chunks),
+                   np.concatenate([np.arange(c, dtype=np.int32) for c in chunks])], axis=1).copy()
+    block_map = torch.from_numpy(bm).cuda()
+    hyper = dict(HYPER)
+    hyper.update(kw)
+    redo = torch.full((len(dev), ), -1, dtype=torch.int32, device='cuda')
+    posts = torch.zeros(len(dev), be.ADAMW_POST_WORDS, dtype=torch.int64, device='cuda')
+    be.adamw_fused_shift(desc, redo, posts, len(tensors), block_map, total, (slack if up else -slack) * ch, w_dt, g_dt, hyper['lr'],
+                         hyper['beta1'], hyper['beta2'], hyper['eps'], hyper['weight_decay'], step,
+                         hyper.get('bias_correction', True), hyper.get('adam_mode', False), hyper.get('maximize', False),
+                         hyper.get('tensor_scale', True))
+    torch.cuda.synchronize()
+    for i, (d, t, r) in enumerate(zip(dev, tensors, redo.tolist())):
+        for kind in 'wmv':
+            d[kind] = view(kind, i, dst, t[kind]).clone()
+        d['redo'] = r
+    if check_clean:    # accumulators and counters of the descriptors are left zeroed
+        assert (desc[:, 15].cpu() == 0).all() and (desc[:, 16].cpu() & 0xffffffff == 0).all()
+        assert (desc[:, 18].cpu() & 0xffffffff == 0).all()
+    return dev
+
+
+@pytest.mark.parametrize('w_fmt,w_dt,g_fmt,g_dt', [(fp8.E4M3, 5, fp8.E5M2, 6), ('f16', 3, fp8.E4M3, 5), (fp8.E5M2, 6, fp8.E4M3, 5)])
+@pytest.mark.parametrize('slack', [256, 300, 4096])
+def test_shifting_step_equals_the_in_place_step(be, w_fmt, w_dt, g_fmt, g_dt, slack):
+    """The one-pass step inside shifting arenas against the two-pass step in place, four steps in a row from the same
+    states, the direction alternating.  The first step starts from zero moments with scale 1, so every guess is wrong and
+    every tensor takes its second round: with little room (256 chunks, exactly the largest tensor: the workgroups that
+    overwrite a chunk meet tensors that have only just finished) those rounds are taken by the workgroups that follow,
+    with 300 partly by them and partly by the closing launch, with more room than data (4096) by the closing launch
+    alone.  Later steps keep their scales; a gradient sixteen times larger moves them again."""
+    sizes = [16384 * 4, 16384 * 2 + 777, 5, 4096 * 1024, 16384]
+    tensors = [_inputs(n, 400 + i, w_fmt, g_fmt, zero_state=True) for i, n in enumerate(sizes)]
+    hits = misses = 0
+    for step in range(1, 5):
+        plain = _fused(be, tensors, w_dt, g_dt, step)
+        moved = _fused_shift(be, tensors, w_dt, g_dt, step, slack, up=step % 2 == 0)
+        for a, b, t in zip(plain, moved, tensors):
+            assert _same_state(a, b), (step, t['w'].numel())
+            changed = not (same_float(a['wm'][0], t['wm']['scale']) and same_float(a['mm'][0], t['mm']['scale']) and
+                           same_float(a['vm'][0], t['vm']['scale']))
+            assert b['redo'] == int(changed)
+            hits += 1 - b['redo']
+            misses += b['redo']
+        tensors = [_next_inputs(t, d, 500 + 10 * step + i, g_fmt, grad_std=1.6e-2 if step == 3 else 1e-3)
+                   for i, (t, d) in enumerate(zip(tensors, plain))]
+    assert hits >= 3 and misses >= len(sizes)
+    be.check_async_error(block=True)
+
+
+@pytest.mark.parametrize('kw', [dict(adam_mode=True), dict(maximize=True), dict(bias_correction=False), dict(weight_decay=0.0),
+                                dict(tensor_scale=False), dict(lr=0.5, eps=0.0)])
+def test_shifting_step_variants(be, kw):
+    t = [_inputs(16384 * 3 + 100, 7, fp8.E4M3, fp8.E5M2), _inputs(16384 * 2, 8, fp8.E4M3, fp8.E5M2)]
+    for step in (2, 3):
+        plain = _fused(be, t, 5, 6, step, **kw)
+        moved = _fused_shift(be, t, 5, 6, step, 4, up=step == 3, **kw)
+        assert all(_same_state(a, b) for a, b in zip(plain, moved))
+        t = [_next_inputs(ti, pi, 60 + step + 7 * i, fp8.E5M2) for i, (ti, pi) in enumerate(zip(t, plain))]
+    be.check_async_error(block=True)
+
+
+def test_shifting_step_many_tensors_little_room(be):
+    """Forty tensors of eight to forty chunks and room for 48 chunks: every workgroup from the 49th on overwrites a
+    chunk whose tensor finished moments ago, and in the first step also does that chunk again."""
+    sizes = [16384 * (8 + (7 * i) % 33) - (i % 3) * 1000 for i in range(40)]
+    tensors = [_inputs(n, 900 + i, fp8.E4M3, fp8.E5M2, zero_state=i % 2 == 0) for i, n in enumerate(sizes)]
+    for step in (1, 2, 3):
+        plain = _fused(be, tensors, 5, 6, step)
+        moved = _fused_shift(be, tensors, 5, 6, step, 48, up=step == 2)
+        assert all(_same_state(a, b) for a, b in zip(plain, moved)), step
+        tensors = [_next_inputs(t, d, 950 + 50 * step + i, fp8.E5M2) for i, (t, d) in enumerate(zip(tensors, plain))]
+    be.check_async_error(block=True)
+
+
+def test_shifting_step_refuses_a_tensor_longer_than_the_room(be):
+    """A tensor of 256 chunks with room for 255: some workgroup would have to overwrite a chunk of its own tensor.  The
+    kernel flags the layout in the sticky error word, leaves those chunks alone and runs to its end."""
+    tensors = [_inputs(16384 * 2, 31, fp8.E4M3, fp8.E5M2), _inputs(4096 * 1024, 32, fp8.E4M3, fp8.E5M2)]
+    be.check_async_error(block=True)
+    saved = be._force_two_pass
+    try:
+        _fused_shift(be, tensors, 5, 6, 2, 255, up=False, check_clean=False)
+        with pytest.raises(be.WaitExpiredError):
+            be.check_async_error(block=True)
+    finally:
+        be._force_two_pass = saved
+    be.check_async_error(block=True)
+
+
 def test_fused_step_is_deterministic(be):
     t = _inputs(16384 * 9, 21, fp8.E4M3, fp8.E5M2)
     a = _fused(be, [t], 5, 6, 2)[0]
