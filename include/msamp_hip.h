@@ -385,15 +385,16 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
  * point at the new places).  No tensor may have more chunks than the room holds (sticky error word otherwise, see
  * below); for the workgroups never to wait for each other in practice, make the room a few thousand chunks larger
  * than the largest tensor.  Results, metas and `redo` as for msamp_adamw_fp8_fused_speculative: the same bits that
- * msamp_adamw_fp8_fused leaves in place.  `posts`: DEVICE array of MSAMP_ADAMW_POST_WORDS 8-byte words per tensor,
- * zeroed once by the caller, through which the workgroups of a call tell each other how a tensor came out.  The
- * descriptors' acc and reserved words must be zero before the first call (the library leaves them at zero).  `workspace`: the MSAMP_WORKSPACE_BYTES buffer of the other entry points; a wait that
+ * msamp_adamw_fp8_fused leaves in place.  `sync`: DEVICE buffer of MSAMP_ADAMW_SYNC_BYTES(n_tensors, n_blocks) bytes,
+ * 8-byte aligned, zeroed once by the caller, through which the workgroups of a call tell each other which chunks are
+ * stored and how a tensor came out.  The descriptors' acc words must be zero before the first call (the library
+ * leaves them at zero).  `workspace`: the MSAMP_WORKSPACE_BYTES buffer of the other entry points; a wait that
  * runs out (msamp_set_spin_limit) or a layout that breaks the rule above sets its sticky error word, reported by
  * msamp_check_async_error: the state is then partly updated and must be restored from a copy. */
 #define MSAMP_ADAMW_POST_WORDS 8
-int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, uint64_t* posts, int n_tensors,
-                                const int32_t* block_map, int n_blocks, long long shift_elems, int weight_dtype, int grad_dtype,
-                                double lr, double beta1,
+#define MSAMP_ADAMW_SYNC_BYTES(n_tensors, n_blocks) ((size_t)(n_tensors) * MSAMP_ADAMW_POST_WORDS * 8 + (size_t)(n_blocks) * 136)
+int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, void* sync, int n_tensors, const int32_t* block_map,
+                                int n_blocks, long long shift_elems, int weight_dtype, int grad_dtype, double lr, double beta1,
                                 double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
                                 int maximize, int tensor_scale, void* workspace, msamp_stream_t stream);
 

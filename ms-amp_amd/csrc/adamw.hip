@@ -319,54 +319,31 @@ __global__ void fused_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, 
     *d.v_amax = av;
 }
 
-// Stores of the fused kernels' outputs.  THRU: written through to where every compute unit of the GPU sees them (the
-// `sc1` stores that an agent-scope atomic store is made of), which the shifting step needs: there a chunk may be
-// written twice, by workgroups on different dies with an L2 each, and a line left dirty in one of them would be
-// written back over the later store.  The stores are assembly because no builtin makes a 16-byte one; the kernel
-// waits for them by hand (s_waitcnt) where their completion matters.
-template <bool THRU>
-__device__ __forceinline__ void put16(void* p, const uint4& v) {
-    if constexpr (THRU) {
-        typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
-        const v4u_t vv = {v.x, v.y, v.z, v.w};
-        // (the wait states after it: a store of more than 8 bytes reads its data registers over several cycles, and the
-        // compiler, which does not know this is one, would not keep the next instruction off them)
-        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(vv) : "memory");
-    } else {
-        *static_cast<uint4*>(p) = v;
-    }
-}
-template <bool THRU, typename T>
-__device__ __forceinline__ void put1(T* p, T v) {
-    if constexpr (THRU) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *p = v;
-}
-
-template <int WDT, bool THRU = false>
+template <int WDT>
 __device__ __forceinline__ void store_w16(void* base, size_t i, const float* f) {
     if constexpr (WDT == MSAMP_DT_F16) {
         uint32_t w[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) w[j] = float_to_f16_bits(f[2 * j]) | (float_to_f16_bits(f[2 * j + 1]) << 16);
         uint4* p = reinterpret_cast<uint4*>(static_cast<uint16_t*>(base) + i);
-        put16<THRU>(p, make_uint4(w[0], w[1], w[2], w[3]));
-        put16<THRU>(p + 1, make_uint4(w[4], w[5], w[6], w[7]));
+        p[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        p[1] = make_uint4(w[4], w[5], w[6], w[7]);
     } else {
         uint4 o;
         o.x = quant4<WDT>(f[0], f[1], f[2], f[3]);
         o.y = quant4<WDT>(f[4], f[5], f[6], f[7]);
         o.z = quant4<WDT>(f[8], f[9], f[10], f[11]);
         o.w = quant4<WDT>(f[12], f[13], f[14], f[15]);
-        put16<THRU>(static_cast<uint8_t*>(base) + i, o);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(base) + i) = o;
     }
 }
 
-template <int WDT, bool THRU = false>
+template <int WDT>
 __device__ __forceinline__ void store_w1(void* base, size_t i, float f) {
     if constexpr (WDT == MSAMP_DT_F16) {
-        put1<THRU>(static_cast<uint16_t*>(base) + i, static_cast<uint16_t>(float_to_f16_bits(f)));
+        static_cast<uint16_t*>(base)[i] = static_cast<uint16_t>(float_to_f16_bits(f));
     } else {
-        put1<THRU>(static_cast<uint8_t*>(base) + i, static_cast<uint8_t>(quant1<WDT>(f)));
+        static_cast<uint8_t*>(base)[i] = static_cast<uint8_t>(quant1<WDT>(f));
     }
 }
 
@@ -382,7 +359,7 @@ __device__ __forceinline__ uint32_t quant_weight_exact(float pj, float m_new, fl
 }
 
 // One lane's 16 elements of the second pass: requantized weight, exp_avg and exp_avg_sq are stored at element i.
-template <int WDT, bool L2, bool THRU = false>
+template <int WDT, bool L2>
 __device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i, float* p, const float* g,
                                            float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
                                            float ms, float vs, const AdamConsts& k) {
@@ -413,18 +390,18 @@ __device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t
     }
     if constexpr (WDT == MSAMP_DT_F16) {
         uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
-        put16<THRU>(o, make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16)));
-        put16<THRU>(o + 1, make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16)));
+        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
+        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
     } else {
         uint4 o;
         o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
         o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
         o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-        put16<THRU>(static_cast<uint8_t*>(w_out) + i, o);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
     }
-    store_w16<MSAMP_DT_E4M3, THRU>(m_out, i, m);
-    store_w16<MSAMP_DT_F16, THRU>(v_out, i, v);
+    store_w16<MSAMP_DT_E4M3>(m_out, i, m);
+    store_w16<MSAMP_DT_F16>(v_out, i, v);
 }
 
 // Second pass: recompute m', v' exactly and requantize them; for the weight, quantize both ends of the
@@ -432,7 +409,7 @@ __device__ __forceinline__ void write_step(void* w_out, uint8_t* m_out, uint16_t
 // exact answer, otherwise (or for anything non-finite) the element takes the exact chain.
 // One chunk of the second pass: the tensor's inputs at d.weight / d.grad / d.exp_avg / d.exp_avg_sq, requantized with
 // the given scales into w_out / m_out / v_out (which may be the inputs' own places).
-template <int WDT, int GDT, bool L2, bool THRU = false>
+template <int WDT, int GDT, bool L2>
 __device__ __forceinline__ void write_chunk(const msamp_adamw_tensor& d, int chunk, void* w_out, uint8_t* m_out, uint16_t* v_out,
                                             float w_si, float g_si, float inv_m, float inv_v, float ws, float ms, float vs,
                                             const AdamConsts& k) {
@@ -444,7 +421,7 @@ __device__ __forceinline__ void write_chunk(const msamp_adamw_tensor& d, int chu
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            write_step<WDT, L2, THRU>(w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
+            write_step<WDT, L2>(w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
@@ -452,10 +429,10 @@ __device__ __forceinline__ void write_chunk(const msamp_adamw_tensor& d, int chu
             float pj, g_plain, m_new, v_new;
             prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj,
                     g_plain, m_new, v_new);
-            store_w1<WDT, THRU>(w_out, i, param_update(pj, m_new, v_new, k) * ws);
+            store_w1<WDT>(w_out, i, param_update(pj, m_new, v_new, k) * ws);
             if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
-            store_w1<MSAMP_DT_E4M3, THRU>(m_out, i, m_new * ms);
-            store_w1<MSAMP_DT_F16, THRU>(v_out, i, v_new * vs);
+            store_w1<MSAMP_DT_E4M3>(m_out, i, m_new * ms);
+            store_w1<MSAMP_DT_F16>(v_out, i, v_new * vs);
         }
     }
 }
@@ -490,12 +467,205 @@ __global__ __launch_bounds__(kAdamThreads) void fused_write_kernel(msamp_adamw_t
 // ones used.  Where they agree the output is what the two passes above produce, bit for bit; a tensor where they do
 // not is done again by fused_write_kernel from its inputs, which this pass does not touch.
 //
-// One lane's 16 elements: as write_step, plus the maxima.  |m'| and |v'| are exact.  For |p'| the estimate gives
-// |p_est| - err <= |p'| <= |p_est| + err; only elements whose upper end reaches the best lower end seen so far are
-// evaluated exactly, and the element that attains the maximum always is.  Elements that took the exact chain for
-// their code (an estimate too close to a rounding boundary, anything non-finite) have their exact |p'| already.
-template <int WDT, int GDT, bool L2, bool THRU = false>
-__device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i,
+// A lane works on eight consecutive elements at a time (one 8-byte load each of weight, gradient and exp_avg codes,
+// one 16-byte load of exp_avg_sq; 2-byte weights: 16 bytes), two such groups per step, 2048 elements apart, so that
+// every load and store instruction of a wavefront covers one contiguous run of whole cache lines.  |m'| and |v'| are
+// exact.  For |p'| the estimate gives |p_est| - err <= |p'| <= |p_est| + err; only elements whose upper end reaches the
+// best lower end seen so far are evaluated exactly, and the element that attains the maximum always is.  Elements that
+// took the exact chain for their code (an estimate too close to a rounding boundary, anything non-finite) have their
+// exact |p'| already.
+constexpr int kGroup = 8;                                              // elements per lane and group
+constexpr int kGroupSpan = kAdamThreads * kGroup;                      // 2048 elements per workgroup and group
+constexpr int kSpecSteps = MSAMP_ADAMW_CHUNK / (2 * kGroupSpan);       // 4 steps of two groups
+
+// Stores of the fused kernels' outputs.  THRU: written through to where every compute unit of the GPU sees them (the
+// `sc1` stores that an agent-scope atomic store is made of), which the shifting step needs: there a chunk may be
+// written twice, by workgroups on different dies with an L2 each, and a line left dirty in one of them would be
+// written back over the later store.  The stores are assembly because no builtin makes a 16-byte one; the kernel
+// waits for them by hand (s_waitcnt) where their completion matters.
+template <bool THRU>
+__device__ __forceinline__ void put16(void* p, const uint4& v) {
+    if constexpr (THRU) {
+        typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+        const v4u_t vv = {v.x, v.y, v.z, v.w};
+        // (the wait states after it: a store of more than 8 bytes reads its data registers over several cycles, and the
+        // compiler, which does not know this is one, would not keep the next instruction off them)
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(vv) : "memory");
+    } else {
+        *static_cast<uint4*>(p) = v;
+    }
+}
+template <bool THRU, typename T>
+__device__ __forceinline__ void put1(T* p, T v) {
+    if constexpr (THRU) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
+template <bool THRU>
+__device__ __forceinline__ void put8(void* p, uint32_t lo, uint32_t hi) {
+    if constexpr (THRU) {
+        __hip_atomic_store(static_cast<uint64_t*>(p), (static_cast<uint64_t>(hi) << 32) | lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        *static_cast<uint2*>(p) = make_uint2(lo, hi);
+    }
+}
+template <int WDT, bool THRU>
+__device__ __forceinline__ void store_one(void* base, size_t i, float f) {
+    if constexpr (WDT == MSAMP_DT_F16) put1<THRU>(static_cast<uint16_t*>(base) + i, static_cast<uint16_t>(float_to_f16_bits(f)));
+    else put1<THRU>(static_cast<uint8_t*>(base) + i, static_cast<uint8_t>(quant1<WDT>(f)));
+}
+
+// eight raw elements of one lane, as loaded: 2 words of FP8 codes or 4 words of float16
+template <int DT>
+struct Raw8 {
+    static constexpr int kWords = DT == MSAMP_DT_F16 ? 4 : 2;
+    uint32_t w[kWords];
+    __device__ __forceinline__ void load(const void* base, size_t i) {
+        if constexpr (DT == MSAMP_DT_F16) {
+            const uint4 a = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(base) + i);
+            w[0] = a.x, w[1] = a.y, w[2] = a.z, w[3] = a.w;
+        } else {
+            const uint2 a = *reinterpret_cast<const uint2*>(static_cast<const uint8_t*>(base) + i);
+            w[0] = a.x, w[1] = a.y;
+        }
+    }
+    // elements 4q .. 4q+3 as floats (exact)
+    __device__ __forceinline__ void quad(int q, float* f) const {
+        if constexpr (DT == MSAMP_DT_F16) {
+            f[0] = f16_bits_to_float(w[2 * q] & 0xffffu), f[1] = f16_bits_to_float(w[2 * q] >> 16);
+            f[2] = f16_bits_to_float(w[2 * q + 1] & 0xffffu), f[3] = f16_bits_to_float(w[2 * q + 1] >> 16);
+        } else {
+            dequant4<DT>(w[q], f[0], f[1], f[2], f[3]);
+        }
+    }
+    template <bool THRU>
+    __device__ __forceinline__ void store(void* base, size_t i) const {
+        if constexpr (DT == MSAMP_DT_F16) put16<THRU>(static_cast<uint16_t*>(base) + i, make_uint4(w[0], w[1], w[2], w[3]));
+        else put8<THRU>(static_cast<uint8_t*>(base) + i, w[0], w[1]);
+    }
+};
+
+// what the speculative pass carries along a chunk
+struct SpecState {
+    float floor_p;    // a lower bound of the tensor's max |p'|
+    uint32_t mxp;     // exact |p'| bit patterns of the candidates (NaN patterns compare highest)
+    float mxm, mxv;
+};
+
+// One group of eight elements at element i: new codes of the weight, exp_avg and exp_avg_sq from the raw inputs, the
+// maxima folded into `st` (TRACK; without it only the codes are made: the other round of a chunk).  Nothing is stored.
+template <int WDT, int GDT, bool L2, bool TRACK = true>
+__device__ __forceinline__ void spec_group(const msamp_adamw_tensor& d, size_t i, const Raw8<WDT>& rw, const Raw8<GDT>& rg,
+                                           const Raw8<MSAMP_DT_E4M3>& rm, const Raw8<MSAMP_DT_F16>& rv, float w_si, float g_si,
+                                           float inv_m, float inv_v, float ws, float ms, float vs, const AdamConsts& k,
+                                           SpecState& st, Raw8<WDT>& ow, Raw8<MSAMP_DT_E4M3>& om, Raw8<MSAMP_DT_F16>& ov) {
+    float hi[kGroup];
+    float lo_max = 0.0f, hi_max = 0.0f;
+    float eps_v = k.eps;
+    asm volatile("" : "+v"(eps_v));
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        float p4[4], g4[4], m4[4], v4[4];
+        rw.quad(q, p4), rg.quad(q, g4), rm.quad(q, m4), rv.quad(q, v4);
+        uint32_t code4[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float pj, g_plain, m_new, v_new, p_est, err;
+            prepare<L2>(p4[e], g4[e], m4[e], v4[e], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+            if constexpr (TRACK) {
+                st.mxm = fmaxf(st.mxm, fabsf(m_new));
+                st.mxv = fmaxf(st.mxv, fabsf(v_new));
+            }
+            estimate(pj, m_new, v_new, k, eps_v, p_est, err);
+            const float lo = (p_est - err) * ws, up = (p_est + err) * ws;
+            bool same;
+            uint32_t code;
+            if constexpr (WDT == MSAMP_DT_F16) {
+                code = float_to_f16_bits(lo);
+                same = code == float_to_f16_bits(up);
+            } else {
+                const uint32_t two = cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(up), 0u, false);
+                code = two & 0xffu;
+                same = code == ((two >> 8) & 0xffu);
+            }
+            float a_hi = fabsf(p_est) + err, a_lo = fabsf(p_est) - err;    // both finite whenever err is
+            if (!(same && err < __uint_as_float(0x7f800000u))) {
+                // the exact chain: its |p'| goes straight into the maximum, and the element leaves the bounds
+                const float pe = param_update(pj, m_new, v_new, k);
+                if constexpr (TRACK) {
+                    const uint32_t ab = __float_as_uint(pe) & 0x7fffffffu;
+                    st.mxp = ab > st.mxp ? ab : st.mxp;
+                }
+                const float scaled = pe * ws;
+                if constexpr (WDT == MSAMP_DT_F16) code = float_to_f16_bits(scaled);
+                else code = quant1<WDT>(scaled);
+                a_hi = 0.0f, a_lo = 0.0f;
+            }
+            code4[e] = code;
+            if constexpr (TRACK) {
+                hi[4 * q + e] = a_hi;
+                hi_max = fmaxf(hi_max, a_hi);
+                lo_max = fmaxf(lo_max, a_lo);
+            }
+            if constexpr (L2) moments(m4[e], v4[e], g_plain, inv_m, inv_v, k, m_new, v_new);    // stored moments ignore the L2 term
+            m4[e] = m_new * ms;
+            v4[e] = v_new * vs;
+        }
+        if constexpr (WDT == MSAMP_DT_F16) {
+            ow.w[2 * q] = code4[0] | (code4[1] << 16), ow.w[2 * q + 1] = code4[2] | (code4[3] << 16);
+        } else {
+            ow.w[q] = code4[0] | (code4[1] << 8) | (code4[2] << 16) | (code4[3] << 24);
+        }
+        om.w[q] = quant4<MSAMP_DT_E4M3>(m4[0], m4[1], m4[2], m4[3]);
+        ov.w[2 * q] = float_to_f16_bits(v4[0]) | (float_to_f16_bits(v4[1]) << 16);
+        ov.w[2 * q + 1] = float_to_f16_bits(v4[2]) | (float_to_f16_bits(v4[3]) << 16);
+    }
+    if constexpr (!TRACK) return;
+    st.floor_p = fmaxf(st.floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
+    const float skip_below = st.floor_p * 0.999999f;    // room for the roundings of the bounds themselves
+    if (hi_max >= skip_below) {    // few lanes get here: the ones that hold an element next to the maximum
+#pragma unroll
+        for (int j = 0; j < kGroup; ++j) {
+            if (hi[j] >= skip_below) {
+                // the inputs are still in memory (this pass writes elsewhere): fetching the element again costs less
+                // than keeping more values per lane alive for the few that come here
+                float pj, g_plain, m_new, v_new;
+                prepare<L2>(load_w1<WDT>(d.weight, i + j), load_w1<GDT>(d.grad, i + j), load_w1<MSAMP_DT_E4M3>(d.exp_avg, i + j),
+                            load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i + j), w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+                const uint32_t ab = __float_as_uint(param_update(pj, m_new, v_new, k)) & 0x7fffffffu;
+                st.mxp = ab > st.mxp ? ab : st.mxp;
+            }
+        }
+    }
+}
+
+// the element-wise tail of a chunk that is not whole (speculative pass)
+template <int WDT, int GDT, bool L2, bool THRU>
+__device__ __forceinline__ void spec_ragged(const msamp_adamw_tensor& d, size_t first, size_t stride, void* w_out, uint8_t* m_out,
+                                            uint16_t* v_out, float w_si, float g_si, float inv_m, float inv_v, float ws, float ms,
+                                            float vs, const AdamConsts& k, SpecState& st) {
+    for (size_t i = first; i < d.numel; i += stride) {
+        const float m_old = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v_old = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
+        float pj, g_plain, m_new, v_new;
+        prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, w_si, g_si, inv_m, inv_v, k, pj, g_plain,
+                    m_new, v_new);
+        const float pn = param_update(pj, m_new, v_new, k);
+        const uint32_t ab = __float_as_uint(pn) & 0x7fffffffu;
+        st.mxp = ab > st.mxp ? ab : st.mxp;
+        st.mxm = fmaxf(st.mxm, fabsf(m_new));
+        st.mxv = fmaxf(st.mxv, fabsf(v_new));
+        store_one<WDT, THRU>(w_out, i, pn * ws);
+        if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
+        store_one<MSAMP_DT_E4M3, THRU>(m_out, i, m_new * ms);
+        store_one<MSAMP_DT_F16, THRU>(v_out, i, v_new * vs);
+    }
+}
+
+// The speculative pass between two sets of buffers works on sixteen consecutive elements per lane (16-byte accesses
+// throughout; measured 6 % faster there than the groups of eight that the shifting step below needs for its
+// written-through stores), one lane's sixteen elements at a time:
+template <int WDT, int GDT, bool L2>
+__device__ __forceinline__ void spec_step16(const msamp_adamw_tensor& d, void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i,
                                           float* p, const float* g,
                                           float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
                                           float ms, float vs, const AdamConsts& k, float& floor_p, uint32_t& mxp,
@@ -547,18 +717,18 @@ __device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_o
     }
     if constexpr (WDT == MSAMP_DT_F16) {
         uint4* o = reinterpret_cast<uint4*>(static_cast<uint16_t*>(w_out) + i);
-        put16<THRU>(o, make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16)));
-        put16<THRU>(o + 1, make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16)));
+        o[0] = make_uint4(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16), wq[4] | (wq[5] << 16), wq[6] | (wq[7] << 16));
+        o[1] = make_uint4(wq[8] | (wq[9] << 16), wq[10] | (wq[11] << 16), wq[12] | (wq[13] << 16), wq[14] | (wq[15] << 16));
     } else {
         uint4 o;
         o.x = wq[0] | (wq[1] << 8) | (wq[2] << 16) | (wq[3] << 24);
         o.y = wq[4] | (wq[5] << 8) | (wq[6] << 16) | (wq[7] << 24);
         o.z = wq[8] | (wq[9] << 8) | (wq[10] << 16) | (wq[11] << 24);
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
-        put16<THRU>(static_cast<uint8_t*>(w_out) + i, o);
+        *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
     }
-    store_w16<MSAMP_DT_E4M3, THRU>(m_out, i, m);
-    store_w16<MSAMP_DT_F16, THRU>(v_out, i, v);
+    store_w16<MSAMP_DT_E4M3>(m_out, i, m);
+    store_w16<MSAMP_DT_F16>(v_out, i, v);
     floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
     const float skip_below = floor_p * 0.999999f;    // room for the roundings of the bounds themselves
     if (hi_max >= skip_below) {    // few lanes get here: the ones that hold an element next to the maximum
@@ -577,11 +747,16 @@ __device__ __forceinline__ void spec_step(const msamp_adamw_tensor& d, void* w_o
     }
 }
 
-// One chunk of the speculative pass: outputs quantized with the scales in force, the chunk's three maxima handed back
-// (valid in the workgroup's first lane).
-template <int WDT, int GDT, bool L2, bool THRU = false>
-__device__ __forceinline__ void spec_chunk(msamp_adamw_tensor& d, int chunk, void* w_out, uint8_t* m_out, uint16_t* v_out,
-                                           const AdamConsts& k, uint32_t* red, uint32_t& max_p, uint32_t& max_m, uint32_t& max_v) {
+template <int WDT, int GDT, bool L2>
+__global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_tensor* __restrict__ tensors,
+                                                                   const int32_t* __restrict__ block_map, AdamConsts k,
+                                                                   const msamp_adamw_buffers* __restrict__ outs) {
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
+    msamp_adamw_tensor& d = tensors[t];
+    void* w_out = outs[t].weight;
+    uint8_t* m_out = outs[t].exp_avg;
+    uint16_t* v_out = outs[t].exp_avg_sq;
     const size_t n = d.numel;
     const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
     const float w_si = *d.w_scale_inv, g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv;
@@ -597,8 +772,8 @@ __device__ __forceinline__ void spec_chunk(msamp_adamw_tensor& d, int chunk, voi
             const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
             float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
             load16<WDT, GDT>(d, i, p, g, m, v);
-            spec_step<WDT, GDT, L2, THRU>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p,
-                                          mxp, mxm, mxv);
+            spec_step16<WDT, GDT, L2>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p, mxp,
+                               mxm, mxv);
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
@@ -611,29 +786,15 @@ __device__ __forceinline__ void spec_chunk(msamp_adamw_tensor& d, int chunk, voi
             mxp = ab > mxp ? ab : mxp;
             mxm = fmaxf(mxm, fabsf(m_new));
             mxv = fmaxf(mxv, fabsf(v_new));
-            store_w1<WDT, THRU>(w_out, i, pn * ws);
+            store_w1<WDT>(w_out, i, pn * ws);
             if constexpr (L2) moments(m_old, v_old, g_plain, inv_m, inv_v, k, m_new, v_new);
-            store_w1<MSAMP_DT_E4M3, THRU>(m_out, i, m_new * ms);
-            store_w1<MSAMP_DT_F16, THRU>(v_out, i, v_new * vs);
+            store_w1<MSAMP_DT_E4M3>(m_out, i, m_new * ms);
+            store_w1<MSAMP_DT_F16>(v_out, i, v_new * vs);
         }
     }
-    // THRU: every wave's stores have arrived before the workgroup's barrier, hence before anything its first lane
-    // publishes afterwards
-    if constexpr (THRU) __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0)
-    max_p = block_max_u32(mxp, red);
-    max_m = block_max_u32(__float_as_uint(mxm), red);
-    max_v = block_max_u32(__float_as_uint(mxv), red);
-}
-
-template <int WDT, int GDT, bool L2>
-__global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_tensor* __restrict__ tensors,
-                                                                   const int32_t* __restrict__ block_map, AdamConsts k,
-                                                                   const msamp_adamw_buffers* __restrict__ outs) {
-    __shared__ uint32_t red[kAdamThreads / kWave];
-    const int t = block_map[2 * blockIdx.x], chunk = block_map[2 * blockIdx.x + 1];
-    msamp_adamw_tensor& d = tensors[t];
-    uint32_t a, b, c;
-    spec_chunk<WDT, GDT, L2>(d, chunk, outs[t].weight, outs[t].exp_avg, outs[t].exp_avg_sq, k, red, a, b, c);
+    const uint32_t a = block_max_u32(mxp, red);
+    const uint32_t b = block_max_u32(__float_as_uint(mxm), red);
+    const uint32_t c = block_max_u32(__float_as_uint(mxv), red);
     if (threadIdx.x == 0) {
         if (a) atomicMax(&d.acc[0], a);
         if (b) atomicMax(&d.acc[1], b);
@@ -646,34 +807,49 @@ __global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_te
 // from the inputs), but not a whole second set of buffers.  Here the payloads of all tensors lie back to back in one
 // arena per kind (weights, exp_avg, exp_avg_sq), each tensor padded to whole chunks, with `slack` chunks of room at
 // one end, and a step moves everything by `slack` chunks towards the room: the workgroup of chunk j writes where the
-// chunk `slack` positions earlier in the walk used to be.  That earlier chunk's tensor must be through by then: every
-// workgroup bumps its tensor's counter when its chunk is stored, the one that bumps it last applies the scale rule
-// (what fused_scales_kernel does for the other forms) and posts the outcome in the tensor's post words.  A workgroup
-// about to overwrite a chunk first waits for that post -- only ever for tensors that lie wholly earlier in the walk,
-// whose workgroups the hardware started earlier, so nobody waits for a workgroup that cannot run -- and, if the post
-// says the tensor takes another round, does that chunk again first, from the inputs it is about to overwrite.  The
-// chunks at the end of the walk, which nobody overwrites, are seen to by fused_shift_tail_kernel.  The next step walks
-// the other way and moves everything back.  Extra memory: `slack` chunks per arena instead of a second copy.
+// chunk `slack` positions earlier in the walk used to be.  That earlier chunk's tensor must be through by then.
+// Every wavefront marks its quarter of a chunk when it is stored.  The workgroup about to overwrite the FIRST chunk
+// of a tensor waits for the marks of all that tensor's chunks, applies the scale rule (what fused_scales_kernel does
+// for the other forms) and posts the outcome; every wavefront about to overwrite any of the tensor's chunks waits for
+// that post.  Nobody ever waits for anything but tensors that lie wholly earlier in the walk, whose workgroups the
+// hardware started earlier, so nobody waits for a workgroup that cannot run; and with the room a few thousand chunks
+// larger than the largest tensor nobody waits at all in practice: the post is asked for when a wavefront starts and
+// looked at when its first outputs are ready to be stored.  If the post says the tensor takes another round, the
+// wavefront does its quarter of that chunk again first, from the inputs it is about to overwrite (the same lanes
+// read there that write there afterwards).  The tensors at the end of the walk, which nobody overwrites, are left to
+// fused_shift_scales_kernel and fused_shift_tail_kernel.  The next step walks the other way and moves everything
+// back.  Extra memory: `slack` chunks per arena instead of a second copy.
 //
 // What crosses between workgroups, and how, without a fence (a release or acquire at agent scope writes back or
-// invalidates a whole L2 on this part, which one workgroup in sixty thousand can afford and every workgroup cannot):
-//  * the maxima and the counter are agent-scope atomics; the counter's increment takes the returned old maxima as an
-//    operand, so it is issued only when those atomics have been performed;
-//  * a post is one 8-byte agent-scope store of {token, value}: whoever reads this call's token beside a value reads
-//    that value;
-//  * payload stores are written through (put16 / put1 with THRU) and every wave waits for its own before the
-//    workgroup's barrier, so a chunk is in memory before its workgroup counts it -- and before any workgroup that then
-//    writes the same places a second time (the other round, possibly from another die) issues its stores;
+// invalidates a whole L2 on this part), without an atomic that every workgroup would have to take in turn, and
+// without a workgroup barrier (the wavefronts of a workgroup come and go on their own):
+//  * a maximum goes out as an agent-scope atomic, only where it raises the word, and the wavefront's mark takes the
+//    returned values as an operand, so it is issued only when those atomics have been performed;
+//  * a mark or a post is one agent-scope store of this call's token, or of {token, value}: whoever reads the token
+//    beside a value reads that value;
+//  * payload stores are written through (THRU) and a wavefront waits for its own before it marks, so its part of the
+//    chunk is in memory before the mark -- and before anybody who then writes the same places a second time (the
+//    other round, possibly from another die) issues its stores;
 //  * inputs are read with ordinary loads: nothing writes them during the launch until their own overwriting.
+constexpr int kWavesPerChunk = kAdamThreads / kWave;
+// sync buffer of a call, in 8-byte words: per tensor kShiftPostWords post words; then per chunk one verdict word
+// {token, another round?} (what the wavefronts about to overwrite that chunk read: one word per chunk, so that no single
+// address is asked for by a whole tensor's wavefronts); then per chunk and wavefront kMarkWords mark words
+// {token, max |p'|}, {token, max |m'|}, {token, max |v'|} (a wavefront's maxima travel in its marks: no atomics)
+constexpr int kMarkWords = 4;
 struct ShiftArgs {
     long long shift;        // output element = input element + shift (its sign is the direction of the walk)
     int slack;              // |shift| in chunks
+    int lead;               // how many chunks ahead of a tensor's first overwriting its outcome is decided
     int n_chunks;
+    int n_tensors;
     uint32_t token;
     uint32_t spin_limit;
     uint32_t* error_word;
     int32_t* redo;
     uint64_t* posts;        // kShiftPostWords words per tensor
+    uint64_t* verdicts;     // one word per chunk
+    uint64_t* marks;        // kWavesPerChunk * kMarkWords words per chunk
     float w_fp_max;
     int tensor_scale;
 };
@@ -685,13 +861,16 @@ constexpr int kShiftPostWords = MSAMP_ADAMW_POST_WORDS;
 __device__ __forceinline__ void post_word(uint64_t* p, uint32_t token, uint32_t value) {
     __hip_atomic_store(p, (static_cast<uint64_t>(token) << 32) | value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ bool anybody_gave_up(const ShiftArgs& a) {
+    return __hip_atomic_load(a.error_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+}
 // the value posted beside this call's token; `ok` is cleared if it does not show up within the limit
 __device__ __forceinline__ uint32_t await_post(const uint64_t* p, const ShiftArgs& a, bool& ok) {
     for (uint32_t spins = 0; ok; ++spins) {
         const uint64_t w = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (static_cast<uint32_t>(w >> 32) == a.token) return static_cast<uint32_t>(w);
         // the limit, or somebody else has given up already: nobody waits any longer
-        if (spins >= a.spin_limit || __hip_atomic_load(a.error_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) ok = false;
+        if (spins >= a.spin_limit || anybody_gave_up(a)) ok = false;
         else __builtin_amdgcn_s_sleep(8);
     }
     return 0u;
@@ -703,113 +882,298 @@ __device__ __forceinline__ void* shifted_weight(void* p, long long shift) {
     else return static_cast<uint8_t*>(p) + shift;
 }
 
-// what fused_scales_kernel does, for one tensor, by the workgroup that stored the tensor's last chunk
-__device__ __forceinline__ void decide_tensor(msamp_adamw_tensor& d, int t, const ShiftArgs& a) {
-    const float ap = __uint_as_float(__hip_atomic_load(&d.acc[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    const float am = __uint_as_float(__hip_atomic_load(&d.acc[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    const float av = __uint_as_float(__hip_atomic_load(&d.acc[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    // left at zero for the next step (atomic stores: the words are only ever touched at that level)
-    __hip_atomic_store(&d.acc[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&d.acc[1], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&d.acc[2], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&d.reserved[0], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const float old_ws = *d.w_scale, old_ms = *d.m_scale, old_vs = *d.v_scale;
-    const float old_wsi = *d.w_scale_inv, old_inv_m = 1.0f / old_ms, old_inv_v = 1.0f / old_vs;
-    d.saved[0] = old_wsi, d.saved[1] = old_inv_m, d.saved[2] = old_inv_v;
-    const float ws = scale_rule(ap, old_ws, a.w_fp_max, 0);
-    const float ms = a.tensor_scale ? scale_rule(am, 1.0f, 448.0f, 0) : 1.0f;
-    const float vs = a.tensor_scale ? scale_rule(av, 1.0f, 65504.0f, 0) : 1.0f;
-    const uint32_t again = (__float_as_uint(ws) != __float_as_uint(old_ws) || __float_as_uint(ms) != __float_as_uint(old_ms) ||
-                            __float_as_uint(vs) != __float_as_uint(old_vs))
-                               ? 1u
-                               : 0u;
-    // for the kernels and the host that come after this launch
-    a.redo[t] = static_cast<int32_t>(again);
-    *d.w_scale = ws;
-    *d.w_scale_inv = 1.0f / ws;
-    *d.w_amax = ap;
-    *d.m_scale = ms;
-    *d.m_scale_inv = 1.0f / ms;
-    *d.m_amax = am;
-    *d.v_scale = vs;
-    *d.v_scale_inv = 1.0f / vs;
-    *d.v_amax = av;
-    // for the workgroups of this launch that will overwrite this tensor's chunks
-    uint64_t* post = a.posts + static_cast<size_t>(t) * kShiftPostWords;
-    if (again) {
-        post_word(post + 1, a.token, __float_as_uint(old_wsi));
-        post_word(post + 2, a.token, __float_as_uint(old_inv_m));
-        post_word(post + 3, a.token, __float_as_uint(old_inv_v));
-        post_word(post + 4, a.token, __float_as_uint(ws));
-        post_word(post + 5, a.token, __float_as_uint(ms));
-        post_word(post + 6, a.token, __float_as_uint(vs));
+// The maxima of a tensor from the marks of its wavefronts, gathered by a whole workgroup (valid in its first lane);
+// returns false if a mark of this call does not show up within the limit.  first_chunk: index of the tensor's first
+// chunk in the launch.  Every lane asks for all its marks at once, a dozen loads in flight: this sits between a
+// tensor and everybody who writes over it.
+__device__ __forceinline__ bool gather_marks(const ShiftArgs& a, int first_chunk, int chunks, uint32_t* red, uint32_t& mp,
+                                             uint32_t& mm, uint32_t& mv) {
+    const uint64_t* marks = a.marks + static_cast<size_t>(first_chunk) * (kWavesPerChunk * kMarkWords);
+    const int n_waves = chunks * kWavesPerChunk;
+    mp = 0, mm = 0, mv = 0;
+    bool mine = true;
+    constexpr int kBatch = 4;    // wavefronts per lane and round: 12 loads in flight
+    for (int w0 = threadIdx.x; w0 < n_waves; w0 += kAdamThreads * kBatch) {
+        uint64_t word[kBatch][3];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int w = w0 + u * kAdamThreads;
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+                word[u][i] = w < n_waves ? __hip_atomic_load(marks + static_cast<size_t>(w) * kMarkWords + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                                         : (static_cast<uint64_t>(a.token) << 32);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int w = w0 + u * kAdamThreads;
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                // not there yet (rare: the tensor has only just been finished): wait for it
+                for (uint32_t spins = 0; static_cast<uint32_t>(word[u][i] >> 32) != a.token; ++spins) {
+                    if (spins >= a.spin_limit || anybody_gave_up(a)) {
+                        mine = false;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(8);
+                    word[u][i] = __hip_atomic_load(marks + static_cast<size_t>(w) * kMarkWords + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            mp = umax(mp, static_cast<uint32_t>(word[u][0])), mm = umax(mm, static_cast<uint32_t>(word[u][1]));
+            mv = umax(mv, static_cast<uint32_t>(word[u][2]));
+        }
     }
-    post_word(post, a.token, again);
+    const bool all = __syncthreads_and(mine) != 0;
+    mp = block_max_u32(mp, red), mm = block_max_u32(mm, red), mv = block_max_u32(mv, red);
+    return all;
+}
+
+// What fused_scales_kernel does, for one tensor whose maxima are known to the workgroup's first lane (the whole
+// workgroup comes here).  in_launch: also tell the wavefronts of this launch that will overwrite the tensor's chunks --
+// the factors another round needs in the tensor's post words, the verdict in every chunk's own word.
+__device__ __forceinline__ void decide_tensor(msamp_adamw_tensor& d, int t, const ShiftArgs& a, int first_chunk, int chunks,
+                                              uint32_t mp, uint32_t mm, uint32_t mv, bool in_launch, uint32_t* red) {
+    if (threadIdx.x == 0) {
+        const float ap = __uint_as_float(mp), am = __uint_as_float(mm), av = __uint_as_float(mv);
+        const float old_ws = *d.w_scale, old_ms = *d.m_scale, old_vs = *d.v_scale;
+        const float old_wsi = *d.w_scale_inv, old_inv_m = 1.0f / old_ms, old_inv_v = 1.0f / old_vs;
+        d.saved[0] = old_wsi, d.saved[1] = old_inv_m, d.saved[2] = old_inv_v;
+        const float ws = scale_rule(ap, old_ws, a.w_fp_max, 0);
+        const float ms = a.tensor_scale ? scale_rule(am, 1.0f, 448.0f, 0) : 1.0f;
+        const float vs = a.tensor_scale ? scale_rule(av, 1.0f, 65504.0f, 0) : 1.0f;
+        const uint32_t again = (__float_as_uint(ws) != __float_as_uint(old_ws) || __float_as_uint(ms) != __float_as_uint(old_ms) ||
+                                __float_as_uint(vs) != __float_as_uint(old_vs))
+                                   ? 1u
+                                   : 0u;
+        red[0] = again;
+        // for the kernels and the host that come after this launch
+        a.redo[t] = static_cast<int32_t>(again);
+        *d.w_scale = ws;
+        *d.w_scale_inv = 1.0f / ws;
+        *d.w_amax = ap;
+        *d.m_scale = ms;
+        *d.m_scale_inv = 1.0f / ms;
+        *d.m_amax = am;
+        *d.v_scale = vs;
+        *d.v_scale_inv = 1.0f / vs;
+        *d.v_amax = av;
+        uint64_t* post = a.posts + static_cast<size_t>(t) * kShiftPostWords;
+        if (in_launch && again) {
+            post_word(post + 1, a.token, __float_as_uint(old_wsi));
+            post_word(post + 2, a.token, __float_as_uint(old_inv_m));
+            post_word(post + 3, a.token, __float_as_uint(old_inv_v));
+            post_word(post + 4, a.token, __float_as_uint(ws));
+            post_word(post + 5, a.token, __float_as_uint(ms));
+            post_word(post + 6, a.token, __float_as_uint(vs));
+        }
+        post_word(post, a.token, again);    // also what tells fused_shift_scales_kernel that the tensor is settled
+    }
+    if (in_launch) {
+        __syncthreads();
+        const uint32_t again = red[0];
+        for (int c = threadIdx.x; c < chunks; c += kAdamThreads) post_word(a.verdicts + first_chunk + c, a.token, again);
+    }
+}
+
+// This wavefront's quarter of the other round of one chunk: what write_chunk does, by the same element functions, in
+// the groups of eight of the speculative pass (whose registers it shares here), written through.  f: the old weight
+// scale_inv, the old reciprocal moment scales, the new weight and moment scales.
+template <int WDT, int GDT, bool L2>
+__device__ __forceinline__ void redo_quarter(const msamp_adamw_tensor& d, int chunk, long long shift, const float (&f)[6],
+                                             const AdamConsts& k) {
+    void* w_out = shifted_weight<WDT>(d.weight, shift);
+    uint8_t* m_out = d.exp_avg + shift;
+    uint16_t* v_out = d.exp_avg_sq + shift;
+    const float g_si0 = *d.g_scale_inv, g_si = k.maximize ? -g_si0 : g_si0;
+    const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
+    SpecState unused;
+    if (base + MSAMP_ADAMW_CHUNK <= d.numel) {
+#pragma unroll 1
+        for (int s = 0; s < 2 * kSpecSteps; ++s) {
+            const size_t i = base + static_cast<size_t>(s) * kGroupSpan + threadIdx.x * kGroup;
+            Raw8<WDT> rw, ow;
+            Raw8<GDT> rg;
+            Raw8<MSAMP_DT_E4M3> rm, om;
+            Raw8<MSAMP_DT_F16> rv, ov;
+            rw.load(d.weight, i), rg.load(d.grad, i), rm.load(d.exp_avg, i), rv.load(d.exp_avg_sq, i);
+            spec_group<WDT, GDT, L2, false>(d, i, rw, rg, rm, rv, f[0], g_si, f[1], f[2], f[3], f[4], f[5], k, unused, ow, om, ov);
+            ow.template store<true>(w_out, i), om.template store<true>(m_out, i), ov.template store<true>(v_out, i);
+        }
+    } else {
+        for (size_t i = base + threadIdx.x; i < d.numel; i += kAdamThreads) {
+            const float m_old = load_w1<MSAMP_DT_E4M3>(d.exp_avg, i), v_old = load_w1<MSAMP_DT_F16>(d.exp_avg_sq, i);
+            float pj, g_plain, m_new, v_new;
+            prepare<L2>(load_w1<WDT>(d.weight, i), load_w1<GDT>(d.grad, i), m_old, v_old, f[0], g_si, f[1], f[2], k, pj, g_plain,
+                        m_new, v_new);
+            store_one<WDT, true>(w_out, i, param_update(pj, m_new, v_new, k) * f[3]);
+            if constexpr (L2) moments(m_old, v_old, g_plain, f[1], f[2], k, m_new, v_new);
+            store_one<MSAMP_DT_E4M3, true>(m_out, i, m_new * f[4]);
+            store_one<MSAMP_DT_F16, true>(v_out, i, v_new * f[5]);
+        }
+    }
 }
 
 template <int WDT, int GDT, bool L2>
 __global__ __launch_bounds__(kAdamThreads) void fused_shift_kernel(msamp_adamw_tensor* __restrict__ tensors,
                                                                     const int32_t* __restrict__ block_map, AdamConsts k,
                                                                     ShiftArgs a) {
-    __shared__ uint32_t red[kAdamThreads / kWave];
-    __shared__ int s_verdict;
-    __shared__ float s_factor[6];
     const int b = blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const bool up = a.shift > 0;    // moving up: walk from the top, so that the room is always ahead
     const int j = up ? a.n_chunks - 1 - b : b;
     const int t = block_map[2 * j], chunk = block_map[2 * j + 1];
-    if (b >= a.slack) {
-        // the chunk that lies where this one's outputs go
-        const int jv = up ? j + a.slack : j - a.slack;
-        const int tv = block_map[2 * jv], cv = block_map[2 * jv + 1];
-        if (threadIdx.x == 0) {
-            int verdict = -1;
-            if (tv == t) {
-                // a tensor longer than the room: the layout is not what this kernel needs
-                report_wait_expired(a.error_word, kErrShiftLayout);
-            } else {
-                const uint64_t* post = a.posts + static_cast<size_t>(tv) * kShiftPostWords;
-                bool ok = true;
-                const uint32_t again = await_post(post, a, ok);
-                if (ok && again) {
-#pragma unroll
-                    for (int i = 0; i < 6; ++i) s_factor[i] = __uint_as_float(await_post(post + 1 + i, a, ok));
-                }
-                if (ok) verdict = static_cast<int>(again);
-                else report_wait_expired(a.error_word, kErrShiftGaveUp);
+    // the chunk that lies where this one's outputs go, if any
+    const bool overwrites = b >= a.slack;
+    const int jv = overwrites ? (up ? j + a.slack : j - a.slack) : j;
+    const int tv = block_map[2 * jv], cv = block_map[2 * jv + 1];
+    msamp_adamw_tensor& d = tensors[t];
+    msamp_adamw_tensor& dv = tensors[tv];
+    const uint64_t* post = a.posts + static_cast<size_t>(tv) * kShiftPostWords;
+    // Who decides a tensor's outcome: the workgroup `lead` chunks ahead of the one that overwrites the tensor's first chunk
+    // (in the order of the walk), so that the outcome is posted by the time anybody needs it -- if the tensor is short
+    // enough to lie wholly before that workgroup; else the workgroup that overwrites its first chunk.
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    auto decides_ahead = [&](int chunks) { return chunks <= a.slack - a.lead; };
+    auto decide = [&](int jt) {    // jt: index of any chunk of the tensor
+        const int tt = block_map[2 * jt], first = jt - block_map[2 * jt + 1];
+        msamp_adamw_tensor& dt = tensors[tt];
+        const int chunks_t = static_cast<int>((dt.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK);
+        uint32_t gp, gm, gv;
+        if (gather_marks(a, first, chunks_t, red, gp, gm, gv)) decide_tensor(dt, tt, a, first, chunks_t, gp, gm, gv, true, red);
+        else if (threadIdx.x == 0) report_wait_expired(a.error_word, kErrShiftGaveUp);
+    };
+    auto first_walked = [&](int jt) {    // is this the chunk of its tensor that the walk meets first?
+        const int ct = block_map[2 * jt + 1];
+        if (!up) return ct == 0;
+        const msamp_adamw_tensor& dt = tensors[block_map[2 * jt]];
+        return ct == static_cast<int>((dt.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK) - 1;
+    };
+    {
+        const int q = b - (a.slack - a.lead);    // position in the walk of the chunk overwritten `lead` workgroups from here
+        if (a.lead > 0 && q >= 0) {
+            const int jq = up ? a.n_chunks - 1 - q : q;
+            if (first_walked(jq)) {
+                const msamp_adamw_tensor& dq = tensors[block_map[2 * jq]];
+                if (decides_ahead(static_cast<int>((dq.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK))) decide(jq);
             }
-            s_verdict = verdict;
-        }
-        __syncthreads();
-        // gave up: this chunk is left as it was (the call has failed; the error word says so)
-        if (s_verdict < 0) return;
-        if (s_verdict > 0) {
-            msamp_adamw_tensor& dv = tensors[tv];
-            const float g_si0 = *dv.g_scale_inv, g_si = k.maximize ? -g_si0 : g_si0;
-            write_chunk<WDT, GDT, L2, true>(dv, cv, shifted_weight<WDT>(dv.weight, a.shift), dv.exp_avg + a.shift,
-                                            dv.exp_avg_sq + a.shift, s_factor[0], g_si, s_factor[1], s_factor[2], s_factor[3],
-                                            s_factor[4], s_factor[5], k);
-            // its loads are through (they fed its stores) before this chunk's outputs land on what they read
-            __syncthreads();
         }
     }
-    msamp_adamw_tensor& d = tensors[t];
-    uint32_t mp, mm, mv;
-    spec_chunk<WDT, GDT, L2, true>(d, chunk, shifted_weight<WDT>(d.weight, a.shift), d.exp_avg + a.shift, d.exp_avg_sq + a.shift, k,
-                                   red, mp, mm, mv);
-    if (threadIdx.x == 0) {
-        const uint32_t chunks = static_cast<uint32_t>((d.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK);
-        // the maxima first; their returned values are an operand of the count, which is therefore issued after them
-        const uint32_t o0 = atomicMax(&d.acc[0], mp), o1 = atomicMax(&d.acc[1], mm), o2 = atomicMax(&d.acc[2], mv);
-        uint32_t one = 1u;
-        asm volatile("" : "+v"(one) : "v"(o0), "v"(o1), "v"(o2));
-        const uint32_t count = atomicAdd(&d.reserved[0], one);
-        if (count == chunks - 1) decide_tensor(d, t, a);
+    uint64_t posted = 0;    // first lane: what the verdict word of the chunk underneath held when this wavefront started
+    if (overwrites) {
+        if (tv == t) {
+            // a tensor longer than the room: the layout is not what this kernel needs
+            if (threadIdx.x == 0) report_wait_expired(a.error_word, kErrShiftLayout);
+            return;
+        }
+        const int chunks_v = static_cast<int>((dv.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK);
+        if (first_walked(jv) && !(a.lead > 0 && decides_ahead(chunks_v))) decide(jv);
+    }
+
+    void* w_out = shifted_weight<WDT>(d.weight, a.shift);
+    uint8_t* m_out = d.exp_avg + a.shift;
+    uint16_t* v_out = d.exp_avg_sq + a.shift;
+    const size_t base = static_cast<size_t>(chunk) * MSAMP_ADAMW_CHUNK;
+    const float w_si = *d.w_scale_inv, g_si = k.maximize ? -*d.g_scale_inv : *d.g_scale_inv;
+    const float ws = *d.w_scale, ms = *d.m_scale, vs = *d.v_scale;    // the guess: the scales in force
+    const float inv_m = 1.0f / ms, inv_v = 1.0f / vs;
+    SpecState st;
+    st.mxp = 0, st.mxm = 0.0f, st.mxv = 0.0f, st.floor_p = 0.0f;
+
+    // Before this wavefront's first store: what became of the tensor underneath.  Returns 0 = go on, 1 = its chunk
+    // has just been done again by these lanes (whatever they held is gone), negative = gave up.
+    bool gate_open = !overwrites;
+    auto gate = [&]() -> int {
+        int verdict = 0;
+        float f[6] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        if (lane == 0) {
+            bool ok = true;
+            const uint32_t again = static_cast<uint32_t>(posted >> 32) == a.token ? static_cast<uint32_t>(posted) : await_post(a.verdicts + jv, a, ok);
+            if (ok && again) {
+#pragma unroll
+                for (int i = 0; i < 6; ++i) f[i] = __uint_as_float(await_post(post + 1 + i, a, ok));
+            }
+            if (!ok) report_wait_expired(a.error_word, kErrShiftGaveUp);
+            verdict = ok ? static_cast<int>(again) : -1;
+        }
+        verdict = __builtin_amdgcn_readfirstlane(verdict);
+        if (verdict > 0) {
+#pragma unroll
+            for (int i = 0; i < 6; ++i) f[i] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(f[i])));
+            redo_quarter<WDT, GDT, L2>(dv, cv, a.shift, f, k);
+            // A whole chunk and a partly filled one are shared out among the lanes differently: if one of the two chunks
+            // is of each kind, these lanes' outputs land on what other wavefronts of the workgroup read for the other
+            // round, and all four must be through with it first (all four come here: the verdict is the tensor's).
+            const bool own_whole = base + MSAMP_ADAMW_CHUNK <= d.numel;
+            const bool other_whole = static_cast<size_t>(cv) * MSAMP_ADAMW_CHUNK + MSAMP_ADAMW_CHUNK <= dv.numel;
+            if (own_whole != other_whole) __syncthreads();
+        }
+        return verdict;
+    };
+
+    if (base + MSAMP_ADAMW_CHUNK <= d.numel) {
+#pragma unroll 1
+        for (int s = 0; s < kSpecSteps;) {
+            const size_t i0 = base + static_cast<size_t>(s) * (2 * kGroupSpan) + threadIdx.x * kGroup, i1 = i0 + kGroupSpan;
+            Raw8<WDT> w0, w1, ow;
+            Raw8<GDT> g0, g1;
+            Raw8<MSAMP_DT_E4M3> m0, m1, om;
+            Raw8<MSAMP_DT_F16> v0, v1, ov;
+            w0.load(d.weight, i0), g0.load(d.grad, i0), m0.load(d.exp_avg, i0), v0.load(d.exp_avg_sq, i0);
+            w1.load(d.weight, i1), g1.load(d.grad, i1), m1.load(d.exp_avg, i1), v1.load(d.exp_avg_sq, i1);
+            // the verdict on the chunk underneath: asked for behind this wavefront's own loads (it comes from further away
+            // than they do, and loads return in order), looked at when the first outputs are ready
+            if (!gate_open && lane == 0) posted = __hip_atomic_load(a.verdicts + jv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const SpecState before = st;
+            spec_group<WDT, GDT, L2>(d, i0, w0, g0, m0, v0, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, st, ow, om, ov);
+            if (!gate_open) {
+                const int verdict = gate();
+                // gave up: this chunk is left as it was; the call has failed and the error word says so
+                if (verdict < 0) return;
+                gate_open = true;
+                if (verdict > 0) {    // start the step again
+                    st = before;
+                    continue;
+                }
+            }
+            ow.template store<true>(w_out, i0), om.template store<true>(m_out, i0), ov.template store<true>(v_out, i0);
+            spec_group<WDT, GDT, L2>(d, i1, w1, g1, m1, v1, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, st, ow, om, ov);
+            ow.template store<true>(w_out, i1), om.template store<true>(m_out, i1), ov.template store<true>(v_out, i1);
+            ++s;
+        }
+    } else {
+        // the tensor's last, partly filled chunk: element by element, a lane's elements the same in both rounds
+        if (!gate_open && gate() < 0) return;
+        spec_ragged<WDT, GDT, L2, true>(d, base + threadIdx.x, kAdamThreads, w_out, m_out, v_out, w_si, g_si, inv_m, inv_v, ws, ms, vs,
+                                        k, st);
+    }
+    // this wavefront's stores have arrived before anything its first lane publishes
+    __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0)
+    const uint32_t mp = wave_max_u32(st.mxp), mm = wave_max_u32(__float_as_uint(st.mxm)), mv = wave_max_u32(__float_as_uint(st.mxv));
+    if (lane == 0) {
+        uint64_t* mark = a.marks + (static_cast<size_t>(j) * kWavesPerChunk + wave) * kMarkWords;
+        post_word(mark, a.token, mp);
+        post_word(mark + 1, a.token, mm);
+        post_word(mark + 2, a.token, mv);
     }
 }
 
+// after the walk: the tensors nobody has decided (their first chunk lies where nothing is written over it); one
+// workgroup per tensor, found through its first chunk in the block map
+__global__ __launch_bounds__(kAdamThreads) void fused_shift_scales_kernel(msamp_adamw_tensor* tensors, const int32_t* block_map,
+                                                                           ShiftArgs a) {
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    const int j = blockIdx.x;
+    if (block_map[2 * j + 1] != 0) return;
+    const int t = block_map[2 * j];
+    if (static_cast<uint32_t>(a.posts[static_cast<size_t>(t) * kShiftPostWords] >> 32) == a.token) return;
+    msamp_adamw_tensor& d = tensors[t];
+    const int chunks = static_cast<int>((d.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK);
+    uint32_t gp, gm, gv;
+    if (gather_marks(a, j, chunks, red, gp, gm, gv)) decide_tensor(d, t, a, j, chunks, gp, gm, gv, false, red);
+    else if (threadIdx.x == 0) report_wait_expired(a.error_word, kErrShiftGaveUp);
+}
+
 // the last `slack` chunks of the walk: nothing is written over them, so nobody has looked at their tensors' marks
-// (a launch of its own: everything the first one stored is in memory by now, ordinary loads do)
+// (a launch of its own: everything the earlier ones stored is in memory by now, ordinary loads and stores do)
 template <int WDT, int GDT, bool L2>
 __global__ __launch_bounds__(kAdamThreads) void fused_shift_tail_kernel(msamp_adamw_tensor* __restrict__ tensors,
                                                                          const int32_t* __restrict__ block_map, AdamConsts k,
@@ -1029,14 +1393,14 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
     MSAMP_CHECK_LAUNCH("fused_write_kernel");
     return MSAMP_OK;
 }
-int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, uint64_t* posts, int n_tensors,
-                                const int32_t* block_map, int n_blocks, long long shift_elems, int weight_dtype, int grad_dtype,
-                                double lr, double beta1, double beta2, double eps, double weight_decay, int step,
-                                int bias_correction, int adam_mode, int maximize, int tensor_scale, void* workspace,
-                                msamp_stream_t stream) {
+int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, void* sync, int n_tensors, const int32_t* block_map,
+                                int n_blocks, long long shift_elems, int weight_dtype, int grad_dtype, double lr, double beta1,
+                                double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
+                                int maximize, int tensor_scale, void* workspace, msamp_stream_t stream) {
     const int rc = fused_args_ok("msamp_adamw_fp8_fused_shift", tensors, n_tensors, block_map, n_blocks, weight_dtype, grad_dtype);
     if (rc != MSAMP_OK || n_tensors == 0 || n_blocks == 0) return rc;
-    MSAMP_REQUIRE(redo != nullptr && posts != nullptr, MSAMP_ERR_NULL, "msamp_adamw_fp8_fused_shift: null redo or posts");
+    MSAMP_REQUIRE(redo != nullptr && sync != nullptr, MSAMP_ERR_NULL, "msamp_adamw_fp8_fused_shift: null redo or sync");
+    MSAMP_REQUIRE(aligned(sync, 8), MSAMP_ERR_ALIGNMENT, "msamp_adamw_fp8_fused_shift: sync must be 8-byte aligned");
     MSAMP_REQUIRE(workspace != nullptr, MSAMP_ERR_WORKSPACE, "msamp_adamw_fp8_fused_shift: workspace required");
     const long long mag = shift_elems < 0 ? -shift_elems : shift_elems;
     MSAMP_REQUIRE(mag > 0 && mag % MSAMP_ADAMW_CHUNK == 0 && mag / MSAMP_ADAMW_CHUNK <= 0x7fffffffLL, MSAMP_ERR_SHAPE,
@@ -1047,16 +1411,22 @@ int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, uint
     ShiftArgs a;
     a.shift = shift_elems;
     a.slack = static_cast<int>(mag / MSAMP_ADAMW_CHUNK);
+    a.lead = a.slack / 2 < 512 ? a.slack / 2 : 512;
     a.n_chunks = n_blocks;
+    a.n_tensors = n_tensors;
     a.token = next_tokens(1);
     a.spin_limit = collector_spin_limit();
     a.error_word = static_cast<uint32_t*>(workspace) + kWsErrorWord;
     a.redo = redo;
-    a.posts = posts;
+    a.posts = static_cast<uint64_t*>(sync);
+    a.verdicts = a.posts + static_cast<size_t>(n_tensors) * kShiftPostWords;
+    a.marks = a.verdicts + n_blocks;
     a.w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
     a.tensor_scale = tensor_scale;
     FUSED_LAUNCH(fused_shift_kernel, n_blocks, tensors, block_map, k, a);
     MSAMP_CHECK_LAUNCH("fused_shift_kernel");
+    hipLaunchKernelGGL(fused_shift_scales_kernel, dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, a);
+    MSAMP_CHECK_LAUNCH("fused_shift_scales_kernel");
     const int tail = n_blocks < a.slack ? n_blocks : a.slack;
     FUSED_LAUNCH(fused_shift_tail_kernel, tail, tensors, block_map, k, a);
     MSAMP_CHECK_LAUNCH("fused_shift_tail_kernel");

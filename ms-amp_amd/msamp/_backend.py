@@ -727,24 +727,29 @@ def adamw_fused_speculative(desc, outputs, redo, n_tensors, block_map, n_blocks,
 ADAMW_POST_WORDS = 8
 
 
-def adamw_fused_shift(desc, redo, posts, n_tensors, block_map, n_blocks, shift_elems, weight_dt, grad_dt, lr, beta1, beta2, eps,
+def adamw_shift_sync_bytes(n_tensors, n_blocks):
+    """Size of the `sync` buffer of adamw_fused_shift (MSAMP_ADAMW_SYNC_BYTES)."""
+    return n_tensors * ADAMW_POST_WORDS * 8 + n_blocks * 136
+
+
+def adamw_fused_shift(desc, redo, sync, n_tensors, block_map, n_blocks, shift_elems, weight_dt, grad_dt, lr, beta1, beta2, eps,
                       weight_decay, step, bias_correction, adam_mode, maximize, tensor_scale):
     """The fused step in one pass inside shifting arenas: every tensor's new payloads land `shift_elems` elements away
     from the old ones (see msamp_adamw_fp8_fused_shift for the layout this needs).  `redo`: int32 device tensor
-    [n_tensors], set by the call where a tensor took the second round; `posts`: int64 device tensor [n_tensors,
-    ADAMW_POST_WORDS], zeroed once, the kernels' own."""
+    [n_tensors], set by the call where a tensor took the second round; `sync`: uint8 device tensor of
+    adamw_shift_sync_bytes(n_tensors, n_blocks) bytes, zeroed once, the kernels' own."""
     lib = load()
     _gpu(desc, 'descriptor table')
     _gpu(redo, 'redo flags')
     if redo.dtype != torch.int32 or redo.numel() != n_tensors or not redo.is_contiguous():
         raise ValueError('redo must be a contiguous int32 tensor of n_tensors flags')
-    _gpu(posts, 'post words')
-    if posts.dtype != torch.int64 or posts.numel() != n_tensors * ADAMW_POST_WORDS or not posts.is_contiguous():
-        raise ValueError('posts must be a contiguous int64 tensor of n_tensors x %d words' % ADAMW_POST_WORDS)
+    _gpu(sync, 'sync buffer')
+    if sync.numel() * sync.element_size() < adamw_shift_sync_bytes(n_tensors, n_blocks) or not sync.is_contiguous():
+        raise ValueError('sync must be a contiguous buffer of at least %d bytes' % adamw_shift_sync_bytes(n_tensors, n_blocks))
     _check(
         lib.msamp_adamw_fp8_fused_shift(
-            _ptr(desc), _ptr(redo), _ptr(posts), n_tensors, _ptr(block_map), n_blocks, int(shift_elems), weight_dt, grad_dt, lr, beta1, beta2,
-            eps, weight_decay, step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0,
+            _ptr(desc), _ptr(redo), _ptr(sync), n_tensors, _ptr(block_map), n_blocks, int(shift_elems), weight_dt, grad_dt, lr,
+            beta1, beta2, eps, weight_decay, step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0,
             1 if tensor_scale else 0, _ptr(workspace(desc.device)), _stream()
         ), 'msamp_adamw_fp8_fused_shift'
     )

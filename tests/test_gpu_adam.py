@@ -330,8 +330,8 @@ def _fused_shift(be, tensors, w_dt, g_dt, step, slack, up, check_clean=True, **k
     hyper = dict(HYPER)
     hyper.update(kw)
     redo = torch.full((len(dev), ), -1, dtype=torch.int32, device='cuda')
-    posts = torch.zeros(len(dev), be.ADAMW_POST_WORDS, dtype=torch.int64, device='cuda')
-    be.adamw_fused_shift(desc, redo, posts, len(tensors), block_map, total, (slack if up else -slack) * ch, w_dt, g_dt, hyper['lr'],
+    sync = torch.zeros(be.adamw_shift_sync_bytes(len(dev), total), dtype=torch.uint8, device='cuda')
+    be.adamw_fused_shift(desc, redo, sync, len(tensors), block_map, total, (slack if up else -slack) * ch, w_dt, g_dt, hyper['lr'],
                          hyper['beta1'], hyper['beta2'], hyper['eps'], hyper['weight_decay'], step,
                          hyper.get('bias_correction', True), hyper.get('adam_mode', False), hyper.get('maximize', False),
                          hyper.get('tensor_scale', True))
@@ -342,7 +342,6 @@ def _fused_shift(be, tensors, w_dt, g_dt, step, slack, up, check_clean=True, **k
         d['redo'] = r
     if check_clean:    # accumulators and counters of the descriptors are left zeroed
         assert (desc[:, 15].cpu() == 0).all() and (desc[:, 16].cpu() & 0xffffffff == 0).all()
-        assert (desc[:, 18].cpu() & 0xffffffff == 0).all()
     return dev
 
 
