@@ -18,25 +18,79 @@ from msamp.optim.adamw_base import LBAdamWBase
 _FUSED_WEIGHT_QTYPES = (Dtypes.kfloat8_e4m3, Dtypes.kfloat8_e5m2, Dtypes.kfloat16)
 
 
+class _FusedPlan:
+    """What one group of fusable parameters needs from step to step: the device tables of the fused kernels and, for
+    the one-pass forms, where the payloads live."""
+    def __init__(self):
+        self.params = ()           # ids of the parameters, in order
+        self.static_sig = None     # addresses that only a rebuild changes (metas of weight and moments)
+        self.sig = None            # addresses that may change between steps (payloads, gradient, its scale_inv)
+        self.desc = None           # [n, ADAMW_DESC_WORDS] int64 on the device (one per phase for the moving forms)
+        self.block_map = None
+        self.n_blocks = 0
+        self.chunks = None
+        self.stage = None          # pinned staging rows for the columns that change
+        # shifting arenas
+        self.arenas = None         # {'w','m','v'}: uint8 tensors
+        self.views = None          # [phase][tensor] -> (w, m, v) views
+        self.phase = 0             # 0: payloads at the top (the room below), 1: at the bottom
+        self.slack = 0
+        self.widths = (1, 1, 2)    # bytes per element of the weight, exp_avg and exp_avg_sq payloads
+        self.redo = None
+        self.sync = None
+        # two sets of buffers
+        self.spare = None
+        self.outputs = None
+
+
 class LBAdamW(LBAdamWBase):
     """AdamW with low-bit moments (default: E4M3 exp_avg, scaled-fp16 exp_avg_sq)."""
     def __init__(self, params, lr=1e-3, bias_correction=True, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2,
                  amsgrad=False, *, maximize=False, exp_avg_dtype=torch.uint8, exp_avg_sq_dtype=torch.float16,
-                 tensor_scale=True, double_buffer=True):
-        """double_buffer (not in the reference): the fused step writes the new weight and moment payloads into a second
-        set of buffers (4 more bytes per parameter) and swaps the two sets afterwards, which lets it read every tensor
-        once instead of twice; the values are the same bit for bit.  The payload tensors (`.value`) remain the same
-        objects, but their memory alternates between two addresses: pass False when something holds those addresses
-        (a captured graph of the forward pass, views taken of `.value`).  Payloads that are themselves views of other
-        storage (a flat buffer) and steps taken under stream capture keep the in-place step."""
+                 tensor_scale=True, one_pass=None, double_buffer=False):
+        """one_pass (not in the reference) selects how the fused step gets at its data; the values are the same bit for
+        bit in every form:
+
+        None (default): in place, as the reference's optimizer works: every payload keeps its address; the step reads
+            every tensor twice (the scales of the new values are only known after a full pass), 14 bytes of memory
+            traffic per parameter.
+        'shift': the optimizer moves the payloads of weights and moments into three arenas of its own, with a little
+            room at one end (a few thousand 16 Ki-element chunks: about 0.3 bytes per parameter for a billion
+            parameters), and every step writes the new payloads that much further along, alternately down and up.
+            The step then reads every tensor once (9 bytes per parameter).  The payload tensors (`.value`) remain the
+            same objects, but their memory alternates between two addresses from step to step.
+        'double': the step writes into a second set of payload buffers (4 more bytes per parameter) and the two sets
+            trade places; one pass as well, and the addresses alternate as well.
+
+        Pass None when something holds the payload addresses across steps (a captured graph of the forward pass, views
+        taken of `.value`).  Steps taken under stream capture, and payloads that are views of somebody else's storage,
+        keep the in-place step whatever is asked for.  `double_buffer=True` is the older spelling of one_pass='double'."""
+        if double_buffer and one_pass is None:
+            one_pass = 'double'
+        if one_pass not in (None, 'shift', 'double'):
+            raise ValueError("one_pass must be None, 'shift' or 'double'")
         self.tensor_scale = tensor_scale
-        self.double_buffer = double_buffer
-        self._fused_cache = {}
-        self._spare = {}    # id(parameter) -> [weight, exp_avg, exp_avg_sq] payload buffers not in use right now
+        self.one_pass = one_pass
+        self._plans = {}
         super().__init__(
             params, lr=lr, bias_correction=bias_correction, betas=betas, eps=eps, weight_decay=weight_decay,
             amsgrad=False, maximize=maximize, exp_avg_dtype=exp_avg_dtype, exp_avg_sq_dtype=exp_avg_sq_dtype
         )
+
+    @property
+    def double_buffer(self):
+        return self.one_pass == 'double'
+
+    def extra_bytes(self):
+        """Device memory the one-pass forms hold beyond the payloads themselves (the room in the arenas, the second
+        set of buffers)."""
+        total = 0
+        for plan in self._plans.values():
+            if plan.arenas is not None:
+                total += sum(plan.slack * _backend.ADAMW_CHUNK * width for width in plan.widths)
+            if plan.spare is not None:
+                total += sum(t.numel() * t.element_size() for trio in plan.spare for t in trio)
+        return total
 
     # ---- fused multi-tensor path ------------------------------------------------------------
     @staticmethod
@@ -58,85 +112,196 @@ class LBAdamW(LBAdamWBase):
             return False
         return all(t.data_ptr() % 16 == 0 for t in tensors)
 
-    def _fused_tables(self, key, params, grads, exp_avgs, exp_avg_sqs):
-        """Device descriptor table + block map for a list of tensors, cached while no pointer changes."""
-        rows = []
-        for p, g, m, v in zip(params, grads, exp_avgs, exp_avg_sqs):
-            rows.append((
-                p.value.data_ptr(), g.value.data_ptr(), m.value.data_ptr(), v.value.data_ptr(),
-                p.meta.scale.data_ptr(), p.meta.scale_inv.data_ptr(), p.meta.amax.data_ptr(),
-                g.meta.scale_inv.data_ptr(),
-                m.meta.scale.data_ptr(), m.meta.scale_inv.data_ptr(), m.meta.amax.data_ptr(),
-                v.meta.scale.data_ptr(), v.meta.scale_inv.data_ptr(), v.meta.amax.data_ptr(),
-                p.value.numel(), 0, 0, 0, 0,
-            ))
-        sig = tuple(rows)
-        cached = self._fused_cache.get(key)
-        if cached is not None and cached[0] == sig:
-            return cached[1], cached[2], cached[3], cached[4]
-        device = params[0].value.device
-        desc = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), _backend.ADAMW_DESC_WORDS)).to(device)
-        chunks = [(p.value.numel() + _backend.ADAMW_CHUNK - 1) // _backend.ADAMW_CHUNK for p in params]
-        tensor_idx = np.repeat(np.arange(len(params), dtype=np.int32), chunks)
-        chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in chunks]) if chunks else np.zeros(0, np.int32)
-        block_map = torch.from_numpy(np.stack([tensor_idx, chunk_idx], axis=1).copy()).to(device)
-        self._fused_cache[key] = (sig, desc, block_map, int(block_map.shape[0]), chunks)
-        return desc, block_map, int(block_map.shape[0]), chunks
+    # columns of a descriptor row that may change between steps: weight, grad, exp_avg, exp_avg_sq payloads and the
+    # gradient's scale_inv
+    _MOVING = (0, 1, 2, 3, 7)
+
+    @staticmethod
+    def _moving_sig(ps, gs, ms, vs):
+        return ([p.value.data_ptr() for p in ps], [g.value.data_ptr() for g in gs], [m.value.data_ptr() for m in ms],
+                [v.value.data_ptr() for v in vs], [g.meta.scale_inv.data_ptr() for g in gs])
+
+    @staticmethod
+    def _static_rows(ps, ms, vs):
+        return [(p.meta.scale.data_ptr(), p.meta.scale_inv.data_ptr(), p.meta.amax.data_ptr(), 0,
+                 m.meta.scale.data_ptr(), m.meta.scale_inv.data_ptr(), m.meta.amax.data_ptr(),
+                 v.meta.scale.data_ptr(), v.meta.scale_inv.data_ptr(), v.meta.amax.data_ptr(), p.value.numel(), 0, 0, 0, 0)
+                for p, m, v in zip(ps, ms, vs)]
+
+    def _plan_for(self, key, ps, ms, vs):
+        """The cached plan of this group if it still describes these parameters, else a fresh one (tables not built)."""
+        ids = tuple(id(p) for p in ps)
+        plan = self._plans.get(key)
+        if plan is not None and plan.params == ids:
+            return plan
+        plan = _FusedPlan()
+        plan.params = ids
+        plan.chunks = [(p.value.numel() + _backend.ADAMW_CHUNK - 1) // _backend.ADAMW_CHUNK for p in ps]
+        device = ps[0].value.device
+        tensor_idx = np.repeat(np.arange(len(ps), dtype=np.int32), plan.chunks)
+        chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in plan.chunks]) if plan.chunks else np.zeros(0, np.int32)
+        plan.block_map = torch.from_numpy(np.stack([tensor_idx, chunk_idx], axis=1).copy()).to(device)
+        plan.n_blocks = int(plan.block_map.shape[0])
+        self._plans[key] = plan
+        return plan
+
+    def _table(self, plan, slot, ps, gs, ms, vs, sig=None):
+        """Device descriptor table `slot` of the plan, brought up to date: built in full the first time (and again when
+        a meta tensor has been replaced), afterwards only the columns whose addresses changed since the last step
+        are sent again."""
+        sig = sig or self._moving_sig(ps, gs, ms, vs)
+        metas = [id(t) for p, m, v in zip(ps, ms, vs) for t in (p.meta.scale, m.meta.scale, v.meta.scale)]
+        if plan.desc is None or plan.static_sig != metas:
+            plan.desc, plan.sig, plan.stage, plan.static_sig = {}, {}, {}, metas
+        desc = plan.desc.get(slot)
+        capturing = torch.cuda.is_current_stream_capturing()
+        if desc is None:
+            if capturing:
+                raise RuntimeError('LBAdamW: the first fused step of a parameter group builds device tables and cannot be '
+                                   'captured; take a step outside the capture first (two with one_pass set).')
+            rows = np.zeros((len(ps), _backend.ADAMW_DESC_WORDS), dtype=np.int64)
+            rows[:, 4:19] = np.asarray(self._static_rows(ps, ms, vs), dtype=np.int64)
+            for col, values in zip(self._MOVING, sig):
+                rows[:, col] = values
+            # a pinned copy of the rows stays with the table: what a captured step sends its new addresses through
+            stage = torch.from_numpy(rows).pin_memory()
+            plan.desc[slot] = torch.empty_like(stage, device=ps[0].value.device)
+            plan.desc[slot].copy_(stage)
+            plan.stage[slot] = stage
+            plan.sig[slot] = sig
+            return plan.desc[slot]
+        old = plan.sig[slot]
+        if old != sig:
+            if capturing:
+                # (gradients made under capture come from the graph's own memory) the whole table again, from pinned
+                # memory: one copy the graph can hold.  The scratch words of the rows are zero between calls anyway.
+                stage = plan.stage[slot]
+                for col, values in zip(self._MOVING, sig):
+                    stage[:, col] = torch.tensor(values, dtype=torch.int64)
+                desc.copy_(stage, non_blocking=True)
+            else:
+                for col, values, before in zip(self._MOVING, sig, old):
+                    if values != before:
+                        desc[:, col] = torch.tensor(values, dtype=torch.int64).to(desc.device)
+            plan.sig[slot] = sig
+        return desc
 
     def _fused_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, step, *, beta1, beta2, lr, weight_decay, eps,
                     maximize):
         ps, gs = [params[i] for i in idx], [grads[i] for i in idx]
         ms, vs = [exp_avgs[i] for i in idx], [exp_avg_sqs[i] for i in idx]
-        wq, gq = ps[0].qtype, gs[0].qtype
-        if self.double_buffer and self._can_swap(ps, ms, vs):
-            # the payload pointers alternate between two sets from step to step: one cached table per set
-            key = (int(wq), int(gq), id(ps[0]), ps[0].value.data_ptr())
-            desc, block_map, n_blocks, _ = self._fused_tables(key, ps, gs, ms, vs)
-            spares = [self._spare_buffers(p, m, v) for p, m, v in zip(ps, ms, vs)]
-            outputs, redo = self._output_tables(key, spares)
-            _backend.adamw_fused_speculative(
-                desc, outputs, redo, len(ps), block_map, n_blocks, int(wq), int(gq), lr, beta1, beta2, eps, weight_decay, step,
-                self.bias_correction, self.use_adam, maximize, self.tensor_scale
-            )
-            # the payload tensors stay the objects they were and trade their memory with the spares
-            for p, m, v, spare in zip(ps, ms, vs, spares):
-                for i, t in enumerate((p.value, m.value, v.value)):
-                    old = t.data
-                    t.data = spare[i]
-                    spare[i] = old
+        wq, gq = int(ps[0].qtype), int(gs[0].qtype)
+        key = (wq, gq, id(ps[0]))
+        plan = self._plan_for(key, ps, ms, vs)
+        hyper = (lr, beta1, beta2, eps, weight_decay, step, self.bias_correction, self.use_adam, maximize, self.tensor_scale)
+        capturing = torch.cuda.is_current_stream_capturing()
+        if self.one_pass == 'shift' and not capturing and self._shift_step(plan, ps, gs, ms, vs, wq, gq, hyper):
             return
-        key = (int(wq), int(gq), id(ps[0]))
-        desc, block_map, n_blocks, chunks = self._fused_tables(key, ps, gs, ms, vs)
-        _backend.adamw_fused(
-            desc, len(ps), block_map, n_blocks, int(wq), int(gq), lr, beta1, beta2, eps, weight_decay, step,
-            self.bias_correction, self.use_adam, maximize, self.tensor_scale, blocks_per_tensor=chunks
-        )
+        if self.one_pass == 'double' and not capturing and self._can_swap(ps, ms, vs):
+            self._double_step(plan, ps, gs, ms, vs, wq, gq, hyper)
+            return
+        # in place, with the table of wherever the payloads are now (a moving form that has run leaves them at one of its
+        # two places, and the table it keeps for that place holds the right addresses)
+        if self.one_pass == 'shift' and plan.arenas is not None:
+            slot = ('shift', plan.phase)
+        elif self.one_pass == 'double' and plan.spare is not None:
+            slot = ('double', ps[0].value.data_ptr())
+        else:
+            slot = ('in_place', ps[0].value.data_ptr())
+        desc = self._table(plan, slot, ps, gs, ms, vs)
+        _backend.adamw_fused(desc, len(ps), plan.block_map, plan.n_blocks, wq, gq, *hyper, blocks_per_tensor=plan.chunks)
+
+    # ---- one pass between two sets of buffers -----------------------------------------------
+    def _double_step(self, plan, ps, gs, ms, vs, wq, gq, hyper):
+        current = [(p.value, m.value, v.value) for p, m, v in zip(ps, ms, vs)]
+        if plan.spare is None or any(s.shape != c.shape or s.dtype != c.dtype or s.device != c.device
+                                     for trio, cur in zip(plan.spare, current) for s, c in zip(trio, cur)):
+            plan.spare = [[torch.empty_like(c) for c in cur] for cur in current]
+            plan.outputs = {}
+        slot = ('double', ps[0].value.data_ptr())
+        desc = self._table(plan, slot, ps, gs, ms, vs)
+        out_sig = [tuple(t.data_ptr() for t in trio) for trio in plan.spare]
+        cached = plan.outputs.get(slot)
+        if cached is None or cached[0] != out_sig:
+            rows = np.asarray([sig + (0, ) for sig in out_sig], dtype=np.int64).reshape(len(ps), _backend.ADAMW_BUFFER_WORDS)
+            cached = (out_sig, torch.from_numpy(rows).to(desc.device))
+            plan.outputs[slot] = cached
+        if plan.redo is None:
+            plan.redo = torch.zeros(len(ps), dtype=torch.int32, device=desc.device)
+        _backend.adamw_fused_speculative(desc, cached[1], plan.redo, len(ps), plan.block_map, plan.n_blocks, wq, gq, *hyper)
+        # the payload tensors stay the objects they were and trade their memory with the spares
+        for cur, trio in zip(current, plan.spare):
+            for i, t in enumerate(cur):
+                old = t.data
+                t.data = trio[i]
+                trio[i] = old
 
     @staticmethod
     def _can_swap(ps, ms, vs):
-        """Swapping payload tensors is safe when nothing else aliases them and no graph is recording their addresses."""
-        if torch.cuda.is_current_stream_capturing():
-            return False
+        """Swapping payload tensors is safe when nothing else aliases them."""
         return all(t.value._base is None for group in (ps, ms, vs) for t in group)
 
-    def _spare_buffers(self, p, m, v):
-        spare = self._spare.get(id(p))
-        current = (p.value, m.value, v.value)
-        if spare is None or any(s.shape != c.shape or s.dtype != c.dtype or s.device != c.device for s, c in zip(spare, current)):
-            spare = [torch.empty_like(c) for c in current]
-            self._spare[id(p)] = spare
-        return spare
+    # ---- one pass inside shifting arenas -----------------------------------------------------
+    # room beyond the largest tensor: what the chip keeps in flight (about a thousand chunks) twice over, plus the lead
+    # with which a tensor's outcome is decided before its first chunk is written over
+    _SHIFT_MARGIN = 2560
 
-    def _output_tables(self, key, spares):
-        rows = tuple((s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), 0) for s in spares)
-        cached = self._fused_cache.get(('out', ) + key)
-        if cached is not None and cached[0] == rows:
-            return cached[1], cached[2]
-        device = spares[0][0].device
-        outputs = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), _backend.ADAMW_BUFFER_WORDS)).to(device)
-        redo = torch.zeros(len(rows), dtype=torch.int32, device=device)
-        self._fused_cache[('out', ) + key] = (rows, outputs, redo)
-        return outputs, redo
+    def _adopt(self, plan, ps, ms, vs):
+        """Move the payloads into arenas of the optimizer's own (once; again if somebody replaced a payload)."""
+        ch = _backend.ADAMW_CHUNK
+        total = sum(plan.chunks)
+        biggest = max(plan.chunks)
+        plan.slack = biggest + min(self._SHIFT_MARGIN, max(total // 4, 1))
+        device = ps[0].value.device
+        plan.widths = (ps[0].value.element_size(), 1, 2)
+        try:
+            arenas = [torch.empty((total + plan.slack) * ch * width, dtype=torch.uint8, device=device) for width in plan.widths]
+        except torch.cuda.OutOfMemoryError:
+            return False
+        pos = np.concatenate([[0], np.cumsum(plan.chunks)]).tolist()
+        plan.views = [[], []]
+        for i, (p, m, v) in enumerate(zip(ps, ms, vs)):
+            for phase, off in ((0, plan.slack), (1, 0)):
+                trio = []
+                for arena, width, t in zip(arenas, plan.widths, (p.value, m.value, v.value)):
+                    first = (pos[i] + off) * ch * width
+                    trio.append(arena[first:first + t.numel() * width].view(t.dtype).view(t.shape))
+                plan.views[phase].append(trio)
+            # one tensor at a time, so that at most one payload exists twice while the arenas fill
+            for t, view in zip((p.value, m.value, v.value), plan.views[0][i]):
+                view.copy_(t)
+                t.data = view
+        plan.arenas = arenas
+        plan.phase = 0
+        plan.redo = torch.zeros(len(ps), dtype=torch.int32, device=device)
+        plan.sync = torch.zeros(_backend.adamw_shift_sync_bytes(len(ps), total), dtype=torch.uint8, device=device)
+        plan.desc = None
+        return True
+
+    def _shift_step(self, plan, ps, gs, ms, vs, wq, gq, hyper):
+        """The step inside the arenas; False if this group cannot be taken that way (the caller then goes in place)."""
+        sig = self._moving_sig(ps, gs, ms, vs)
+        if plan.arenas is not None:
+            home = plan.views[plan.phase]
+            if any(w != trio[0].data_ptr() or m != trio[1].data_ptr() or v != trio[2].data_ptr()
+                   for w, m, v, trio in zip(sig[0], sig[2], sig[3], home)):
+                plan.arenas = None    # somebody put other tensors in place of the payloads (load_state_dict, .data): adopt again
+        if plan.arenas is None:
+            if not self._can_swap(ps, ms, vs) or len({p.value.element_size() for p in ps}) != 1:
+                return False
+            if not self._adopt(plan, ps, ms, vs):
+                return False
+            sig = self._moving_sig(ps, gs, ms, vs)
+        desc = self._table(plan, ('shift', plan.phase), ps, gs, ms, vs, sig)
+        shift = (-plan.slack if plan.phase == 0 else plan.slack) * _backend.ADAMW_CHUNK
+        _backend.adamw_fused_shift(desc, plan.redo, plan.sync, len(ps), plan.block_map, plan.n_blocks, shift, wq, gq, *hyper)
+        plan.phase = 1 - plan.phase
+        # the payload tensors stay the objects they were; their memory is now the other place in the arena
+        for p, m, v, trio in zip(ps, ms, vs, plan.views[plan.phase]):
+            p.value.data = trio[0]
+            m.value.data = trio[1]
+            v.value.data = trio[2]
+        return True
 
     # ---- per-tensor path (reference recipe) -----------------------------------------------
     def _staged_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, state_steps, *, beta1, beta2, lr, weight_decay,

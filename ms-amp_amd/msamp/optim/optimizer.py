@@ -23,11 +23,13 @@ class LBOptimizer(Optimizer):
 
     def step(self, closure=None):
         """One optimization step followed by the scaling-factor update of all FP8 layers."""
+        # A bounded wait that ran out inside a cast, GEMM or optimizer kernel of an earlier step surfaces here, before this
+        # step changes anything, and without a device-to-host synchronisation (the copy of the error word requested by
+        # the previous step is looked at).  What such a kernel wrote is invalid, and so is what was computed from it
+        # since: the caller goes back to its last good state.
+        _backend.check_async_error(block=False)
         rtn = self.lb_step(closure)
         self._update_scaling_factors()
-        # a bounded wait that ran out inside a cast or GEMM kernel of an earlier step surfaces here, without a
-        # device-to-host synchronisation (the copy of the error word requested by the previous step is looked at)
-        _backend.check_async_error(block=False)
         return rtn
 
     def all_reduce_grads(self, model):

@@ -314,22 +314,24 @@ def test_fused_adamw_only_for_weights_under_in_time_scaling(monkeypatch):
     assert torch.allclose(w_fused, w_staged, rtol=0, atol=float(w_fused.abs().max()) * 2e-3)
 
 
-def test_double_buffered_adamw_matches_the_in_place_step():
-    """LBAdamW(double_buffer=True) takes the fused step in one pass into spare buffers and swaps memory afterwards: same
-    weights, moments and metas as double_buffer=False after every step, with the payload tensors staying the objects
-    they were while their addresses alternate."""
+def test_one_pass_adamw_matches_the_in_place_step():
+    """LBAdamW(one_pass='double') takes the fused step in one pass into spare buffers and swaps memory afterwards;
+    one_pass='shift' takes it inside arenas of its own, writing a little further along each time: same weights, moments
+    and metas as the default in-place step after every step, with the payload tensors staying the objects they were
+    while their addresses alternate between two places."""
     torch.manual_seed(13)
-    lin = torch.nn.Sequential(torch.nn.Linear(256, 512, bias=False), torch.nn.Linear(512, 128, bias=False)).cuda()
+    lin = torch.nn.Sequential(torch.nn.Linear(256, 512, bias=False), torch.nn.Linear(512, 128, bias=False),
+                              torch.nn.Linear(128, 70, bias=False)).cuda()
     x = torch.randn(64, 256, device='cuda')
     runs = {}
-    for double in (False, True):
+    for mode in (None, 'double', 'shift'):
         model_state.clear()
         model = LinearReplacer.replace(copy.deepcopy(lin), Dtypes.kfloat8_e4m3)
-        opt = LBAdamW(model.parameters(), lr=1e-2, double_buffer=double)
+        opt = LBAdamW(model.parameters(), lr=1e-2, one_pass=mode)
         values = [p.value for p in model.parameters()]
         addresses = []
         history = []
-        for step in range(5):
+        for step in range(6):
             model(x * (1 + step)).square().mean().backward()
             opt.all_reduce_grads(model)
             opt.step()
@@ -339,14 +341,148 @@ def test_double_buffered_adamw_matches_the_in_place_step():
                              opt.state[p]['exp_avg'].meta.scale.clone(), opt.state[p]['exp_avg_sq'].value.clone(),
                              opt.state[p]['exp_avg_sq'].meta.scale.clone()) for p in model.parameters()])
         assert all(p.value is v for p, v in zip(model.parameters(), values))
-        if double:
-            assert addresses[0] != addresses[1] and addresses[0] == addresses[2] and addresses[1] == addresses[3]
-        else:
+        if mode is None:
             assert all(a == addresses[0] for a in addresses)
-        runs[double] = history
-    for a, b in zip(runs[False], runs[True]):
+            assert opt.extra_bytes() == 0
+        else:
+            assert addresses[0] != addresses[1] and addresses[0] == addresses[2] and addresses[1] == addresses[3]
+            assert opt.extra_bytes() > 0
+        runs[mode] = history
+    for mode in ('double', 'shift'):
+        for a, b in zip(runs[None], runs[mode]):
+            for pa, pb in zip(a, b):
+                assert all(torch.equal(ta, tb) for ta, tb in zip(pa, pb)), mode
+    from msamp import _backend
+    _backend.check_async_error(block=True)
+
+
+def test_shifting_adamw_survives_a_replaced_state_and_a_state_dict_round_trip():
+    """one_pass='shift' keeps the payloads in its own arenas; when something puts other tensors in their place
+    (load_state_dict does) the optimizer adopts them again, and training goes on as it does in place."""
+    torch.manual_seed(14)
+    lin = torch.nn.Sequential(torch.nn.Linear(64, 96, bias=False), torch.nn.Linear(96, 32, bias=False)).cuda()
+    x = torch.randn(32, 64, device='cuda')
+
+    def run(mode):
+        model_state.clear()
+        model = LinearReplacer.replace(copy.deepcopy(lin), Dtypes.kfloat8_e4m3)
+        opt = LBAdamW(model.parameters(), lr=1e-2, one_pass=mode)
+        out = []
+        for step in range(5):
+            model(x * (1 + step)).square().mean().backward()
+            opt.all_reduce_grads(model)
+            opt.step()
+            opt.zero_grad()
+            if step == 2:
+                saved = copy.deepcopy(opt.state_dict())
+                opt.load_state_dict(saved)
+            out.append([(p.value.clone(), opt.state[p]['exp_avg'].value.clone(), opt.state[p]['exp_avg_sq'].value.clone())
+                        for p in model.parameters()])
+        return out
+
+    for a, b in zip(run(None), run('shift')):
         for pa, pb in zip(a, b):
             assert all(torch.equal(ta, tb) for ta, tb in zip(pa, pb))
+
+
+def test_captured_forward_and_backward_see_the_weights_of_eager_steps():
+    """The default optimizer step leaves every payload where it was, so a graph captured of forward and backward keeps
+    reading the current weights while the optimizer steps eagerly between replays."""
+    torch.manual_seed(15)
+    lin = torch.nn.Linear(128, 256, bias=False).cuda().bfloat16()
+
+    def build():
+        model_state.clear()
+        model = LinearReplacer.replace(copy.deepcopy(lin), Dtypes.kfloat8_e4m3)
+        return model, LBAdamW(model.parameters(), lr=1e-2)
+
+    xs = [torch.randn(256, 128, device='cuda').bfloat16() * (1 + i % 3) for i in range(6)]
+    dy = (torch.randn(256, 256, device='cuda') * 1e-2).bfloat16()
+    # eager reference
+    model, opt = build()
+    want = []
+    for x in xs:
+        y = model(x)
+        y.backward(dy)
+        opt.all_reduce_grads(model)
+        opt.step()
+        opt.zero_grad()
+        want.append((y.detach().clone(), model.weight.value.clone()))
+    # forward and backward from a graph, the step eager
+    model, opt = build()
+    x = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        model(x).backward(dy)
+        model.weight.grad = None
+    torch.cuda.current_stream().wait_stream(side)
+    model_state.clear()
+    model, opt = build()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = model(x)
+        y.backward(dy)
+    grad = model.weight.grad
+    for i, xi in enumerate(xs):
+        x.copy_(xi)
+        graph.replay()
+        model.weight.grad = grad
+        model_state.ready_to_scale_tensor = True
+        opt.all_reduce_grads(model)
+        opt.step()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[i][0]), i
+        assert torch.equal(model.weight.value, want[i][1]), i
+
+
+def test_optimizer_step_under_capture_after_an_eager_step():
+    """A fused step can be captured once an eager step has built the device tables: the gradients made under capture live
+    elsewhere, their addresses reach the table through a pinned copy that the graph holds.  (Bias correction is
+    computed on the host from the step count, so a captured step repeats the one it was captured with: off here.)"""
+    torch.manual_seed(16)
+    lin = torch.nn.Linear(128, 256, bias=False).cuda().bfloat16()
+    xs = [torch.randn(256, 128, device='cuda').bfloat16() * (1 + i % 3) for i in range(5)]
+    dy = (torch.randn(256, 256, device='cuda') * 1e-2).bfloat16()
+
+    def build():
+        model_state.clear()
+        model = LinearReplacer.replace(copy.deepcopy(lin), Dtypes.kfloat8_e4m3)
+        return model, LBAdamW(model.parameters(), lr=1e-2, bias_correction=False)
+
+    model, opt = build()
+    want = []
+    for x in xs:
+        model(x).backward(dy)
+        opt.all_reduce_grads(model)
+        opt.step()
+        opt.zero_grad()
+        want.append((model.weight.value.clone(), opt.state[model.weight]['exp_avg'].value.clone()))
+    model, opt = build()
+    x = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        model(x).backward(dy)
+        opt.all_reduce_grads(model)
+        opt.step()
+        model.weight.grad = None
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert torch.equal(model.weight.value, want[0][0])
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        model(x).backward(dy)
+        model_state.ready_to_scale_tensor = True
+        opt.step()
+        model.weight.grad = None
+    for i in range(1, len(xs)):
+        x.copy_(xs[i])
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(model.weight.value, want[i][0]), i
+        assert torch.equal(opt.state[model.weight]['exp_avg'].value, want[i][1]), i
+        assert torch.isfinite(xs[i].float().sum()).item()    # eager work between replays
 
 
 def test_historical_window_quantization():
