@@ -1157,18 +1157,23 @@ __global__ __launch_bounds__(kAdamThreads) void fused_shift_kernel(msamp_adamw_t
 }
 
 // after the walk: the tensors nobody has decided (their first chunk lies where nothing is written over it); one
-// workgroup per tensor, found through its first chunk in the block map
+// workgroup per tensor, which finds the tensor's first chunk in the block map (tensors in order there) by bisection
 __global__ __launch_bounds__(kAdamThreads) void fused_shift_scales_kernel(msamp_adamw_tensor* tensors, const int32_t* block_map,
                                                                            ShiftArgs a) {
     __shared__ uint32_t red[kAdamThreads / kWave];
-    const int j = blockIdx.x;
-    if (block_map[2 * j + 1] != 0) return;
-    const int t = block_map[2 * j];
+    const int t = blockIdx.x;
     if (static_cast<uint32_t>(a.posts[static_cast<size_t>(t) * kShiftPostWords] >> 32) == a.token) return;
+    int lo = 0, hi = a.n_chunks;    // first chunk whose tensor is >= t
+    while (lo < hi) {
+        const int mid = lo + (hi - lo) / 2;
+        if (block_map[2 * mid] < t) lo = mid + 1;
+        else hi = mid;
+    }
+    if (lo >= a.n_chunks || block_map[2 * lo] != t) return;    // a tensor without elements has no chunk
     msamp_adamw_tensor& d = tensors[t];
     const int chunks = static_cast<int>((d.numel + MSAMP_ADAMW_CHUNK - 1) / MSAMP_ADAMW_CHUNK);
     uint32_t gp, gm, gv;
-    if (gather_marks(a, j, chunks, red, gp, gm, gv)) decide_tensor(d, t, a, j, chunks, gp, gm, gv, false, red);
+    if (gather_marks(a, lo, chunks, red, gp, gm, gv)) decide_tensor(d, t, a, lo, chunks, gp, gm, gv, false, red);
     else if (threadIdx.x == 0) report_wait_expired(a.error_word, kErrShiftGaveUp);
 }
 
@@ -1425,7 +1430,7 @@ int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, void
     a.tensor_scale = tensor_scale;
     FUSED_LAUNCH(fused_shift_kernel, n_blocks, tensors, block_map, k, a);
     MSAMP_CHECK_LAUNCH("fused_shift_kernel");
-    hipLaunchKernelGGL(fused_shift_scales_kernel, dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, a);
+    hipLaunchKernelGGL(fused_shift_scales_kernel, dim3(n_tensors), dim3(kAdamThreads), 0, st, tensors, block_map, a);
     MSAMP_CHECK_LAUNCH("fused_shift_scales_kernel");
     const int tail = n_blocks < a.slack ? n_blocks : a.slack;
     FUSED_LAUNCH(fused_shift_tail_kernel, tail, tensors, block_map, k, a);

@@ -186,7 +186,12 @@ def check_async_error(block=True):
             continue
         entry = _pending_error_reads.get(key)
         if entry is None:
-            entry = {'host': torch.zeros(1, dtype=torch.int32, pin_memory=True), 'event': torch.cuda.Event(), 'in_flight': False}
+            # the word is sticky, so it may be read at any time: on a stream of its own, where the copy does not stand
+            # between two kernels of the stream that does the work
+            with torch.cuda.device(ws.device):
+                side = torch.cuda.Stream()
+            entry = {'host': torch.zeros(1, dtype=torch.int32, pin_memory=True), 'event': torch.cuda.Event(), 'in_flight': False,
+                     'stream': side}
             _pending_error_reads[key] = entry
         if entry['in_flight'] and entry['event'].query():
             entry['in_flight'] = False
@@ -195,8 +200,9 @@ def check_async_error(block=True):
                 failed = f'a kernel whose workgroups wait for each other gave up waiting (code {code})'
                 ws[WS_ERROR_BYTE:WS_ERROR_BYTE + 4].zero_()
         if not entry['in_flight']:
-            entry['host'].copy_(ws[WS_ERROR_BYTE:WS_ERROR_BYTE + 4].view(torch.int32), non_blocking=True)
-            entry['event'].record()
+            with torch.cuda.stream(entry['stream']):
+                entry['host'].copy_(ws[WS_ERROR_BYTE:WS_ERROR_BYTE + 4].view(torch.int32), non_blocking=True)
+                entry['event'].record()
             entry['in_flight'] = True
     if failed is not None:
         _force_two_pass = True

@@ -72,6 +72,7 @@ class LBAdamW(LBAdamWBase):
         self.tensor_scale = tensor_scale
         self.one_pass = one_pass
         self._plans = {}
+        self._groups = None
         super().__init__(
             params, lr=lr, bias_correction=bias_correction, betas=betas, eps=eps, weight_decay=weight_decay,
             amsgrad=False, maximize=maximize, exp_avg_dtype=exp_avg_dtype, exp_avg_sq_dtype=exp_avg_sq_dtype
@@ -193,6 +194,12 @@ class LBAdamW(LBAdamWBase):
         wq, gq = int(ps[0].qtype), int(gs[0].qtype)
         key = (wq, gq, id(ps[0]))
         plan = self._plan_for(key, ps, ms, vs)
+        if any(g.value.data_ptr() % 16 or not g.value.is_contiguous() for g in gs):
+            # a gradient the fused kernels do not take (the grouping is kept from an earlier step): this step tensor by tensor
+            self._groups = None
+            self._staged_step(idx, params, grads, exp_avgs, exp_avg_sqs, [step] * len(params), beta1=beta1, beta2=beta2, lr=lr,
+                              weight_decay=weight_decay, eps=eps, maximize=maximize)
+            return
         hyper = (lr, beta1, beta2, eps, weight_decay, step, self.bias_correction, self.use_adam, maximize, self.tensor_scale)
         capturing = torch.cuda.is_current_stream_capturing()
         if self.one_pass == 'shift' and not capturing and self._shift_step(plan, ps, gs, ms, vs, wq, gq, hyper):
@@ -358,16 +365,26 @@ class LBAdamW(LBAdamWBase):
         if amsgrad:
             raise ValueError('Only amsgrad=False is supported for now.')
         if len(exp_avgs) > 0 and exp_avgs[0].dtype != torch.float32:
-            fused = {}
-            staged = []
-            for i in range(len(params)):
-                if self._fusable(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i]):
-                    fused.setdefault((int(params[i].qtype), int(grads[i].qtype), state_steps[i]), []).append(i)
-                else:
-                    staged.append(i)
+            # Which parameters take the fused call is looked into once per set of parameters, states, gradient formats and
+            # step counts (the look costs more host time than everything else in a step); what may change from step to
+            # step without showing here -- where a gradient's payload lies -- is checked in _fused_step.
+            key = (tuple(map(id, params)), tuple(map(id, exp_avgs)), tuple(map(id, exp_avg_sqs)),
+                   tuple(g.qtype if isinstance(g, ScalingTensor) else None for g in grads),
+                   tuple(n - state_steps[0] for n in state_steps), ScalingMeta.in_time_scaling)
+            if self._groups is not None and self._groups[0] == key:
+                fused, staged = self._groups[1], self._groups[2]
+            else:
+                fused = {}
+                staged = []
+                for i in range(len(params)):
+                    if self._fusable(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i]):
+                        fused.setdefault((int(params[i].qtype), int(grads[i].qtype), state_steps[i]), []).append(i)
+                    else:
+                        staged.append(i)
+                self._groups = (key, fused, staged)
             hyper = dict(beta1=beta1, beta2=beta2, lr=lr, weight_decay=weight_decay, eps=eps, maximize=maximize)
-            for (_, _, step), idx in fused.items():
-                self._fused_step(idx, params, grads, exp_avgs, exp_avg_sqs, step, **hyper)
+            for idx in fused.values():    # (one call per weight format, gradient format and step count)
+                self._fused_step(idx, params, grads, exp_avgs, exp_avg_sqs, state_steps[idx[0]], **hyper)
             self._staged_step(staged, params, grads, exp_avgs, exp_avg_sqs, state_steps, **hyper)
             return
         # float32 moments: whole-tensor float32 update, then requantize the parameter if it is low-bit
