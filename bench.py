@@ -586,6 +586,108 @@ def cpu_baseline():
     }
 
 
+def bench_power(seconds=2.0):
+    """Socket power and shader clock, sampled from the amdgpu driver's sysfs files at 20 Hz by a host thread, while
+    (a) nothing runs, (b) the FP8 GEMM of the Llama-70B gate projection [16384 x 28672 x 8192] and (c) a register-only
+    FP8 MFMA loop (msamp_mfma_probe) each run back to back for `seconds`.  Reported so that a GEMM rate can be read
+    against what the matrix pipes sustain under the device's power limit, not only against the nominal peak."""
+    import glob
+    import threading
+    import torch
+    from msamp import _backend as be
+
+    def first(pattern):
+        hits = sorted(glob.glob(pattern))
+        return hits[0] if hits else None
+
+    hwmon = '/sys/class/drm/card*/device/hwmon/hwmon*/'
+    power = first(hwmon + 'power1_average') or first(hwmon + 'power1_input')
+    cap = first(hwmon + 'power1_cap')
+    dpm = first('/sys/class/drm/card*/device/pp_dpm_sclk')
+
+    def read(path):
+        try:
+            with open(path) as f:
+                return f.read().strip()
+        except (OSError, TypeError):
+            return None
+
+    def clock_now():
+        for line in (read(dpm) or '').splitlines():
+            if line.endswith('*'):
+                return float(line.split()[1].lower().replace('mhz', ''))
+        return None
+
+    def sample_while(fn, duration):
+        fn()
+        torch.cuda.synchronize()
+        watts, mhz, stop = [], [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                p, c = read(power), clock_now()
+                if p is not None and p.isdigit():
+                    watts.append(int(p) / 1e6)
+                if c is not None:
+                    mhz.append(c)
+                time.sleep(0.05)
+
+        th = threading.Thread(target=sampler)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        th.start()
+        t0, calls = time.perf_counter(), 0
+        e0.record()
+        while time.perf_counter() - t0 < duration:
+            for _ in range(20):
+                fn()
+            calls += 20
+            torch.cuda.synchronize()
+        e1.record()
+        e1.synchronize()
+        stop.set()
+        th.join()
+
+        def mmm(v):
+            # the first quarter second holds the ramp from idle
+            v = v[5:] if len(v) > 10 else v
+            return {'min': round(min(v)), 'mean': round(sum(v) / len(v)), 'max': round(max(v))} if v else None
+
+        return e0.elapsed_time(e1) / calls, {'samples': len(watts), 'power_W': mmm(watts), 'sclk_MHz': mmm(mhz)}
+
+    out = {'sources': {'power': power, 'clock': dpm}, 'power_cap_W': None}
+    if read(cap) and read(cap).isdigit():
+        out['power_cap_W'] = int(read(cap)) / 1e6
+    _, out['idle'] = sample_while(lambda: None, 1.0)
+
+    tokens, d_out, d_in = 16384, 28672, 8192
+    g = torch.Generator(device='cuda').manual_seed(1)
+
+    def quantized(shape, std):
+        x = (torch.randn(shape, device='cuda', generator=g) * std).bfloat16()
+        s, si, am = torch.ones((), device='cuda'), torch.ones((), device='cuda'), torch.zeros(1, device='cuda')
+        return be.cast_to_fp8_intime(x, s, am, si, be.DT_E4M3), si
+
+    x, xs = quantized((tokens, d_in), 1.0)
+    w, ws = quantized((d_out, d_in), 0.02)
+    y = torch.empty(tokens, d_out, dtype=torch.bfloat16, device='cuda')
+    ms, row = sample_while(lambda: be.fp8_gemm(w, be.DT_E4M3, ws, x, be.DT_E4M3, xs, y), seconds)
+    row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(2.0 * tokens * d_out * d_in / ms / 1e9, 1)})
+    out['fp8_gemm_16384x28672x8192'] = row
+    del x, w, y
+
+    seed = quantized((4096, ), 1.0)[0]
+    sink = torch.zeros(1, device='cuda')
+    flop = [0.0]
+
+    def probe():
+        flop[0] = be.mfma_probe(seed, sink, 20000, 1024)
+
+    ms, row = sample_while(probe, seconds)
+    row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(flop[0] / ms / 1e9, 1)})
+    out['register_only_fp8_mfma_loop'] = row
+    return out
+
+
 def pmc_calibration_copy():
     """One plain copy of known size -- scale_cast fp32 -> fp32 at scale 1 over 64 Mi elements: 256 MiB read,
     256 MiB written -- so that a `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` run of this program holds a
@@ -624,7 +726,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--skip-cpu', action='store_true', help='leave out the CPU-oracle baseline')
     ap.add_argument('--skip-extra', action='store_true', help='leave out the sweep, cast and Adam kernel sections')
-    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'cast', 'adam', 'grad_side'), default=None,
+    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'cast', 'adam', 'grad_side', 'power'), default=None,
                     help='run one kernel section alone (after the calibration copy), for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -648,6 +750,8 @@ def main():
             out = _round_kernels(bench_cast())
         elif args.only == 'grad_side':
             out = _round_kernels(bench_grad_side())
+        elif args.only == 'power':
+            out = bench_power()
         else:
             out = bench_adam()
         print(json.dumps({'only': args.only, 'result': out}))
@@ -751,6 +855,8 @@ def main():
                             "one_pass='shift' (arenas of the optimizer's own, one pass)": adam_row(adam['shift']),
                             "one_pass='double' (second set of payload buffers, one pass)": adam_row(adam['double'])},
         })
+        torch.cuda.empty_cache()
+        result['power_and_clock'] = bench_power()
         result['kernels'] = {
             'cast': _round_kernels(cast),
             'fused_adamw': fused,

@@ -290,6 +290,13 @@ int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, 
                         float* scale, float* amax, float* scale_inv, int m, int n, int k, int margin, int flags,
                         void* workspace, msamp_stream_t stream);
 
+/* Calibration aid, no counterpart in the reference: `workgroups` workgroups of four wavefronts each issue
+ * iters x 16 FP8 16x16x128 MFMAs on registers loaded once from seed (4096 bytes of FP8 codes, device memory); nothing
+ * else moves and nothing is written (sink: one float of device memory, never stored to in practice).  *flop (host,
+ * may be null) receives the floating-point operations of the launch.  Timed, it gives the rate the matrix pipes
+ * sustain on this device under its power limit, the practical ceiling beside the nominal peak. */
+int msamp_mfma_probe(const void* seed, float* sink, int iters, int workgroups, double* flop, msamp_stream_t stream);
+
 /* msamp_adamw.adamw_fp8_stage1_compute (adamw.cu:99-127): fp32 param/grad, quantized moments;
  * updates param in place and atomically maxes |m'|, |v'| into the two amax cells.
  * exp_avg_dtype: E4M3/E5M2/F16/F32, exp_avg_sq_dtype: F16/F32/E4M3/E5M2. */

@@ -52,6 +52,7 @@ _SIGNATURES = {
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_cast': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp], _i),
+    'msamp_mfma_probe': ([_vp, _vp, _i, _i, _vp, _vp], _i),
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
     'msamp_fp8_norms': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
     'msamp_bucket_amax': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
@@ -557,6 +558,17 @@ def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, sc
     return out
 
 
+def mfma_probe(seed, sink, iters, workgroups):
+    """Launch the register-only FP8 MFMA loop (calibration aid); returns the floating-point operations of the launch.
+    seed: at least 4096 bytes of FP8 codes on the device, sink: one float32 on the device."""
+    assert seed.is_cuda and seed.is_contiguous() and seed.numel() * seed.element_size() >= 4096
+    assert sink.is_cuda and sink.dtype == torch.float32
+    flop = ctypes.c_double(0.0)
+    _check(load().msamp_mfma_probe(_ptr(seed), _ptr(sink), int(iters), int(workgroups), ctypes.byref(flop), _stream()),
+           'msamp_mfma_probe')
+    return flop.value
+
+
 # ---- gradient buckets -----------------------------------------------------------------------------
 BUCKET_CHUNK = 16384
 BUCKET_ITEM_WORDS = 7    # int64 words per msamp_bucket_item (56 bytes)
@@ -624,25 +636,37 @@ def bucket_cast(items, block_map, in_dt, fp8_dt, pre_scale, scale_inv_div=1.0, m
 NORM_ITEM_WORDS = 5    # int64 words per msamp_norm_item (40 bytes)
 
 
+_NORM_TABLES = {}
+
+
 def fp8_norms(values, scale_invs, fp8_dt, norm_type):
-    """Per-tensor p-norms (p = 1, 2 or inf) of FP8 payloads times their scale_inv, as one float32 vector."""
+    """Per-tensor p-norms (p = 1, 2 or inf) of FP8 payloads times their scale_inv, as one float32 vector.  The
+    descriptor table is kept per set of payload and scale_inv addresses (a training loop asks for the same gradients'
+    norms every step), the result is a fresh tensor every time."""
     import numpy as np
     kind = {1.0: 1, 2.0: 2, float('inf'): 0}[float(norm_type)]
     lib = load()
-    device = values[0].device
-    out = torch.empty(len(values), dtype=torch.float32, device=device)
-    rows = [(v.data_ptr(), si.data_ptr(), out.data_ptr() + 4 * i, v.numel(), 0) for i, (v, si) in enumerate(zip(values, scale_invs))]
-    for v in values:
-        _gpu(v, 'fp8 tensor')
-        if not v.is_contiguous():
-            raise ValueError('fp8 tensors must be contiguous')
-    items = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), NORM_ITEM_WORDS)).to(device)
-    block_map = chunk_map([v.numel() for v in values], device)
+    sig = (tuple(v.data_ptr() for v in values), tuple(si.data_ptr() for si in scale_invs), tuple(v.numel() for v in values))
+    cached = _NORM_TABLES.get(sig)
+    if cached is None:
+        for v in values:
+            _gpu(v, 'fp8 tensor')
+            if not v.is_contiguous():
+                raise ValueError('fp8 tensors must be contiguous')
+        device = values[0].device
+        result = torch.empty(len(values), dtype=torch.float32, device=device)
+        rows = [(v.data_ptr(), si.data_ptr(), result.data_ptr() + 4 * i, v.numel(), 0) for i, (v, si) in enumerate(zip(values, scale_invs))]
+        items = torch.from_numpy(np.asarray(rows, dtype=np.int64).reshape(len(rows), NORM_ITEM_WORDS)).to(device)
+        cached = (items, chunk_map(sig[2], device), result)
+        if len(_NORM_TABLES) >= 8:
+            _NORM_TABLES.pop(next(iter(_NORM_TABLES)))
+        _NORM_TABLES[sig] = cached
+    items, block_map, result = cached
     _check(
         lib.msamp_fp8_norms(_ptr(items), len(values), _ptr(block_map), block_map.shape[0], fp8_dt, kind, _stream()),
         'msamp_fp8_norms'
     )
-    return out
+    return result.clone()
 
 
 # ---- AdamW --------------------------------------------------------------------------------------

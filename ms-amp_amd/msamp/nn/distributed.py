@@ -35,6 +35,7 @@ class GradientBucket:
             self._views.append(self.flat.narrow(0, offset, n))
             offset += n
         self._tables = None
+        self._wrapped = None
 
     def _get_tables(self, grads):
         sig = tuple(g.data_ptr() for g in grads)
@@ -67,4 +68,8 @@ class GradientBucket:
             reduce_amax([m.amax[0:1] for m in self.metas])
         # the division of each finished tensor by the world size (a division of its scale_inv) rides along
         _backend.bucket_cast(items, block_map, in_dt, int(self.qtype), 1.0 / math.sqrt(world_size), float(world_size))
-        return [ScalingTensor(view.view(g.shape), meta) for g, view, meta in zip(grads, self._views, self.metas)]
+        # the wrappers of the flat buffer's parts are the same from call to call while the shapes are
+        shapes = tuple(g.shape for g in grads)
+        if self._wrapped is None or self._wrapped[0] != shapes:
+            self._wrapped = (shapes, [ScalingTensor(view.view(g.shape), meta) for g, view, meta in zip(grads, self._views, self.metas)])
+        return list(self._wrapped[1])

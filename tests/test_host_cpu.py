@@ -304,6 +304,6 @@ def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(gemm_a
             if re.search(r'scratch_(load|store)', line):
                 c[2] += 1
     # bf16 / f16 / float outputs, row- and K-major operands, both parities, the fused and the speculative cast
-    assert len(found) >= 40
+    assert len(found) >= 36
     for name, (ours, compilers, scratch) in found.items():
         assert ours >= 512 and compilers == 0 and scratch == 0, (name, ours, compilers, scratch)
