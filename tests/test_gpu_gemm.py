@@ -606,6 +606,30 @@ def test_generic_and_direct_to_lds_kernels_agree_to_the_bit(be, m, n, k, out_dty
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize('m,n,k', [(4396, 4616, 384), (4352, 4608, 640), (8192, 4352, 256)])
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('mode', ['plain', 'bias_and_sum'])
+def test_several_rounds_of_tiles_agree_with_the_generic_kernel(be, m, n, k, out_dtype, mode):
+    """More 256 x 256 tiles than compute units (several rounds of workgroups, whole tiles and tiles on the ragged edges
+    mixed), every output type, with and without bias and sum: the direct-to-LDS kernel compared bit for bit with the
+    generic kernel (the same operands with 16 zero bytes appended to every row)."""
+    a, b = _gpu_codes((m, k), 5, 5 * m + k), _gpu_codes((n, k), 6, 11 * n + k)
+    sa, sb = torch.tensor(0.5, device='cuda'), torch.tensor(0.125, device='cuda')
+    a2, b2 = torch.nn.functional.pad(a, (0, 16)).contiguous(), torch.nn.functional.pad(b, (0, 16)).contiguous()
+    g = torch.Generator(device='cuda').manual_seed(m + n)
+    bias = prev = None
+    if mode == 'bias_and_sum':
+        bias = torch.randn(m, device='cuda', generator=g).to(out_dtype)
+        prev = torch.randn(n, m, device='cuda', generator=g).to(out_dtype)
+    outs = []
+    for x, y in ((a, b), (a2, b2)):
+        out = prev.clone() if prev is not None else torch.full((n, m), float('nan'), dtype=out_dtype, device='cuda')
+        outs.append(be.fp8_gemm(x, 5, sa, y, 6, sb, out, accumulate=prev is not None, bias=bias))
+    assert torch.equal(outs[0].view(torch.int32 if out_dtype == torch.float32 else torch.int16),
+                       outs[1].view(torch.int32 if out_dtype == torch.float32 else torch.int16))
+    assert not bool(outs[0].isnan().any())
+
+
 def test_random_small_ragged_problems_with_bias_and_accumulation(be):
     """Random shapes up to 700 x 700 with K both a multiple of 128 (direct-to-LDS kernel, whose 256 x 256 tiles are
     mostly padding here) and not (generic kernel), every output type, with and without bias and accumulation."""
