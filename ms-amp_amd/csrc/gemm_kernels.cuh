@@ -869,11 +869,11 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                             }
                         }
                         uint8_t* qo = qa.q + static_cast<size_t>(grow) * NC + gcol;
-                        const uint32_t c0 = quant4<MSAMP_DT_E4M3>(rr[0] * guess, rr[1] * guess, rr[2] * guess, rr[3] * guess);
+                        const uint32_t c0 = quant4_in_range<MSAMP_DT_E4M3>(rr[0] * guess, rr[1] * guess, rr[2] * guess, rr[3] * guess);
                         if constexpr (kEsz == 4) {
                             if (ok[t]) __builtin_nontemporal_store(c0, reinterpret_cast<uint32_t*>(qo));
                         } else {
-                            const uint32_t c1 = quant4<MSAMP_DT_E4M3>(rr[4] * guess, rr[5] * guess, rr[6] * guess, rr[7] * guess);
+                            const uint32_t c1 = quant4_in_range<MSAMP_DT_E4M3>(rr[4] * guess, rr[5] * guess, rr[6] * guess, rr[7] * guess);
                             typedef uint32_t v2u_t __attribute__((ext_vector_type(2)));
                             const v2u_t cc = {c0, c1};
                             if (ok[t]) __builtin_nontemporal_store(cc, reinterpret_cast<v2u_t*>(qo));
@@ -940,7 +940,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                     }
                     if constexpr (QSPEC)
                         *reinterpret_cast<uint32_t*>(cpatch + (h * 16 + l16) * kCPitch + j * 16 + g4 * 4) =
-                            quant4<MSAMP_DT_E4M3>(r0 * guess, r1 * guess, r2 * guess, r3 * guess);
+                            quant4_in_range<MSAMP_DT_E4M3>(r0 * guess, r1 * guess, r2 * guess, r3 * guess);
                 });
             });
             // no wait between the writes above and the reads below, nor before the next unit's writes: the patch is
@@ -1014,23 +1014,31 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         __shared__ uint32_t spec_red[kGemmThreads / kWave];
         m = block_max_u32(m, spec_red);    // valid in lane 0 of wave 0
         if (threadIdx.x == 0) {
-            // fold into the call's one word; the fence puts that before the ticket, and whoever draws the last ticket
-            // therefore sees every workgroup's maximum
+            // Fold into the call's one word, then draw a ticket.  Both are atomics of agent scope on neighbouring words,
+            // carried out where all XCDs meet; the maximum's old value has come back before the ticket is asked for, so
+            // whoever draws the last ticket finds every workgroup's maximum in the word.  No fence: at agent scope a
+            // fence writes this XCD's L2 back, outputs of the other compute units included, once per workgroup.
             uint32_t* w = qa.spec_words;
-            if (m > __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(w, m);
-            __threadfence();
-            const uint32_t ticket = atomicAdd(w + 1, 1u);
+            uint32_t before = 0;
+            if (m > __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+                before = __hip_atomic_fetch_max(w, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(before) : : "memory");
+            const uint32_t ticket = __hip_atomic_fetch_add(w + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if (ticket == gridDim.x - 1) {
-                __threadfence();
                 const uint32_t mm = __hip_atomic_load(w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                w[0] = 0u, w[1] = 0u;    // ready for the next call
+                __hip_atomic_store(w, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);    // ready for the next call
+                __hip_atomic_store(w + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 float am = __uint_as_float(mm);
                 if ((qa.flags & MSAMP_FLAG_NAN_TO_INF) && !(am < __uint_as_float(0x7f800000u))) am = __uint_as_float(0x7f800000u);
                 const float sc = scale_rule(am, guess, qa.fp_max, qa.margin);
                 *qa.amax = am;
                 *qa.scale = sc;
                 *qa.scale_inv = 1.0f / sc;
-                w[2] = __float_as_uint(sc) != __float_as_uint(guess) ? 1u : 0u;    // the codes must be written again
+                // The codes stand if the rule confirms the scale they were written with and every output times that scale
+                // is finite and inside the format (they were converted without clamp or NaN patch); otherwise the
+                // caller's next kernel writes them again from the stored output.
+                const bool stand = __float_as_uint(sc) == __float_as_uint(guess) && am * guess <= qa.fp_max;
+                w[2] = stand ? 0u : 1u;
             }
         }
         return;
