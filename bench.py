@@ -280,6 +280,36 @@ def bench_gemm_sweep(cfg, iters=10, accumulate_row=None, vendor=True):
     return {'rows': rows, 'aggregate': aggregate}
 
 
+def bench_small_gemms(iters=50):
+    """Forward GEMMs of layers too small to fill the chip with 256 x 256 tiles (64 of them each, a quarter of the compute units): the library's pick
+    (128 x 128 tiles), the large tile forced, and hipBLASLt."""
+    import torch
+    from msamp import _backend
+    E4 = _backend.DT_E4M3
+    rows = []
+    for tokens, d_out, d_in in ((2048, 2048, 4096), (1024, 4096, 4096)):
+        x, x_si = fp8_randn((tokens, d_in), 1.0, E4, seed=tokens)
+        w, w_si = fp8_randn((d_out, d_in), 0.02, E4, seed=d_out + 1)
+        y = torch.empty(tokens, d_out, dtype=torch.bfloat16, device='cuda')
+        fn = lambda: _backend.fp8_gemm(w, E4, w_si, x, E4, x_si, y)
+        fl = 2.0 * tokens * d_out * d_in
+        ms = _time_gpu(fn, iters)
+        try:
+            _backend.set_small_tile_limit(0)
+            ms_large = _time_gpu(fn, iters)
+        finally:
+            _backend.set_small_tile_limit(128)
+        row = {'tokens': tokens, 'm': d_out, 'n': tokens, 'k': d_in, 'ms': round(ms, 4), 'tflops': round(fl / ms / 1e9, 1),
+               'frac_mfma': round(fl / ms / 1e9 / FP8_PEAK_TFLOPS, 4),
+               'large_tile_ms': round(ms_large, 4), 'large_tile_tflops': round(fl / ms_large / 1e9, 1)}
+        vms = _time_vendor(x, w, iters)
+        if vms is not None:
+            row['hipblaslt_ms'] = round(vms, 4)
+            row['hipblaslt_tflops'] = round(fl / vms / 1e9, 1)
+        rows.append(row)
+    return rows
+
+
 def _time_vendor(rows_op, cols_op, iters):
     """torch._scaled_mm (hipBLASLt) on FP8 payloads: out[n, m] = rows_op[n, k] . cols_op[m, k]^T, unit scales, bf16 out.
     Operands are uint8 payloads or callables that make them; None if this build of torch does not take the call."""
@@ -726,7 +756,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--skip-cpu', action='store_true', help='leave out the CPU-oracle baseline')
     ap.add_argument('--skip-extra', action='store_true', help='leave out the sweep, cast and Adam kernel sections')
-    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'cast', 'adam', 'grad_side', 'power'), default=None,
+    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'gemm_small', 'cast', 'adam', 'grad_side', 'power'), default=None,
                     help='run one kernel section alone (after the calibration copy), for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -752,6 +782,8 @@ def main():
             out = _round_kernels(bench_grad_side())
         elif args.only == 'power':
             out = bench_power()
+        elif args.only == 'gemm_small':
+            out = bench_small_gemms()
         else:
             out = bench_adam()
         print(json.dumps({'only': args.only, 'result': out}))
@@ -814,6 +846,7 @@ def main():
         result['gemm_sweep'] = {'c4_llama7b': bench_gemm_sweep(LLAMA_7B, accumulate_row='gate')}
         torch.cuda.empty_cache()
         result['gemm_sweep']['c5_llama70b'] = bench_gemm_sweep(LLAMA_70B, iters=5)
+        result['gemm_sweep']['small_layers_fwd'] = bench_small_gemms()
         torch.cuda.empty_cache()
         cast = bench_cast()
         torch.cuda.empty_cache()

@@ -4,6 +4,8 @@
 // X (= B of the API, N rows) and the one that supplies D's columns is Y (= A of the API, M rows).
 #include "gemm_call.h"
 
+#include <atomic>
+
 namespace msamp {
 
 static int dispatch_pair(int x_type, int y_type, const GemmCall& c) {
@@ -19,9 +21,16 @@ static bool kmajor_shape_ok(int NR, int NC, int K, bool xt, bool yt) {
     return K % kBK == 0 && K >= 2 * kBK && fits32 && (!xt || NR % kDmaTile == 0) && (!yt || NC % kDmaTile == 0);
 }
 
+static std::atomic<int> g_small_tile_limit{128};
+int small_tile_limit() { return g_small_tile_limit.load(std::memory_order_relaxed); }
+
 }    // namespace msamp
 
 using namespace msamp;
+
+extern "C" void msamp_set_small_tile_limit(int big_tiles) {
+    msamp::g_small_tile_limit.store(big_tiles < 0 ? 0 : big_tiles, std::memory_order_relaxed);
+}
 
 // words of the workspace that the speculative form of msamp_fp8_gemm_cast uses: running maximum, ticket counter (both
 // left at zero by every call) and the flag its second launch reads

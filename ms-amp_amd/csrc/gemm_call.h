@@ -46,6 +46,9 @@ struct GemmCall {
 template <int XF, int YF>
 int run_gemm_pair(const GemmCall& c);
 
+// Row-major problems of at most this many 256 x 256 tiles take the kernel with 128 x 128 tiles (msamp_set_small_tile_limit).
+int small_tile_limit();
+
 // Implemented with the cast kernels: q = FP8(d * *scale) over n elements, unless *redo is zero (then nothing is done).
 int cast_again_if_flagged(const void* d, int d_dtype, size_t n, const float* scale, uint8_t* q, int q_type, const uint32_t* redo,
                           hipStream_t st);

@@ -1164,6 +1164,10 @@ static int launch_gemm(const uint8_t* X, const uint8_t* Y, void* D, int NR, int 
     return launch_gemm_k<BR, BC, XF, YF, OT, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
 }
 
+}    // namespace msamp
+#include "gemm_small_tile.cuh"
+namespace msamp {
+
 template <int XF, int YF, typename OT>
 static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                      const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
@@ -1171,6 +1175,11 @@ static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC
     // faster one at every size (measured 2.2x from a single 256 x 256 tile up to 121 tiles).  Everything else takes
     // the generic register-staged kernel with 128 x 128 tiles.
     const bool fits32 = static_cast<unsigned long long>(NR) * K < (1ull << 32) && static_cast<unsigned long long>(NC) * K < (1ull << 32);
+    if (K % kBK == 0 && K >= 4 * kBK && fits32) {
+        // few 256 x 256 tiles leave most compute units idle: 128 x 128 tiles then (see gemm_small_tile.cuh)
+        const long big_tiles = static_cast<long>((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
+        if (big_tiles <= small_tile_limit()) return launch_gemm_dma128<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    }
     if (K % kBK == 0 && K >= 2 * kBK && fits32)
         return launch_gemm_dma<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
     return launch_gemm<128, 128, XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);

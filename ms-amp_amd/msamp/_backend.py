@@ -53,6 +53,7 @@ _SIGNATURES = {
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_cast': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp], _i),
     'msamp_mfma_probe': ([_vp, _vp, _i, _i, _vp, _vp], _i),
+    'msamp_set_small_tile_limit': ([_i], None),
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
     'msamp_fp8_norms': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
     'msamp_bucket_amax': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
@@ -556,6 +557,11 @@ def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, sc
         return None
     _check(rc, 'msamp_fp8_gemm_cast')
     return out
+
+
+def set_small_tile_limit(big_tiles):
+    """Row-major GEMMs of at most this many 256 x 256 output tiles run 128 x 128 tiles (default 128, 0 = never)."""
+    load().msamp_set_small_tile_limit(int(big_tiles))
 
 
 def mfma_probe(seed, sink, iters, workgroups):

@@ -630,6 +630,42 @@ def test_several_rounds_of_tiles_agree_with_the_generic_kernel(be, m, n, k, out_
     assert not bool(outs[0].isnan().any())
 
 
+@pytest.mark.parametrize('m,n,k', [(2048, 2048, 4096), (4096, 1024, 4096), (1024, 768, 1024), (2056, 1100, 512), (300, 200, 640),
+                                   (128, 128, 512), (1031, 1999, 1152)])
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize('mode', ['plain', 'bias_and_sum'])
+def test_small_and_large_tiles_agree_to_the_bit(be, m, n, k, out_dtype, mode):
+    """Problems with few 256 x 256 tiles run 128 x 128 tiles (four stages, fragments read a slice ahead).  The same
+    problem through both, the limit set to take the one and then the other: every output equal bit for bit, on whole
+    and ragged tiles, rows that 16-byte stores do not fit, all output types, with and without bias and sum."""
+    for a_dt, b_dt in ((5, 5), (5, 6), (6, 5)):
+        a, b = _gpu_codes((m, k), a_dt, 5 * m + k + a_dt), _gpu_codes((n, k), b_dt, 11 * n + k + b_dt)
+        sa, sb = torch.tensor(0.5, device='cuda'), torch.tensor(0.125, device='cuda')
+        g = torch.Generator(device='cuda').manual_seed(m + n)
+        bias = prev = None
+        if mode == 'bias_and_sum':
+            bias = torch.randn(m, device='cuda', generator=g).to(out_dtype)
+            prev = torch.randn(n, m, device='cuda', generator=g).to(out_dtype)
+        outs = []
+        try:
+            for limit in (1 << 20, 0):
+                be.set_small_tile_limit(limit)
+                buf = torch.full((n + 2, m), 7.0, dtype=out_dtype, device='cuda')
+                out = buf[1:n + 1]
+                if prev is not None:
+                    out.copy_(prev)
+                else:
+                    out.fill_(float('nan'))
+                be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, out, accumulate=prev is not None, bias=bias)
+                assert bool((buf[0] == 7).all()) and bool((buf[n + 1] == 7).all())
+                outs.append(out.clone())
+        finally:
+            be.set_small_tile_limit(128)
+        view = torch.int32 if out_dtype == torch.float32 else torch.int16
+        assert torch.equal(outs[0].view(view), outs[1].view(view)), (a_dt, b_dt)
+        assert not bool(outs[0].isnan().any())
+
+
 def test_random_small_ragged_problems_with_bias_and_accumulation(be):
     """Random shapes up to 700 x 700 with K both a multiple of 128 (direct-to-LDS kernel, whose 256 x 256 tiles are
     mostly padding here) and not (generic kernel), every output type, with and without bias and accumulation."""
