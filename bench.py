@@ -281,32 +281,41 @@ def bench_gemm_sweep(cfg, iters=10, accumulate_row=None, vendor=True):
 
 
 def bench_small_gemms(iters=50):
-    """Forward GEMMs of layers too small to fill the chip with 256 x 256 tiles (64 of them each, a quarter of the compute units): the library's pick
-    (128 x 128 tiles), the large tile forced, and hipBLASLt."""
+    """The three GEMMs of layers too small to fill the chip with 256 x 256 tiles (64 of them per output and fewer):
+    the library's pick (128 x 128 tiles), the large tile forced, and hipBLASLt on the forward problem."""
     import torch
     from msamp import _backend
-    E4 = _backend.DT_E4M3
+    E4, E5 = _backend.DT_E4M3, _backend.DT_E5M2
     rows = []
     for tokens, d_out, d_in in ((2048, 2048, 4096), (1024, 4096, 4096)):
         x, x_si = fp8_randn((tokens, d_in), 1.0, E4, seed=tokens)
         w, w_si = fp8_randn((d_out, d_in), 0.02, E4, seed=d_out + 1)
+        dy, dy_si = fp8_randn((tokens, d_out), 1e-3, E5, seed=d_out + 2)
         y = torch.empty(tokens, d_out, dtype=torch.bfloat16, device='cuda')
-        fn = lambda: _backend.fp8_gemm(w, E4, w_si, x, E4, x_si, y)
-        fl = 2.0 * tokens * d_out * d_in
-        ms = _time_gpu(fn, iters)
-        try:
-            _backend.set_small_tile_limit(0)
-            ms_large = _time_gpu(fn, iters)
-        finally:
-            _backend.set_small_tile_limit(128)
-        row = {'tokens': tokens, 'm': d_out, 'n': tokens, 'k': d_in, 'ms': round(ms, 4), 'tflops': round(fl / ms / 1e9, 1),
-               'frac_mfma': round(fl / ms / 1e9 / FP8_PEAK_TFLOPS, 4),
-               'large_tile_ms': round(ms_large, 4), 'large_tile_tflops': round(fl / ms_large / 1e9, 1)}
-        vms = _time_vendor(x, w, iters)
-        if vms is not None:
-            row['hipblaslt_ms'] = round(vms, 4)
-            row['hipblaslt_tflops'] = round(fl / vms / 1e9, 1)
-        rows.append(row)
+        dx = torch.empty(tokens, d_in, dtype=torch.bfloat16, device='cuda')
+        dw = torch.empty(d_out, d_in, dtype=torch.bfloat16, device='cuda')
+        passes = [
+            ('fwd', lambda: _backend.fp8_gemm(w, E4, w_si, x, E4, x_si, y), (d_out, tokens, d_in)),
+            ('dgrad', lambda: _backend.fp8_gemm(w, E4, w_si, dy, E5, dy_si, dx, a_kmajor=True), (d_in, tokens, d_out)),
+            ('wgrad', lambda: _backend.fp8_gemm(x, E4, x_si, dy, E5, dy_si, dw, a_kmajor=True, b_kmajor=True), (d_in, d_out, tokens)),
+        ]
+        for pname, fn, (m, n, k) in passes:
+            fl = 2.0 * m * n * k
+            ms = _time_gpu(fn, iters)
+            try:
+                _backend.set_small_tile_limit(0)
+                ms_large = _time_gpu(fn, iters)
+            finally:
+                _backend.set_small_tile_limit(128)
+            row = {'tokens': tokens, 'pass': pname, 'm': m, 'n': n, 'k': k, 'ms': round(ms, 4), 'tflops': round(fl / ms / 1e9, 1),
+                   'frac_mfma': round(fl / ms / 1e9 / FP8_PEAK_TFLOPS, 4),
+                   'large_tile_ms': round(ms_large, 4), 'large_tile_tflops': round(fl / ms_large / 1e9, 1)}
+            if pname == 'fwd':
+                vms = _time_vendor(x, w, iters)
+                if vms is not None:
+                    row['hipblaslt_ms'] = round(vms, 4)
+                    row['hipblaslt_tflops'] = round(fl / vms / 1e9, 1)
+            rows.append(row)
     return rows
 
 
@@ -846,7 +855,7 @@ def main():
         result['gemm_sweep'] = {'c4_llama7b': bench_gemm_sweep(LLAMA_7B, accumulate_row='gate')}
         torch.cuda.empty_cache()
         result['gemm_sweep']['c5_llama70b'] = bench_gemm_sweep(LLAMA_70B, iters=5)
-        result['gemm_sweep']['small_layers_fwd'] = bench_small_gemms()
+        result['gemm_sweep']['small_layers'] = bench_small_gemms()
         torch.cuda.empty_cache()
         cast = bench_cast()
         torch.cuda.empty_cache()

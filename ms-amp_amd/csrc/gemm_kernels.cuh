@@ -1168,6 +1168,13 @@ static int launch_gemm(const uint8_t* X, const uint8_t* Y, void* D, int NR, int 
 #include "gemm_small_tile.cuh"
 namespace msamp {
 
+// few 256 x 256 tiles leave most compute units idle: 128 x 128 tiles then (see gemm_small_tile.cuh)
+static bool takes_small_tiles(int NR, int NC, int K) {
+    const long big_tiles = static_cast<long>((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
+    return K % kBK == 0 && K >= 4 * kBK && big_tiles <= small_tile_limit();
+}
+
+
 template <int XF, int YF, typename OT>
 static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                      const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
@@ -1175,11 +1182,8 @@ static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC
     // faster one at every size (measured 2.2x from a single 256 x 256 tile up to 121 tiles).  Everything else takes
     // the generic register-staged kernel with 128 x 128 tiles.
     const bool fits32 = static_cast<unsigned long long>(NR) * K < (1ull << 32) && static_cast<unsigned long long>(NC) * K < (1ull << 32);
-    if (K % kBK == 0 && K >= 4 * kBK && fits32) {
-        // few 256 x 256 tiles leave most compute units idle: 128 x 128 tiles then (see gemm_small_tile.cuh)
-        const long big_tiles = static_cast<long>((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
-        if (big_tiles <= small_tile_limit()) return launch_gemm_dma128<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
-    }
+    if (fits32 && takes_small_tiles(NR, NC, K))
+        return launch_gemm_dma128<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
     if (K % kBK == 0 && K >= 2 * kBK && fits32)
         return launch_gemm_dma<XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
     return launch_gemm<128, 128, XF, YF, OT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
@@ -1198,16 +1202,25 @@ static int pick_out(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, in
     }
 }
 
+template <int XF, int YF, typename OT, bool XT, bool YT>
+static int pick_tile_kmajor(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs, const float* ys,
+                            int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    // (the entry point has checked the shape: whole 256-row tiles of every K-major operand, 32-bit offsets)
+    if (takes_small_tiles(NR, NC, K))
+        return launch_gemm_dma128<XF, YF, OT, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+    return launch_gemm_dma<XF, YF, OT, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+}
+
 template <int XF, int YF, bool XT, bool YT>
 static int pick_out_kmajor(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, int NR, int NC, int K, const float* xs,
                            const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     switch (d_dtype) {
         case MSAMP_DT_F32:
-            return launch_gemm_dma<XF, YF, float, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+            return pick_tile_kmajor<XF, YF, float, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
         case MSAMP_DT_F16:
-            return launch_gemm_dma<XF, YF, f16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+            return pick_tile_kmajor<XF, YF, f16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
         default:
-            return launch_gemm_dma<XF, YF, bf16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+            return pick_tile_kmajor<XF, YF, bf16_t, XT, YT>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
     }
 }
 

@@ -1,6 +1,8 @@
 // The direct-to-LDS FP8 GEMM with 128 x 128 output tiles, for problems that leave most compute units idle with
-// 256 x 256 tiles (a 2048 x 2048 output is 64 of those, a quarter of the chip, and 256 of these).  Row-major
-// (K-contiguous) operands, K a multiple of 128 and at least 512.
+// 256 x 256 tiles (a 2048 x 2048 output is 64 of those, a quarter of the chip, and 256 of these).  K a multiple of 128
+// and at least 512; operands row-major (K-contiguous) or, with XT / YT, K-major ([K][rows], rows a multiple of 128):
+// the slice then lies in LDS as 128 k-rows of 128 bytes, the 16-byte position XOR-ed with k % 8, and the fragments
+// come from the transposing LDS read, as in the large tile.
 //
 // Four wavefronts, each owning a 64 x 64 quadrant as 4 x 4 accumulators of the 16x16x128 FP8 MFMA, in fixed AGPRs like
 // those of the large tile (block (i, j) in a[16i + 4j .. + 3]; left to the register allocator they were renumbered
@@ -27,7 +29,7 @@ constexpr int kSmallTile = 128;
 constexpr int kSmallStage = 2 * kSmallTile * kBK;    // 32 KiB
 constexpr int kSmallStages = 5;    // all 160 KiB of the LDS
 
-template <int XF, int YF, typename OT>
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma128_kernel(const uint8_t* __restrict__ X, const uint8_t* __restrict__ Y,
                                                                         OT* __restrict__ D, int NR, int NC, int K,
                                                                         const float* __restrict__ x_scale_inv,
@@ -45,7 +47,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma128_kernel(const uin
 
     // ---- global -> LDS: one wave instruction fills 8 rows of 128 bytes (lane l: row l / 8, 16-byte position l % 8,
     // fetching the logical chunk position ^ swizzle(row)); rows past the end of the matrix are clamped to its last row
+    // K-major operand: one wave instruction fills 8 k-rows of 128 bytes (lane l: k-row l / 8, position l % 8, fetching
+    // the logical chunk position ^ (k-row % 8))
     const int chunk = (lane & 7) ^ (lane >> 3) ^ (wave & 1);
+    const int chunk_t = (lane & 7) ^ (lane >> 3);
     const uint32_t lds_base = __builtin_amdgcn_readfirstlane(
         static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) uint8_t*)smem)));
     uint32_t xoff[4], yoff[4];
@@ -55,13 +60,17 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma128_kernel(const uin
         int gx = row0 + r, gy = col0 + r;
         gx = gx < NR ? gx : NR - 1;
         gy = gy < NC ? gy : NC - 1;
-        xoff[i] = static_cast<uint32_t>(gx) * static_cast<uint32_t>(K) + chunk * 16;
-        yoff[i] = static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
+        const int krow = (i * 4 + wave) * 8 + (lane >> 3);
+        xoff[i] = XT ? static_cast<uint32_t>(krow) * static_cast<uint32_t>(NR) + row0 + chunk_t * 16
+                     : static_cast<uint32_t>(gx) * static_cast<uint32_t>(K) + chunk * 16;
+        yoff[i] = YT ? static_cast<uint32_t>(krow) * static_cast<uint32_t>(NC) + col0 + chunk_t * 16
+                     : static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
     }
     // one of the 8 loads of a slice (0..3: X rows, 4..7: Y rows); assembly for the reason given at the large tile
     auto dma = [&](int kt, int which) __attribute__((always_inline)) {
         const bool is_x = which < 4;
-        const uint8_t* src = (is_x ? X : Y) + static_cast<size_t>(kt) * kBK;
+        const size_t slice = static_cast<size_t>(kt) * kBK;
+        const uint8_t* src = is_x ? X + (XT ? slice * NR : slice) : Y + (YT ? slice * NC : slice);
         const uint32_t off = is_x ? xoff[which] : yoff[which - 4];
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + (kt % kSmallStages) * kSmallStage +
                                                             (is_x ? 0 : kSmallTile * kBK) + ((which & 3) * 4 + wave) * 1024);
@@ -79,14 +88,28 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma128_kernel(const uin
     const int off_lo = ((2 * g4) ^ fsw) << 4;
     const int xrow = (wr * 64 + l16) * kBK;
     const int yrow = kSmallTile * kBK + (wc * 64 + l16) * kBK;
-    // piece p of a slice's 16: 0..7 X (block p / 2, half p % 2), 8..15 Y
+    const int tj = l16 >> 1;
+    const int t_lane = (g4 * 32 + tj) * kBK + (l16 & 1) * 8;    // k-row and 8-byte half of this lane's transposing reads
+    // A slice's fragments arrive in pieces: two 16-byte reads per 16-row block of a row-major operand (block p / 2, half
+    // p % 2), four 8-byte transposing reads per block of a K-major one (block p / 4, eight k each); X pieces first.
+    constexpr int kPX = XT ? 16 : 8, kPY = YT ? 16 : 8, kPieces = kPX + kPY;
     auto read_piece = [&](int* fxd, int* fyd, int kt, int p) __attribute__((always_inline)) {
         const uint8_t* base = smem + (kt % kSmallStages) * kSmallStage;
-        const bool is_x = p < 8;
-        const int b = (p & 7) >> 1, hf = p & 1;
-        const v4i val = *reinterpret_cast<const v4i*>(base + (is_x ? xrow : yrow) + b * 16 * kBK + (off_lo ^ (hf * 16)));
-        int* d = (is_x ? fxd : fyd) + b * 8 + hf * 4;
-        d[0] = val[0], d[1] = val[1], d[2] = val[2], d[3] = val[3];
+        const bool is_x = p < kPX;
+        const int q = is_x ? p : p - kPX;
+        if ((is_x && !XT) || (!is_x && !YT)) {
+            const int b = q >> 1, hf = q & 1;
+            const v4i val = *reinterpret_cast<const v4i*>(base + (is_x ? xrow : yrow) + b * 16 * kBK + (off_lo ^ (hf * 16)));
+            int* d = (is_x ? fxd : fyd) + b * 8 + hf * 4;
+            d[0] = val[0], d[1] = val[1], d[2] = val[2], d[3] = val[3];
+        } else {
+            const int b = q >> 2, qq = q & 3;
+            const int wq = is_x ? wr : wc;
+            const int addr = (is_x ? 0 : kSmallTile * kBK) + t_lane + (qq * 8) * kBK + (((wq * 4 + b) ^ tj) << 4);
+            const v2i val = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)(base + addr));
+            int* d = (is_x ? fxd : fyd) + b * 8 + qq * 2;
+            d[0] = val[0], d[1] = val[1];
+        }
     };
 
     acc_clear();
@@ -107,12 +130,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma128_kernel(const uin
                 const v8i vx = {cx[0], cx[1], cx[2], cx[3], cx[4], cx[5], cx[6], cx[7]};
                 const v8i vy = {cy[0], cy[1], cy[2], cy[3], cy[4], cy[5], cy[6], cy[7]};
                 mfma_fixed<i * 4 + j, cb, bl>(vy, vx);
-                // the 16 reads go with the first eight MFMAs, two each, and have come back by the barrier that follows the
-                // last one; nothing moves across, so they stay spread as written
+                // the fragment reads go with the first eight MFMAs (two to four each) and have come back by the barrier that
+                // follows the last one; nothing moves across, so they stay spread as written
                 constexpr int n = j * 4 + i;
                 if (do_read && n < 8) {
-                    read_piece(fx[cur ^ 1], fy[cur ^ 1], rd_kt, 2 * n);
-                    read_piece(fx[cur ^ 1], fy[cur ^ 1], rd_kt, 2 * n + 1);
+#pragma unroll
+                    for (int p = n * kPieces / 8; p < (n + 1) * kPieces / 8; ++p) read_piece(fx[cur ^ 1], fy[cur ^ 1], rd_kt, p);
                 }
                 // the eight tile loads of slice ld_kt, one every other MFMA: issued in one go they hold the wave, and with
                 // it its MFMAs, for as long as the memory pipe takes to accept them
@@ -132,7 +155,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma128_kernel(const uin
     wait_vmcnt<24>();
     __syncthreads();
 #pragma unroll
-    for (int p = 0; p < 16; ++p) read_piece(fx[0], fy[0], 0, p);
+    for (int p = 0; p < kPieces; ++p) read_piece(fx[0], fy[0], 0, p);
 
     // Before the step of slice kt: slices kt + 1 .. kt + 3 are on their way (24 loads of this wave), slice kt is in
     // registers.  Wait for slice kt + 1, meet (it has landed in every wave's part of the stage, and nobody reads the
@@ -252,12 +275,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma128_kernel(const uin
     });
 }
 
-template <int XF, int YF, typename OT>
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
 static int launch_gemm_dma128(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs, const float* ys,
                               int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     constexpr int smem = kSmallStages * kSmallStage;
     static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
-    auto kern = fp8_gemm_dma128_kernel<XF, YF, OT>;
+    auto kern = fp8_gemm_dma128_kernel<XF, YF, OT, XT, YT>;
     if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma128_kernel)");

@@ -666,6 +666,34 @@ def test_small_and_large_tiles_agree_to_the_bit(be, m, n, k, out_dtype, mode):
         assert not bool(outs[0].isnan().any())
 
 
+@pytest.mark.parametrize('m,n,k', [(2048, 2048, 1024), (1024, 512, 640), (256, 256, 512), (2048, 1024, 4096), (512, 3072, 1152)])
+@pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('both', [False, True])
+def test_small_tiles_read_kmajor_operands_like_the_large_tile(be, m, n, k, out_dtype, both):
+    """The backward GEMMs of a small layer hand their operands over K-major ([K, rows]).  The kernel with 128 x 128
+    tiles reads them in place as the large one does (k-rows of 128 bytes in LDS, transposing reads): both kernels on
+    the same operands, equal bit for bit, and equal to the row-major call on the transposed copies."""
+    for a_dt, b_dt in ((5, 6), (5, 5), (6, 6)):
+        a, b = _gpu_codes((m, k), a_dt, 3 * m + k + a_dt), _gpu_codes((n, k), b_dt, 7 * n + k + b_dt)
+        sa, sb = torch.tensor(0.25, device='cuda'), torch.tensor(2.0, device='cuda')
+        a_t, b_t = a.t().contiguous(), b.t().contiguous()
+        outs = []
+        try:
+            for limit in (1 << 20, 0):
+                be.set_small_tile_limit(limit)
+                out = torch.full((n, m), float('nan'), dtype=out_dtype, device='cuda')
+                be.fp8_gemm(a_t, a_dt, sa, b_t if both else b, b_dt, sb, out, a_kmajor=True, b_kmajor=both)
+                outs.append(out)
+            be.set_small_tile_limit(1 << 20)
+            outs.append(be.fp8_gemm(a, a_dt, sa, b, b_dt, sb, torch.full((n, m), float('nan'), dtype=out_dtype, device='cuda')))
+        finally:
+            be.set_small_tile_limit(128)
+        view = torch.int32 if out_dtype == torch.float32 else torch.int16
+        assert torch.equal(outs[0].view(view), outs[1].view(view)), (a_dt, b_dt)
+        assert torch.equal(outs[0].view(view), outs[2].view(view)), (a_dt, b_dt)
+        assert not bool(outs[0].isnan().any())
+
+
 def test_random_small_ragged_problems_with_bias_and_accumulation(be):
     """Random shapes up to 700 x 700 with K both a multiple of 128 (direct-to-LDS kernel, whose 256 x 256 tiles are
     mostly padding here) and not (generic kernel), every output type, with and without bias and accumulation."""
