@@ -292,9 +292,9 @@ int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, 
 
 /* msamp_fp8_gemm with row-major operands runs 256 x 256 output tiles, one workgroup each; a problem with few of them
  * (a 2048 x 2048 output has 64, a quarter of the compute units) runs 128 x 128 tiles instead when it has at most
- * `big_tiles` of the large ones, K is a multiple of 128 and at least 512.  Same bits either way.  Default 128 (up to two
- * small tiles per compute unit: measured faster up to there); 0 = the large tile always.  Process-wide; no
- * counterpart in the reference. */
+ * `big_tiles` of the large ones (at most half that many if K < 3072), K is a multiple of 128 and at least 512.  Same
+ * bits either way.  Default 128 (up to two small tiles per compute unit: measured faster up to there); 0 = the large
+ * tile always.  Process-wide; no counterpart in the reference. */
 void msamp_set_small_tile_limit(int big_tiles);
 
 /* Calibration aid, no counterpart in the reference: `workgroups` workgroups of four wavefronts each issue
