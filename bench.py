@@ -627,8 +627,9 @@ def cpu_baseline():
 
 def bench_power(seconds=2.0):
     """Socket power and shader clock, sampled from the amdgpu driver's sysfs files at 20 Hz by a host thread, while
-    (a) nothing runs, (b) the FP8 GEMM of the Llama-70B gate projection [16384 x 28672 x 8192] and (c) a register-only
-    FP8 MFMA loop (msamp_mfma_probe) each run back to back for `seconds`.  Reported so that a GEMM rate can be read
+    (a) nothing runs, (b) the FP8 GEMMs of the Llama-70B gate projection [16384 x 28672 x 8192] and of the Llama-7B QKV
+    projection [16384 x 12288 x 4096] and (c) a register-only FP8 MFMA loop (msamp_mfma_probe) each run back to back for
+    `seconds`.  Reported so that a GEMM rate can be read
     against what the matrix pipes sustain under the device's power limit, not only against the nominal peak."""
     import glob
     import threading
@@ -712,6 +713,16 @@ def bench_power(seconds=2.0):
     ms, row = sample_while(lambda: be.fp8_gemm(w, be.DT_E4M3, ws, x, be.DT_E4M3, xs, y), seconds)
     row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(2.0 * tokens * d_out * d_in / ms / 1e9, 1)})
     out['fp8_gemm_16384x28672x8192'] = row
+    del x, w, y
+
+    # the forward GEMM of the Llama-7B QKV projection: K = 4096, where the time outside the K loop weighs most
+    d_out, d_in = 12288, 4096
+    x, xs = quantized((tokens, d_in), 1.0)
+    w, ws = quantized((d_out, d_in), 0.02)
+    y = torch.empty(tokens, d_out, dtype=torch.bfloat16, device='cuda')
+    ms, row = sample_while(lambda: be.fp8_gemm(w, be.DT_E4M3, ws, x, be.DT_E4M3, xs, y), seconds)
+    row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(2.0 * tokens * d_out * d_in / ms / 1e9, 1)})
+    out['fp8_gemm_16384x12288x4096'] = row
     del x, w, y
 
     seed = quantized((4096, ), 1.0)[0]
