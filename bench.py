@@ -729,12 +729,13 @@ def bench_power(seconds=2.0):
     sink = torch.zeros(1, device='cuda')
     flop = [0.0]
 
-    def probe():
-        flop[0] = be.mfma_probe(seed, sink, 20000, 1024)
+    for key, distinct in (('register_only_fp8_mfma_loop', False), ('register_only_fp8_mfma_loop_8x8_operands', True)):
+        def probe():
+            flop[0] = be.mfma_probe(seed, sink, 20000, 1024, distinct_operands=distinct)
 
-    ms, row = sample_while(probe, seconds)
-    row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(flop[0] / ms / 1e9, 1)})
-    out['register_only_fp8_mfma_loop'] = row
+        ms, row = sample_while(probe, seconds)
+        row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(flop[0] / ms / 1e9, 1)})
+        out[key] = row
     return out
 
 

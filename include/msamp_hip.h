@@ -298,11 +298,14 @@ int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, 
 void msamp_set_small_tile_limit(int big_tiles);
 
 /* Calibration aid, no counterpart in the reference: `workgroups` workgroups of four wavefronts each issue
- * iters x 16 FP8 16x16x128 MFMAs on registers loaded once from seed (4096 bytes of FP8 codes, device memory); nothing
- * else moves and nothing is written (sink: one float of device memory, never stored to in practice).  *flop (host,
+ * iters x 16 FP8 16x16x128 MFMAs (iters a multiple of 4) on registers loaded once from seed (4096 bytes of FP8 codes,
+ * device memory); nothing else moves and nothing is written (sink: one float of device memory, never stored to in
+ * practice).  distinct_operands == 0: every MFMA takes the same two operands; != 0: eight X and eight Y fragments,
+ * every pair in turn as in a K slice of the GEMM, so that the operand buses toggle as they do there.  *flop (host,
  * may be null) receives the floating-point operations of the launch.  Timed, it gives the rate the matrix pipes
  * sustain on this device under its power limit, the practical ceiling beside the nominal peak. */
-int msamp_mfma_probe(const void* seed, float* sink, int iters, int workgroups, double* flop, msamp_stream_t stream);
+int msamp_mfma_probe(const void* seed, float* sink, int iters, int workgroups, int distinct_operands, double* flop,
+                     msamp_stream_t stream);
 
 /* msamp_adamw.adamw_fp8_stage1_compute (adamw.cu:99-127): fp32 param/grad, quantized moments;
  * updates param in place and atomically maxes |m'|, |v'| into the two amax cells.

@@ -119,21 +119,29 @@ extern "C" int msamp_fp8_gemm(const uint8_t* a, int a_type, const float* a_scale
 
 // Calibration aid: what the matrix pipes of this device sustain when nothing else moves.  Every wavefront issues
 // 16x16x128 FP8 MFMAs on registers it loaded once; the sum is stored only if it equals a value it cannot take, so
-// the loop is not optimised away and nothing is written.
+// the loop is not optimised away and nothing is written.  FRAGS = 1: the same two operands for every MFMA (the
+// operand buses never toggle); FRAGS = 8: eight X and eight Y fragments, every pair once per turn as in a K slice of
+// the GEMM, so that consecutive MFMAs see different operands.
 namespace msamp {
 typedef int mfma_probe_v8i __attribute__((ext_vector_type(8)));
 typedef float mfma_probe_v4f __attribute__((ext_vector_type(4)));
+template <int FRAGS>
 __global__ __launch_bounds__(256) void mfma_probe_kernel(const int* __restrict__ seed, float* __restrict__ sink, int iters) {
-    mfma_probe_v8i a, b;
-    for (int i = 0; i < 8; ++i) {
-        a[i] = seed[(threadIdx.x * 8 + i) & 1023];
-        b[i] = seed[(threadIdx.x * 8 + i + 512) & 1023];
-    }
+    mfma_probe_v8i a[FRAGS], b[FRAGS];
+    for (int f = 0; f < FRAGS; ++f)
+        for (int i = 0; i < 8; ++i) {
+            a[f][i] = seed[(threadIdx.x * 8 + i + f * 37) & 1023];
+            b[f][i] = seed[(threadIdx.x * 8 + i + 512 + f * 53) & 1023];
+        }
     mfma_probe_v4f acc[16];
     for (int i = 0; i < 16; ++i) acc[i] = mfma_probe_v4f{0, 0, 0, 0};
-    for (int it = 0; it < iters; ++it) {
+    constexpr int kTurns = FRAGS == 1 ? 1 : 4;    // 16 or 64 MFMAs per turn of the loop
+    for (int it = 0; it < iters; it += kTurns) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[i], 0, 0, 0, 0, 0, 0);
+        for (int n = 0; n < 16 * kTurns; ++n) {
+            const int i = (n / FRAGS) % FRAGS, j = n % FRAGS;
+            acc[n % 16] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[i], b[j], acc[n % 16], 0, 0, 0, 0, 0, 0);
+        }
     }
     float s = 0;
     for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
@@ -141,12 +149,17 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(const int* __restrict__
 }
 }    // namespace msamp
 
-extern "C" int msamp_mfma_probe(const void* seed, float* sink, int iters, int workgroups, double* flop, msamp_stream_t stream) {
+extern "C" int msamp_mfma_probe(const void* seed, float* sink, int iters, int workgroups, int distinct_operands, double* flop,
+                                msamp_stream_t stream) {
     MSAMP_REQUIRE(seed && sink, MSAMP_ERR_NULL, "msamp_mfma_probe: null pointer");
-    MSAMP_REQUIRE(iters > 0 && workgroups > 0 && workgroups <= 65536, MSAMP_ERR_SHAPE, "msamp_mfma_probe: iters=%d workgroups=%d",
-                  iters, workgroups);
-    hipLaunchKernelGGL(mfma_probe_kernel, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const int*>(seed), sink, iters);
+    MSAMP_REQUIRE(iters > 0 && iters % 4 == 0 && workgroups > 0 && workgroups <= 65536, MSAMP_ERR_SHAPE,
+                  "msamp_mfma_probe: iters=%d (a positive multiple of 4) workgroups=%d", iters, workgroups);
+    if (distinct_operands)
+        hipLaunchKernelGGL(mfma_probe_kernel<8>, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const int*>(seed), sink, iters);
+    else
+        hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(workgroups), dim3(256), 0, static_cast<hipStream_t>(stream),
+                           static_cast<const int*>(seed), sink, iters);
     if (flop) *flop = 4.0 * workgroups * iters * 16.0 * 2.0 * 16 * 16 * 128;
     MSAMP_CHECK_LAUNCH("msamp_mfma_probe");
     return MSAMP_OK;

@@ -52,7 +52,7 @@ _SIGNATURES = {
     'msamp_fp8_gemm': ([_vp, _i, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_kmajor': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_fp8_gemm_cast': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp], _i),
-    'msamp_mfma_probe': ([_vp, _vp, _i, _i, _vp, _vp], _i),
+    'msamp_mfma_probe': ([_vp, _vp, _i, _i, _i, _vp, _vp], _i),
     'msamp_set_small_tile_limit': ([_i], None),
     'msamp_scale_update_groups': ([_vp, _i, _i, _vp], _i),
     'msamp_fp8_norms': ([_vp, _i, _vp, _i, _i, _i, _vp], _i),
@@ -564,14 +564,15 @@ def set_small_tile_limit(big_tiles):
     load().msamp_set_small_tile_limit(int(big_tiles))
 
 
-def mfma_probe(seed, sink, iters, workgroups):
+def mfma_probe(seed, sink, iters, workgroups, distinct_operands=False):
     """Launch the register-only FP8 MFMA loop (calibration aid); returns the floating-point operations of the launch.
-    seed: at least 4096 bytes of FP8 codes on the device, sink: one float32 on the device."""
+    seed: at least 4096 bytes of FP8 codes on the device, sink: one float32 on the device.  distinct_operands: eight X
+    and eight Y fragments taken in turn instead of one pair for every MFMA."""
     assert seed.is_cuda and seed.is_contiguous() and seed.numel() * seed.element_size() >= 4096
     assert sink.is_cuda and sink.dtype == torch.float32
     flop = ctypes.c_double(0.0)
-    _check(load().msamp_mfma_probe(_ptr(seed), _ptr(sink), int(iters), int(workgroups), ctypes.byref(flop), _stream()),
-           'msamp_mfma_probe')
+    _check(load().msamp_mfma_probe(_ptr(seed), _ptr(sink), int(iters), int(workgroups), 1 if distinct_operands else 0,
+                                   ctypes.byref(flop), _stream()), 'msamp_mfma_probe')
     return flop.value
 
 
