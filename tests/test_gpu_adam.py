@@ -398,6 +398,26 @@ def test_shifting_step_many_tensors_little_room(be):
     be.check_async_error(block=True)
 
 
+def test_config3_full_size_shifting_step_matches(be):
+    """1.0e9 parameters as 238 tensors of [4096, 1024] and a tail, 61 036 chunks, with the room the optimizer gives them
+    (2816 chunks): one shifting step up and one down from the same state, every tensor compared with the in-place
+    step on the same bytes (all full tensors hold the same bytes, so one in-place result serves them all)."""
+    per, total = 4096 * 1024, 1_000_000_000
+    n_full, tail = total // per, total % per
+    base = _inputs(per, 77, fp8.E4M3, fp8.E5M2)
+    last = {k: (v[:tail].clone() if isinstance(v, torch.Tensor) else {kk: vv.clone() for kk, vv in v.items()})
+            for k, v in base.items()}
+    want_full, want_tail = _fused(be, [base, last], 5, 6, 2)
+    tensors = [base] * n_full + [last]
+    for up in (True, False):
+        moved = _fused_shift(be, tensors, 5, 6, 2, 2816, up=up)
+        assert _same_state(want_tail, moved[-1])
+        for i, d in enumerate(moved[:n_full]):
+            assert _same_state(want_full, d), (up, i)
+        del moved
+    be.check_async_error(block=True)
+
+
 def test_shifting_step_refuses_a_tensor_longer_than_the_room(be):
     """A tensor of 256 chunks with room for 255: some workgroup would have to overwrite a chunk of its own tensor.  The
     kernel flags the layout in the sticky error word, leaves those chunks alone and runs to its end."""
