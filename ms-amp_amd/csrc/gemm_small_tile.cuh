@@ -10,9 +10,9 @@
 // and 128 Y rows of 128 bytes, 32 KiB, brought in by eight direct-to-LDS loads per wavefront with the same swizzle
 // as the large tile; five stages -- the whole LDS -- so that three slices are on their way while one is being read and
 // another worked on (a slice is only 16 MFMAs per wavefront, a fifth of a microsecond, and the way to L2 is close to
-// a microsecond).  The fragments of slice kt + 1 are read from LDS between the first MFMAs of slice kt and the loads
-// of slice kt + 4 go out between the others, one every other MFMA (issued in one go after the barrier they held the
-// wave, and its MFMAs, while the memory pipe accepted them: 0.54 against 0.43 us per slice); one barrier per slice.
+// a microsecond).  The fragments of slice kt + 1 are read from LDS between the first eight MFMAs of slice kt, and the
+// eight loads of slice kt + 4 go out one every other MFMA (issued in one go after the barrier they held the wave, and
+// its MFMAs, while the memory pipe accepted them: 0.54 against 0.43 us per slice); one barrier per slice.
 //
 // Per flop this tile needs twice the L2 -> LDS bytes of the large one (32 KiB per 16 MFMAs per wavefront against
 // 64 KiB per 64), which is what bounds it once every compute unit runs one: 2048 x 2048 x 4096 takes 16.7 us with the
