@@ -631,7 +631,7 @@ def test_several_rounds_of_tiles_agree_with_the_generic_kernel(be, m, n, k, out_
 
 
 @pytest.mark.parametrize('m,n,k', [(2048, 2048, 4096), (4096, 1024, 4096), (1024, 768, 1024), (2056, 1100, 512), (300, 200, 640),
-                                   (128, 128, 512), (1031, 1999, 1152)])
+                                   (128, 128, 512), (1031, 1999, 1152), (1, 1, 512), (33, 65, 1024), (7, 513, 768)])
 @pytest.mark.parametrize('out_dtype', [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('mode', ['plain', 'bias_and_sum'])
 def test_small_and_large_tiles_agree_to_the_bit(be, m, n, k, out_dtype, mode):
