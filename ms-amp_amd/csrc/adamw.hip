@@ -4,6 +4,8 @@
 // multiply-adds, so the second pass reproduces the first one bit for bit.
 #include "common.cuh"
 
+#include <type_traits>
+
 #include <cmath>
 #include <limits>
 
@@ -15,6 +17,7 @@ struct AdamConsts {
     float beta1, beta2, omb1, omb2, eps, step_size, sbc2, inv_sbc2, decay, wd;
     float bound_rsq, bound_eps;    // first pass: |update| <= step_size * |m'| * min(bound_rsq * rsq(v'), bound_eps)
     int adam_mode, maximize, use_decay;
+    int rule_scales;    // the moments' scales follow the scale rule (tensor_scale): what the clamp-free fast path needs
 };
 
 // float step_size and sqrt(bias_correction2) from float betas and a double pow, then narrowed
@@ -554,11 +557,67 @@ struct SpecState {
 
 // One group of eight elements at element i: new codes of the weight, exp_avg and exp_avg_sq from the raw inputs, the
 // maxima folded into `st` (TRACK; without it only the codes are made: the other round of a chunk).  Nothing is stored.
-template <int WDT, int GDT, bool L2, bool TRACK = true>
+// ---- the step with the dequantization factors folded into the coefficients ------------------------------------------
+// With all four factors (weight, gradient, exp_avg, exp_avg_sq scale_inv) exact powers of two -- what the scale rule
+// produces -- multiplying by them is exact, so it commutes with the roundings of the chain:
+//   (w * w_si) * decay            = w * (w_si * decay)
+//   (beta1 * m) * inv_m           = (beta1 * inv_m) * m
+//   omb1 * (g * g_si)             = (omb1 * g_si) * g
+//   (beta2 * v) * inv_v           = (beta2 * inv_v) * v
+//   omb2 * ((g * g_si)(g * g_si)) = (omb2 * g_si^2) * (g * g)      (g * g is exact: an FP8 code has at most 4 significant bits)
+// bit for bit, as long as nothing underflows or overflows on the way: 8 instructions per element instead of 12.
+// fold_ok() admits factors 2^-40 .. 2^40 and coefficients of ordinary size; the smallest intermediates are then
+// 2^-16 (E5M2) * 2^-40 * 2^-20 and its like, far from the denormals.  Anything else takes the plain chain.
+struct Folded {
+    float cw, cm, cg1, cv, c3;
+};
+__device__ __forceinline__ bool pow2_in_range(float x) {
+    const uint32_t b = __float_as_uint(x) & 0x7fffffffu;
+    const uint32_t e = b >> 23;
+    return (b & 0x007fffffu) == 0u && e >= 127u - 40u && e <= 127u + 40u;
+}
+__device__ __forceinline__ bool ordinary(float c) { return c >= 0x1.0p-20f && c <= 2.0f; }
+__device__ __forceinline__ bool fold_ok(float w_si, float g_si, float inv_m, float inv_v, const AdamConsts& k) {
+    return pow2_in_range(w_si) && pow2_in_range(g_si) && pow2_in_range(inv_m) && pow2_in_range(inv_v) && ordinary(k.beta1) &&
+           ordinary(k.beta2) && ordinary(k.omb1) && ordinary(k.omb2) && ordinary(k.decay);
+}
+__device__ __forceinline__ Folded fold(float w_si, float g_si, float inv_m, float inv_v, const AdamConsts& k) {
+    Folded f;
+    // (the same in every lane; this part has no scalar float arithmetic, so they are worked out in a vector register and
+    // handed to scalar ones, where they cost the loop nothing)
+    auto uniform = [](float x) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(x))); };
+    f.cw = uniform(w_si * k.decay), f.cm = uniform(k.beta1 * inv_m), f.cg1 = uniform(k.omb1 * g_si);
+    f.cv = uniform(k.beta2 * inv_v), f.c3 = uniform(k.omb2 * (g_si * g_si));
+    return f;
+}
+// pj, m', v' of one element from its raw codes (decoupled decay only: the L2 form needs the plain gradient)
+__device__ __forceinline__ void prepare_folded(float w_raw, float g_raw, float m_raw, float v_raw, const Folded& f, float& pj,
+                                               float& m_new, float& v_new) {
+#pragma clang fp contract(off)
+    pj = w_raw * f.cw;
+    const float t2 = f.cm * m_raw;
+    const float t3 = f.cg1 * g_raw;
+    m_new = t2 + t3;
+    const float u2 = f.cv * v_raw;
+    const float gg = g_raw * g_raw;
+    const float u3 = f.c3 * gg;
+    v_new = u2 + u3;
+}
+// any of the four packed FP8 codes all ones below the sign: what the converter makes of NaN, Inf and values beyond the
+// format (E4M3; the codes of finite values in range end at 0x7e)
+__device__ __forceinline__ bool any_code_7f(uint32_t w) { return (((w & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u) != 0u; }
+
+template <int WDT, int GDT, bool L2, bool TRACK = true, bool FAST = false>
 __device__ __forceinline__ void spec_group(const msamp_adamw_tensor& d, size_t i, const Raw8<WDT>& rw, const Raw8<GDT>& rg,
                                            const Raw8<MSAMP_DT_E4M3>& rm, const Raw8<MSAMP_DT_F16>& rv, float w_si, float g_si,
                                            float inv_m, float inv_v, float ws, float ms, float vs, const AdamConsts& k,
-                                           SpecState& st, Raw8<WDT>& ow, Raw8<MSAMP_DT_E4M3>& om, Raw8<MSAMP_DT_F16>& ov) {
+                                           SpecState& st, Raw8<WDT>& ow, Raw8<MSAMP_DT_E4M3>& om, Raw8<MSAMP_DT_F16>& ov,
+                                           const Folded& fc = Folded{}) {
+    // FAST (the caller has checked fold_ok(), decoupled decay and scales that follow the rule): folded factors; no clamp
+    // in front of the converters -- with the guessed scales confirmed nothing leaves the formats, and a tensor whose
+    // scales are not confirmed is done again through the plain path -- and the codes of exp_avg looked at once per
+    // four for what the converter makes of NaN and Inf, which then take the plain conversion.
+    static_assert(!(FAST && L2), "the folded chain has no plain gradient");
     float hi[kGroup];
     float lo_max = 0.0f, hi_max = 0.0f;
     float eps_v = k.eps;
@@ -570,8 +629,9 @@ __device__ __forceinline__ void spec_group(const msamp_adamw_tensor& d, size_t i
         uint32_t code4[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            float pj, g_plain, m_new, v_new, p_est, err;
-            prepare<L2>(p4[e], g4[e], m4[e], v4[e], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+            float pj, g_plain = 0.0f, m_new, v_new, p_est, err;
+            if constexpr (FAST) prepare_folded(p4[e], g4[e], m4[e], v4[e], fc, pj, m_new, v_new);
+            else prepare<L2>(p4[e], g4[e], m4[e], v4[e], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
             if constexpr (TRACK) {
                 st.mxm = fmaxf(st.mxm, fabsf(m_new));
                 st.mxv = fmaxf(st.mxv, fabsf(v_new));
@@ -584,7 +644,7 @@ __device__ __forceinline__ void spec_group(const msamp_adamw_tensor& d, size_t i
                 code = float_to_f16_bits(lo);
                 same = code == float_to_f16_bits(up);
             } else {
-                const uint32_t two = cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(up), 0u, false);
+                const uint32_t two = FAST ? cvt_pk<WDT>(lo, up, 0u, false) : cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(up), 0u, false);
                 code = two & 0xffu;
                 same = code == ((two >> 8) & 0xffu);
             }
@@ -616,7 +676,13 @@ __device__ __forceinline__ void spec_group(const msamp_adamw_tensor& d, size_t i
         } else {
             ow.w[q] = code4[0] | (code4[1] << 8) | (code4[2] << 16) | (code4[3] << 24);
         }
-        om.w[q] = quant4<MSAMP_DT_E4M3>(m4[0], m4[1], m4[2], m4[3]);
+        if constexpr (FAST) {
+            uint32_t mc = quant4_in_range<MSAMP_DT_E4M3>(m4[0], m4[1], m4[2], m4[3]);
+            if (__builtin_expect(any_code_7f(mc), 0)) mc = quant4<MSAMP_DT_E4M3>(m4[0], m4[1], m4[2], m4[3]);
+            om.w[q] = mc;
+        } else {
+            om.w[q] = quant4<MSAMP_DT_E4M3>(m4[0], m4[1], m4[2], m4[3]);
+        }
         ov.w[2 * q] = float_to_f16_bits(v4[0]) | (float_to_f16_bits(v4[1]) << 16);
         ov.w[2 * q + 1] = float_to_f16_bits(v4[2]) | (float_to_f16_bits(v4[3]) << 16);
     }
@@ -664,12 +730,13 @@ __device__ __forceinline__ void spec_ragged(const msamp_adamw_tensor& d, size_t 
 // The speculative pass between two sets of buffers works on sixteen consecutive elements per lane (16-byte accesses
 // throughout; measured 6 % faster there than the groups of eight that the shifting step below needs for its
 // written-through stores), one lane's sixteen elements at a time:
-template <int WDT, int GDT, bool L2>
+template <int WDT, int GDT, bool L2, bool FAST = false>
 __device__ __forceinline__ void spec_step16(const msamp_adamw_tensor& d, void* w_out, uint8_t* m_out, uint16_t* v_out, size_t i,
                                           float* p, const float* g,
                                           float* m, float* v, float w_si, float g_si, float inv_m, float inv_v, float ws,
                                           float ms, float vs, const AdamConsts& k, float& floor_p, uint32_t& mxp,
-                                          float& mxm, float& mxv) {
+                                          float& mxm, float& mxv, const Folded& fc = Folded{}) {
+    static_assert(!(FAST && L2), "the folded chain has no plain gradient");    // FAST: as in spec_group
     uint32_t wq[kEPT];
     float hi[kEPT];
     float lo_max = 0.0f, hi_max = 0.0f;
@@ -677,8 +744,9 @@ __device__ __forceinline__ void spec_step16(const msamp_adamw_tensor& d, void* w
     asm volatile("" : "+v"(eps_v));
 #pragma unroll
     for (int j = 0; j < kEPT; ++j) {
-        float pj, g_plain, m_new, v_new, p_est, err;
-        prepare<L2>(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
+        float pj, g_plain = 0.0f, m_new, v_new, p_est, err;
+        if constexpr (FAST) prepare_folded(p[j], g[j], m[j], v[j], fc, pj, m_new, v_new);
+        else prepare<L2>(p[j], g[j], m[j], v[j], w_si, g_si, inv_m, inv_v, k, pj, g_plain, m_new, v_new);
         mxm = fmaxf(mxm, fabsf(m_new));
         mxv = fmaxf(mxv, fabsf(v_new));
         estimate(pj, m_new, v_new, k, eps_v, p_est, err);
@@ -689,7 +757,7 @@ __device__ __forceinline__ void spec_step16(const msamp_adamw_tensor& d, void* w
             code = float_to_f16_bits(lo);
             same = code == float_to_f16_bits(up);
         } else {
-            const uint32_t two = cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(up), 0u, false);
+            const uint32_t two = FAST ? cvt_pk<WDT>(lo, up, 0u, false) : cvt_pk<WDT>(sat<WDT>(lo), sat<WDT>(up), 0u, false);
             code = two & 0xffu;
             same = code == ((two >> 8) & 0xffu);
         }
@@ -727,7 +795,17 @@ __device__ __forceinline__ void spec_step16(const msamp_adamw_tensor& d, void* w
         o.w = wq[12] | (wq[13] << 8) | (wq[14] << 16) | (wq[15] << 24);
         *reinterpret_cast<uint4*>(static_cast<uint8_t*>(w_out) + i) = o;
     }
-    store_w16<MSAMP_DT_E4M3>(m_out, i, m);
+    if constexpr (FAST) {
+        uint32_t o[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            o[q] = quant4_in_range<MSAMP_DT_E4M3>(m[4 * q], m[4 * q + 1], m[4 * q + 2], m[4 * q + 3]);
+            if (__builtin_expect(any_code_7f(o[q]), 0)) o[q] = quant4<MSAMP_DT_E4M3>(m[4 * q], m[4 * q + 1], m[4 * q + 2], m[4 * q + 3]);
+        }
+        *reinterpret_cast<uint4*>(m_out + i) = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+        store_w16<MSAMP_DT_E4M3>(m_out, i, m);
+    }
     store_w16<MSAMP_DT_F16>(v_out, i, v);
     floor_p = fmaxf(floor_p, __uint_as_float(wave_max_u32(__float_as_uint(lo_max))));
     const float skip_below = floor_p * 0.999999f;    // room for the roundings of the bounds themselves
@@ -767,13 +845,30 @@ __global__ __launch_bounds__(kAdamThreads) void fused_spec_kernel(msamp_adamw_te
     float floor_p = __uint_as_float(__hip_atomic_load(&d.acc[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     if (!(floor_p >= 0.0f)) floor_p = 0.0f;
     if (base + MSAMP_ADAMW_CHUNK <= n) {
+        // the folded, clamp-free form of the step where the tensor's factors allow it (see spec_group)
+        bool fast = !L2 && k.rule_scales && fold_ok(w_si, g_si, inv_m, inv_v, k);
+        fast = __builtin_amdgcn_readfirstlane(fast);
+        const Folded fc = fold(w_si, g_si, inv_m, inv_v, k);
+        if (!L2 && fast) {
+            if constexpr (!L2) {
 #pragma unroll 1
-        for (int s = 0; s < kSteps; ++s) {
-            const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
-            float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
-            load16<WDT, GDT>(d, i, p, g, m, v);
-            spec_step16<WDT, GDT, L2>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p, mxp,
-                               mxm, mxv);
+                for (int s = 0; s < kSteps; ++s) {
+                    const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
+                    float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
+                    load16<WDT, GDT>(d, i, p, g, m, v);
+                    spec_step16<WDT, GDT, L2, true>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k,
+                                                    floor_p, mxp, mxm, mxv, fc);
+                }
+            }
+        } else {
+#pragma unroll 1
+            for (int s = 0; s < kSteps; ++s) {
+                const size_t i = base + (static_cast<size_t>(s) * kAdamThreads + threadIdx.x) * kEPT;
+                float p[kEPT], g[kEPT], m[kEPT], v[kEPT];
+                load16<WDT, GDT>(d, i, p, g, m, v);
+                spec_step16<WDT, GDT, L2>(d, w_out, m_out, v_out, i, p, g, m, v, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, floor_p,
+                                          mxp, mxm, mxv);
+            }
         }
     } else {
         for (size_t i = base + threadIdx.x; i < n; i += kAdamThreads) {
@@ -1110,35 +1205,50 @@ __global__ __launch_bounds__(kAdamThreads) void fused_shift_kernel(msamp_adamw_t
     };
 
     if (base + MSAMP_ADAMW_CHUNK <= d.numel) {
-#pragma unroll 1
-        for (int s = 0; s < kSpecSteps;) {
-            const size_t i0 = base + static_cast<size_t>(s) * (2 * kGroupSpan) + threadIdx.x * kGroup, i1 = i0 + kGroupSpan;
-            Raw8<WDT> w0, w1, ow;
-            Raw8<GDT> g0, g1;
-            Raw8<MSAMP_DT_E4M3> m0, m1, om;
-            Raw8<MSAMP_DT_F16> v0, v1, ov;
-            w0.load(d.weight, i0), g0.load(d.grad, i0), m0.load(d.exp_avg, i0), v0.load(d.exp_avg_sq, i0);
-            w1.load(d.weight, i1), g1.load(d.grad, i1), m1.load(d.exp_avg, i1), v1.load(d.exp_avg_sq, i1);
-            // the verdict on the chunk underneath: asked for behind this wavefront's own loads (it comes from further away
-            // than they do, and loads return in order), looked at when the first outputs are ready
-            if (!gate_open && lane == 0) posted = __hip_atomic_load(a.verdicts + jv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const SpecState before = st;
-            spec_group<WDT, GDT, L2>(d, i0, w0, g0, m0, v0, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, st, ow, om, ov);
-            if (!gate_open) {
-                const int verdict = gate();
-                // gave up: this chunk is left as it was; the call has failed and the error word says so
-                if (verdict < 0) return;
-                gate_open = true;
-                if (verdict > 0) {    // start the step again
-                    st = before;
-                    continue;
-                }
+        // the folded, clamp-free form of the step where the tensor's factors allow it (see spec_group)
+        bool fast = !L2 && a.tensor_scale && fold_ok(w_si, g_si, inv_m, inv_v, k);
+        fast = __builtin_amdgcn_readfirstlane(fast);
+        const Folded fc = fold(w_si, g_si, inv_m, inv_v, k);
+        // (the loop twice, as a macro: behind a generic lambda the kernel's argument structures moved to the stack)
+#define MSAMP_SHIFT_WALK(FASTV)                                                                                                  \
+    _Pragma("unroll 1") for (int s = 0; s < kSpecSteps;) {                                                                       \
+        const size_t i0 = base + static_cast<size_t>(s) * (2 * kGroupSpan) + threadIdx.x * kGroup, i1 = i0 + kGroupSpan;          \
+        Raw8<WDT> w0, w1, ow;                                                                                                     \
+        Raw8<GDT> g0, g1;                                                                                                         \
+        Raw8<MSAMP_DT_E4M3> m0, m1, om;                                                                                           \
+        Raw8<MSAMP_DT_F16> v0, v1, ov;                                                                                            \
+        w0.load(d.weight, i0), g0.load(d.grad, i0), m0.load(d.exp_avg, i0), v0.load(d.exp_avg_sq, i0);                            \
+        w1.load(d.weight, i1), g1.load(d.grad, i1), m1.load(d.exp_avg, i1), v1.load(d.exp_avg_sq, i1);                            \
+        /* the verdict on the chunk underneath: asked for behind this wavefront's own loads (it comes from further away  */      \
+        /* than they do, and loads return in order), looked at when the first outputs are ready                          */      \
+        if (!gate_open && lane == 0) posted = __hip_atomic_load(a.verdicts + jv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);     \
+        const SpecState before = st;                                                                                              \
+        spec_group<WDT, GDT, L2, true, FASTV>(d, i0, w0, g0, m0, v0, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, st, ow, om, ov, fc); \
+        if (!gate_open) {                                                                                                         \
+            const int verdict = gate();                                                                                           \
+            /* gave up: this chunk is left as it was; the call has failed and the error word says so */                          \
+            if (verdict < 0) return;                                                                                              \
+            gate_open = true;                                                                                                     \
+            if (verdict > 0) { /* start the step again */                                                                         \
+                st = before;                                                                                                      \
+                continue;                                                                                                         \
+            }                                                                                                                     \
+        }                                                                                                                         \
+        ow.template store<true>(w_out, i0), om.template store<true>(m_out, i0), ov.template store<true>(v_out, i0);               \
+        spec_group<WDT, GDT, L2, true, FASTV>(d, i1, w1, g1, m1, v1, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, st, ow, om, ov, fc); \
+        ow.template store<true>(w_out, i1), om.template store<true>(m_out, i1), ov.template store<true>(v_out, i1);               \
+        ++s;                                                                                                                      \
+    }
+        if constexpr (L2) {
+            MSAMP_SHIFT_WALK(false)
+        } else {
+            if (fast) {
+                MSAMP_SHIFT_WALK(true)
+            } else {
+                MSAMP_SHIFT_WALK(false)
             }
-            ow.template store<true>(w_out, i0), om.template store<true>(m_out, i0), ov.template store<true>(v_out, i0);
-            spec_group<WDT, GDT, L2>(d, i1, w1, g1, m1, v1, w_si, g_si, inv_m, inv_v, ws, ms, vs, k, st, ow, om, ov);
-            ow.template store<true>(w_out, i1), om.template store<true>(m_out, i1), ov.template store<true>(v_out, i1);
-            ++s;
         }
+#undef MSAMP_SHIFT_WALK
     } else {
         // the tensor's last, partly filled chunk: element by element, a lane's elements the same in both rounds
         if (!gate_open && gate() < 0) return;
@@ -1385,6 +1495,7 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
     MSAMP_REQUIRE(outputs && redo, MSAMP_ERR_NULL, "msamp_adamw_fp8_fused_speculative: null outputs or redo");
     AdamConsts k;
     const bool l2 = fused_consts(lr, beta1, beta2, eps, weight_decay, step, bias_correction, adam_mode, maximize, k);
+    k.rule_scales = tensor_scale != 0;
     const float w_fp_max = weight_dtype == MSAMP_DT_F16 ? 65504.0f : fp8_max(weight_dtype);
     hipStream_t st = static_cast<hipStream_t>(stream);
     FUSED_LAUNCH(fused_spec_kernel, n_blocks, tensors, block_map, k, outputs);

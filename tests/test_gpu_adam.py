@@ -418,6 +418,36 @@ def test_config3_full_size_shifting_step_matches(be):
     be.check_async_error(block=True)
 
 
+def _rescaled(t, w=0, g=0, m=0, v=0, g_factor=1.0):
+    """The same payloads read through other factors: every scale times 2^k (scale_inv divided), the gradient's scale_inv
+    times g_factor on top.  Dequantized values change, codes do not."""
+    out = {k: (x.clone() if isinstance(x, torch.Tensor) else {kk: vv.clone() for kk, vv in x.items()}) for k, x in t.items()}
+    for key, k in (('wm', w), ('gm', g), ('mm', m), ('vm', v)):
+        out[key]['scale'] = out[key]['scale'] * 2.0 ** k
+        out[key]['scale_inv'] = out[key]['scale_inv'] * 2.0 ** -k
+    out['gm']['scale_inv'] = out['gm']['scale_inv'] * g_factor
+    return out
+
+
+@pytest.mark.parametrize('shifts', [dict(w=28, g=10, m=25, v=20), dict(w=-25, g=-38, m=-27, v=-28), dict(w=45), dict(g=-70),
+                                    dict(m=60, v=-60), dict(g_factor=0.3), dict(g_factor=-1.0), dict(g=12, g_factor=1.0 + 2.0 ** -23)])
+def test_one_pass_steps_fold_their_factors_only_where_that_is_exact(be, shifts):
+    """The one-pass kernels fold the four dequantization factors into the update's coefficients when all of them are
+    powers of two between 2^-40 and 2^40, and take the plain chain otherwise.  Payloads read through factors well inside
+    that range, at its edges, beyond it, and through a gradient factor that is no power of two (or negative): both
+    one-pass forms against the in-place step, which never folds, bit for bit."""
+    sizes = [16384 * 2, 16384 + 4001, 16384 * 5]
+    tensors = [_rescaled(_inputs(n, 1200 + i, fp8.E4M3, fp8.E5M2), **shifts) for i, n in enumerate(sizes)]
+    for step in (2, 3):
+        plain = _fused(be, tensors, 5, 6, step)
+        moved = _fused_shift(be, tensors, 5, 6, step, 8, up=step == 3)
+        spec = _fused(be, tensors, 5, 6, step, speculative=True)
+        for a, b, c in zip(plain, moved, spec):
+            assert _same_state(a, b) and _same_state(a, c), (step, shifts)
+        tensors = [_next_inputs(t, d, 1300 + 10 * step + i, fp8.E5M2) for i, (t, d) in enumerate(zip(tensors, plain))]
+    be.check_async_error(block=True)
+
+
 def test_shifting_step_refuses_a_tensor_longer_than_the_room(be):
     """A tensor of 256 chunks with room for 255: some workgroup would have to overwrite a chunk of its own tensor.  The
     kernel flags the layout in the sticky error word, leaves those chunks alone and runs to its end."""
