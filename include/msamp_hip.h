@@ -282,7 +282,8 @@ int msamp_fp8_gemm_kmajor(const uint8_t* a, int a_type, const float* a_scale_inv
  *    scale does a second launch read d again and rewrite the codes.  On return d holds the (accumulated) product.
  *    Not taken with MSAMP_FLAG_NO_SPECULATION, nor for d_dtype float32.
  * Both need m and n multiples of 256, k a multiple of 128 and at least 256, q_type E4M3, both operands K-major or
- * neither.  d may be null: then only the first form is considered.
+ * neither, and a problem too large for the GEMM with 128 x 128 tiles (msamp_set_small_tile_limit): below that size the
+ * two steps are the faster way.  d may be null: then only the first form is considered.
  * Returns MSAMP_NOT_FUSED (1), having done nothing, when neither form applies and the caller has to take the two steps. */
 #define MSAMP_NOT_FUSED 1
 int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b, int b_type,

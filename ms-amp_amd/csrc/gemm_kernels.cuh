@@ -1168,15 +1168,7 @@ static int launch_gemm(const uint8_t* X, const uint8_t* Y, void* D, int NR, int 
 #include "gemm_small_tile.cuh"
 namespace msamp {
 
-// few 256 x 256 tiles leave most compute units idle: 128 x 128 tiles then (see gemm_small_tile.cuh)
-static bool takes_small_tiles(int NR, int NC, int K) {
-    const long big_tiles = static_cast<long>((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
-    // up to half the limit always (one small tile per compute unit with the default limit); up to the limit where K
-    // is long enough for the second round to pay (measured: 128 large tiles level at K = 2048, 15 % ahead at 4096)
-    const int limit = small_tile_limit();
-    return K % kBK == 0 && K >= 4 * kBK && (big_tiles <= limit / 2 || (big_tiles <= limit && K >= 3072));
-}
-
+// few 256 x 256 tiles leave most compute units idle: 128 x 128 tiles then (takes_small_tiles(), gemm_small_tile.cuh)
 
 template <int XF, int YF, typename OT>
 static int pick_tile(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,

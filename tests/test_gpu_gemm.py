@@ -25,6 +25,15 @@ def be():
     return _backend
 
 
+@pytest.fixture
+def large_tiles_only(be):
+    """Problems small enough for the GEMM with 128 x 128 tiles decline the fused GEMM + cast (the two steps are faster
+    there); with the small tile switched off the fused forms take them, which keeps these small cases on the fused path."""
+    be.set_small_tile_limit(0)
+    yield
+    be.set_small_tile_limit(128)
+
+
 def _rand_fp8(shape, fp8_dt, seed, spread=1.0):
     """Random FP8 payload (finite codes) built by quantizing N(0, spread) on the CPU."""
     g = torch.Generator().manual_seed(seed)
@@ -365,7 +374,7 @@ def _two_steps(be, a, a_dt, sa, b, b_dt, sb, hp, nan_to_inf, kmajor, old_scale=1
 @pytest.mark.parametrize('m,n,k', [(256, 256, 256), (1024, 512, 384), (4096, 4096, 512), (2048, 8192, 256), (512, 256, 640)])
 @pytest.mark.parametrize('hp', [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize('kmajor', [True, False])
-def test_gemm_with_fused_cast_matches_the_two_steps(be, a_dt, b_dt, m, n, k, hp, kmajor):
+def test_gemm_with_fused_cast_matches_the_two_steps(be, large_tiles_only, a_dt, b_dt, m, n, k, hp, kmajor):
     """GEMM + in-time cast in one launch: payload, amax, scale and scale_inv must equal, bit for bit, what the GEMM
     into an hp buffer followed by the in-time cast of that buffer gives (the weight-gradient path of FP8Linear)."""
     a = _rand_fp8((m, k), a_dt, 3 * m + k).cuda()
@@ -427,6 +436,15 @@ def test_gemm_with_fused_cast_declines_what_it_cannot_take(be):
     for layout in (dict(), dict(a_kmajor=True, b_kmajor=True)):
         got, *_ = call(256, 256, 256, **layout)
         assert got is not None
+    # small enough for the 128 x 128 tiles (K of four slices and more, few large tiles): the two steps are faster
+    assert call(512, 256, 640) == (None, 2.0, 3.0, 5.0)
+    assert call(2048, 2048, 1024, a_kmajor=True, b_kmajor=True) == (None, 2.0, 3.0, 5.0)
+    try:
+        be.set_small_tile_limit(0)
+        got, *_ = call(512, 256, 640)
+        assert got is not None
+    finally:
+        be.set_small_tile_limit(128)
 
 
 def _spec_case(be, a, a_dt, sa, b, b_dt, sb, hp, kmajor, meta, old=None):
@@ -453,7 +471,7 @@ def _spec_case(be, a, a_dt, sa, b, b_dt, sb, hp, kmajor, meta, old=None):
 @pytest.mark.parametrize('m,n,k', [(4352, 4096, 256), (4096, 11008, 384), (8192, 28672, 256), (512, 256, 640)])
 @pytest.mark.parametrize('hp', [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize('kmajor', [True, False])
-def test_gemm_with_speculative_cast_matches_the_two_steps(be, a_dt, b_dt, m, n, k, hp, kmajor):
+def test_gemm_with_speculative_cast_matches_the_two_steps(be, large_tiles_only, a_dt, b_dt, m, n, k, hp, kmajor):
     """More output tiles than compute units (272, 688 and 3584 tiles; the small case is sent the same way by keeping
     the waiting kernels off): the GEMM stores the product and, beside it, the codes for the scale the meta holds.  A
     fresh meta (scale 1: the rule moves it, the product is cast again), the same operands again (the scale stands:
@@ -531,7 +549,7 @@ def test_gemm_with_speculative_cast_replays_from_a_graph(be):
         assert same_float(am, am0) and same_float(s, s0) and same_float(si, si0), factor
 
 
-def test_fp8linear_weight_gradient_uses_the_fused_kernel_and_matches():
+def test_fp8linear_weight_gradient_uses_the_fused_kernel_and_matches(be, large_tiles_only):
     """FP8Linear backward: the weight gradient from the fused launch equals the one from the two steps."""
     import msamp
     from msamp import _backend
@@ -569,7 +587,7 @@ def test_fp8linear_weight_gradient_uses_the_fused_kernel_and_matches():
     assert torch.equal(q1, q0) and same_float(s1, s0) and same_float(si1, si0) and same_float(am1, am0)
 
 
-def test_gemm_with_fused_cast_many_random_cases(be):
+def test_gemm_with_fused_cast_many_random_cases(be, large_tiles_only):
     """A sweep over seeds, scales, layouts and output types, with few tiles (where the unfused row-major GEMM runs the
     generic kernel) and many: every case equal to the two steps, to the bit."""
     cases = 0
