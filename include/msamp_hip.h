@@ -409,6 +409,17 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
  * leaves them at zero).  `workspace`: the MSAMP_WORKSPACE_BYTES buffer of the other entry points; a wait that
  * runs out (msamp_set_spin_limit) or a layout that breaks the rule above sets its sticky error word, reported by
  * msamp_check_async_error: the state is then partly updated and must be restored from a copy. */
+/* The same step (adamw.py:148-199: stage 1, the scale rule on the two amaxs, stage 2) for parameters kept in high
+ * precision -- biases, norm weights: a plain F32 / F16 / BF16 parameter and gradient, exp_avg in E4M3, exp_avg_sq in scaled
+ * F16 -- for n_tensors of them in one launch, one workgroup per parameter, with nothing read back by the host (the
+ * reference takes a dozen launches and two host round trips per parameter).  Uses the weight (the parameter, updated in
+ * place in param_dtype), grad (grad_dtype, passed through the uint8_t pointer), exp_avg, exp_avg_sq, m_* and v_* fields
+ * of the descriptors; meant for small tensors (a workgroup walks its whole parameter twice).  Same bits as
+ * msamp_adamw_fp8_stage1 / _stage2 with the parameter rounded to its type in between. */
+int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, int param_dtype, int grad_dtype, double lr, double beta1,
+                            double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
+                            int maximize, int tensor_scale, msamp_stream_t stream);
+
 #define MSAMP_ADAMW_POST_WORDS 8
 #define MSAMP_ADAMW_SYNC_BYTES(n_tensors, n_blocks) ((size_t)(n_tensors) * MSAMP_ADAMW_POST_WORDS * 8 + (size_t)(n_blocks) * 136)
 int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, void* sync, int n_tensors, const int32_t* block_map,

@@ -1331,6 +1331,63 @@ static bool state_dt_ok(int dt) {
         default: { constexpr int VDT = MSAMP_DT_F32; __VA_ARGS__ } break;             \
     }
 
+// ---- the step for parameters kept in high precision ---------------------------------------------------------------
+// Biases, norm weights and the like: a plain float32 / float16 / bfloat16 parameter with a gradient of such a type,
+// exp_avg in E4M3 and exp_avg_sq in scaled float16.  The reference (and the per-tensor path here) takes them one by one
+// through stage 1, a look at the two amaxs on the host, and stage 2: a dozen launches and two round trips to the host
+// per parameter, for tensors of a few thousand elements.  Here one workgroup takes one parameter through both
+// stages: m', v', p' with the expressions of the stages, p' stored in the parameter's type, max |m'| and max |v'| over
+// the workgroup, the scale rule, and the moments again from the still untouched stored ones with the new scales
+// (Adam mode: without the L2 term, as stage 2 has it).  Uses the weight, grad, exp_avg, exp_avg_sq, m_* and v_* fields
+// of the descriptor.
+template <typename PT, typename GT, bool L2>
+__global__ __launch_bounds__(kAdamThreads) void plain_step_kernel(msamp_adamw_tensor* __restrict__ tensors, AdamConsts k) {
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    __shared__ float s_scales[2];
+    msamp_adamw_tensor& d = tensors[blockIdx.x];
+    const size_t n = d.numel;
+    PT* param = static_cast<PT*>(d.weight);
+    const GT* grad = reinterpret_cast<const GT*>(d.grad);
+    const float inv_m = 1.0f / *d.m_scale, inv_v = 1.0f / *d.v_scale;
+    float mxm = 0.0f, mxv = 0.0f;
+    for (size_t i = threadIdx.x; i < n; i += kAdamThreads) {
+#pragma clang fp contract(off)
+        float pj = Elem<PT>::load(param + i);
+        float gj = Elem<GT>::load(grad + i);
+        if (k.maximize) gj = -gj;
+        if constexpr (L2) {
+            gj = fmaf(k.wd, pj, gj);    // torch's add(other, alpha=) on the GPU, which the per-tensor path takes: one rounding
+        } else {
+            pj = pj * k.decay;
+        }
+        float m_new, v_new;
+        moments(dequant1<MSAMP_DT_E4M3>(d.exp_avg[i]), f16_bits_to_float(d.exp_avg_sq[i]), gj, inv_m, inv_v, k, m_new, v_new);
+        mxm = fmaxf(mxm, fabsf(m_new));
+        mxv = fmaxf(mxv, fabsf(v_new));
+        Elem<PT>::store(param + i, param_update(pj, m_new, v_new, k));
+    }
+    const uint32_t a = block_max_u32(__float_as_uint(mxm), red);
+    const uint32_t b = block_max_u32(__float_as_uint(mxv), red);
+    if (threadIdx.x == 0) {
+        const float am = __uint_as_float(a), av = __uint_as_float(b);
+        const float ms = k.rule_scales ? scale_rule(am, 1.0f, 448.0f, 0) : 1.0f;
+        const float vs = k.rule_scales ? scale_rule(av, 1.0f, 65504.0f, 0) : 1.0f;
+        s_scales[0] = ms, s_scales[1] = vs;
+        *d.m_scale = ms, *d.m_scale_inv = 1.0f / ms, *d.m_amax = am;
+        *d.v_scale = vs, *d.v_scale_inv = 1.0f / vs, *d.v_amax = av;
+    }
+    __syncthreads();
+    const float ms = s_scales[0], vs = s_scales[1];
+    for (size_t i = threadIdx.x; i < n; i += kAdamThreads) {
+        float gj = Elem<GT>::load(grad + i);
+        if (k.maximize) gj = -gj;
+        float m_new, v_new;
+        moments(dequant1<MSAMP_DT_E4M3>(d.exp_avg[i]), f16_bits_to_float(d.exp_avg_sq[i]), gj, inv_m, inv_v, k, m_new, v_new);
+        d.exp_avg[i] = static_cast<uint8_t>(quant1<MSAMP_DT_E4M3>(m_new * ms));
+        d.exp_avg_sq[i] = static_cast<uint16_t>(float_to_f16_bits(v_new * vs));
+    }
+}
+
 }    // namespace msamp
 
 using namespace msamp;
@@ -1509,6 +1566,38 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
     MSAMP_CHECK_LAUNCH("fused_write_kernel");
     return MSAMP_OK;
 }
+int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, int param_dtype, int grad_dtype, double lr, double beta1,
+                            double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
+                            int maximize, int tensor_scale, msamp_stream_t stream) {
+    MSAMP_REQUIRE(n_tensors >= 0, MSAMP_ERR_SHAPE, "msamp_adamw_plain_fused: n_tensors=%d", n_tensors);
+    if (n_tensors == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(tensors, MSAMP_ERR_NULL, "msamp_adamw_plain_fused: null pointer");
+    MSAMP_REQUIRE(is_hp(param_dtype) && is_hp(grad_dtype), MSAMP_ERR_DTYPE, "msamp_adamw_plain_fused: dtypes %d, %d", param_dtype,
+                  grad_dtype);
+    AdamConsts k;
+    const bool l2 = fused_consts(lr, beta1, beta2, eps, weight_decay, step, bias_correction, adam_mode, maximize, k);
+    k.rule_scales = tensor_scale != 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define PLAIN_LAUNCH(PT, GT)                                                                                              \
+    do {                                                                                                                  \
+        if (l2) hipLaunchKernelGGL((plain_step_kernel<PT, GT, true>), dim3(n_tensors), dim3(kAdamThreads), 0, st, tensors, k); \
+        else hipLaunchKernelGGL((plain_step_kernel<PT, GT, false>), dim3(n_tensors), dim3(kAdamThreads), 0, st, tensors, k);   \
+    } while (0)
+#define PLAIN_GRAD(PT)                                                   \
+    do {                                                                 \
+        if (grad_dtype == MSAMP_DT_F32) PLAIN_LAUNCH(PT, float);         \
+        else if (grad_dtype == MSAMP_DT_F16) PLAIN_LAUNCH(PT, f16_t);    \
+        else PLAIN_LAUNCH(PT, bf16_t);                                   \
+    } while (0)
+    if (param_dtype == MSAMP_DT_F32) PLAIN_GRAD(float);
+    else if (param_dtype == MSAMP_DT_F16) PLAIN_GRAD(f16_t);
+    else PLAIN_GRAD(bf16_t);
+#undef PLAIN_GRAD
+#undef PLAIN_LAUNCH
+    MSAMP_CHECK_LAUNCH("plain_step_kernel");
+    return MSAMP_OK;
+}
+
 int msamp_adamw_fp8_fused_shift(msamp_adamw_tensor* tensors, int32_t* redo, void* sync, int n_tensors, const int32_t* block_map,
                                 int n_blocks, long long shift_elems, int weight_dtype, int grad_dtype, double lr, double beta1,
                                 double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,

@@ -62,6 +62,7 @@ _SIGNATURES = {
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_adamw_plain_fused': ([_vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
     'msamp_adamw_fp8_fused_shift': ([_vp, _vp, _vp, _i, _vp, _i, ctypes.c_longlong, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _vp], _i),
     'msamp_adamw_fp8_fused_speculative': ([_vp, _vp, _vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
 }
@@ -736,6 +737,28 @@ def adamw_fused(desc, n_tensors, block_map, n_blocks, weight_dt, grad_dt, lr, be
             step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0, 1 if tensor_scale else 0,
             ctypes.cast(bpt, ctypes.c_void_p) if bpt is not None else None, gb if bpt is not None else 0, _stream()
         ), 'msamp_adamw_fp8_fused'
+    )
+
+
+def hp_dt(tensor):
+    """Library code of a float32 / float16 / bfloat16 tensor's element type."""
+    return _dt(tensor)
+
+
+def adamw_plain_fused(desc, n_tensors, param_dt, grad_dt, lr, beta1, beta2, eps, weight_decay, step, bias_correction,
+                      adam_mode, maximize, tensor_scale):
+    """Both stages of the step for n_tensors small high-precision parameters with E4M3 / scaled-fp16 moments, one launch.
+    `desc`: int64 device tensor [n_tensors, ADAMW_DESC_WORDS] with the parameter, gradient, moment payloads, moment metas
+    and numel columns filled in."""
+    lib = load()
+    _gpu(desc, 'descriptor table')
+    if desc.dtype != torch.int64 or desc.numel() != n_tensors * ADAMW_DESC_WORDS or not desc.is_contiguous():
+        raise ValueError('desc must be a contiguous int64 tensor of n_tensors x %d words' % ADAMW_DESC_WORDS)
+    _check(
+        lib.msamp_adamw_plain_fused(
+            _ptr(desc), n_tensors, param_dt, grad_dt, lr, beta1, beta2, eps, weight_decay, step, 1 if bias_correction else 0,
+            1 if adam_mode else 0, 1 if maximize else 0, 1 if tensor_scale else 0, _stream()
+        ), 'msamp_adamw_plain_fused'
     )
 
 

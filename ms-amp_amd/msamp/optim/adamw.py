@@ -1,8 +1,9 @@
 """LBAdamW: the FP8 AdamW step on HIP kernels (msamp/optim/adamw.py:19-235).
 
 Quantized-state parameters whose weight, gradient and both moments are ScalingTensors of the
-supported formats take one fused multi-tensor call (three launches for the whole group); everything
-else follows the reference's two-stage recipe tensor by tensor.
+supported formats take one fused multi-tensor call (three launches for the whole group); small parameters
+kept in high precision (biases, norm weights) with quantized moments take one launch for all of them;
+everything else follows the reference's two-stage recipe tensor by tensor.
 """
 
 import math
@@ -310,6 +311,67 @@ class LBAdamW(LBAdamWBase):
             v.value.data = trio[2]
         return True
 
+    # ---- parameters kept in high precision: one launch for all of them ---------------------
+    _PLAIN_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+    _PLAIN_LIMIT = 1 << 16    # elements; one workgroup walks a whole parameter, so only biases, norm weights and the like
+
+    @classmethod
+    def _plain_fusable(cls, p, g, m, v):
+        if isinstance(p, ScalingTensor) or isinstance(g, ScalingTensor) or not torch.is_tensor(p) or not torch.is_tensor(g):
+            return False
+        if not (isinstance(m, ScalingTensor) and isinstance(v, ScalingTensor)):
+            return False
+        if p.dtype not in cls._PLAIN_DTYPES or g.dtype not in cls._PLAIN_DTYPES:
+            return False
+        if m.qtype != Dtypes.kfloat8_e4m3 or v.qtype != Dtypes.kfloat16 or v.value.dtype != torch.float16:
+            return False
+        if not 0 < p.numel() <= cls._PLAIN_LIMIT or m.meta.amax.numel() != 1 or v.meta.amax.numel() != 1:
+            return False
+        tensors = (p, g, m.value, v.value)
+        return all(t.is_cuda and t.is_contiguous() and t.numel() == p.numel() for t in tensors)
+
+    def _plain_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, step, *, beta1, beta2, lr, weight_decay, eps, maximize):
+        """Both stages of the reference recipe (msamp/optim/adamw.py:148-199) for all plain parameters of one type in
+        one launch, nothing read back by the host."""
+        ps, gs = [params[i] for i in idx], [grads[i] for i in idx]
+        ms, vs = [exp_avgs[i] for i in idx], [exp_avg_sqs[i] for i in idx]
+        if any(not g.is_contiguous() or g.numel() != p.numel() for p, g in zip(ps, gs)):
+            self._groups = None    # (the grouping is kept from an earlier step) this step tensor by tensor
+            self._staged_step(idx, params, grads, exp_avgs, exp_avg_sqs, [step] * len(params), beta1=beta1, beta2=beta2, lr=lr,
+                              weight_decay=weight_decay, eps=eps, maximize=maximize)
+            return
+        key = ('plain', ps[0].dtype, gs[0].dtype, id(ps[0]))
+        plan = self._plans.get(key)
+        ids = tuple(id(p) for p in ps)
+        if plan is None or plan.params != ids:
+            plan = _FusedPlan()
+            plan.params = ids
+            self._plans[key] = plan
+        static = [id(t) for m, v in zip(ms, vs) for t in (m.meta.scale, m.meta.scale_inv, m.meta.amax, v.meta.scale,
+                                                           v.meta.scale_inv, v.meta.amax)]
+        sig = ([p.data_ptr() for p in ps], [g.data_ptr() for g in gs], [m.value.data_ptr() for m in ms],
+               [v.value.data_ptr() for v in vs])
+        if plan.desc is None or plan.static_sig != static:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError('LBAdamW: the first step of a parameter group builds device tables and cannot be captured; '
+                                   'take a step outside the capture first.')
+            rows = np.zeros((len(ps), _backend.ADAMW_DESC_WORDS), dtype=np.int64)
+            for col, values in enumerate(sig):
+                rows[:, col] = values
+            for r, (m, v) in enumerate(zip(ms, vs)):
+                rows[r, 8:14] = (m.meta.scale.data_ptr(), m.meta.scale_inv.data_ptr(), m.meta.amax.data_ptr(),
+                                 v.meta.scale.data_ptr(), v.meta.scale_inv.data_ptr(), v.meta.amax.data_ptr())
+                rows[r, 14] = ps[r].numel()
+            plan.desc = torch.from_numpy(rows).to(ps[0].device)
+            plan.static_sig, plan.sig = static, sig
+        elif plan.sig != sig:
+            for col, (values, before) in enumerate(zip(sig, plan.sig)):
+                if values != before:
+                    plan.desc[:, col] = torch.tensor(values, dtype=torch.int64).to(plan.desc.device)
+            plan.sig = sig
+        _backend.adamw_plain_fused(plan.desc, len(ps), _backend.hp_dt(ps[0]), _backend.hp_dt(gs[0]), lr, beta1, beta2, eps,
+                                   weight_decay, step, self.bias_correction, self.use_adam, maximize, self.tensor_scale)
+
     # ---- per-tensor path (reference recipe) -----------------------------------------------
     def _staged_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, state_steps, *, beta1, beta2, lr, weight_decay,
                      eps, maximize):
@@ -369,22 +431,26 @@ class LBAdamW(LBAdamWBase):
             # step counts (the look costs more host time than everything else in a step); what may change from step to
             # step without showing here -- where a gradient's payload lies -- is checked in _fused_step.
             key = (tuple(map(id, params)), tuple(map(id, exp_avgs)), tuple(map(id, exp_avg_sqs)),
-                   tuple(g.qtype if isinstance(g, ScalingTensor) else None for g in grads),
+                   tuple(g.qtype if isinstance(g, ScalingTensor) else g.dtype for g in grads),
                    tuple(n - state_steps[0] for n in state_steps), ScalingMeta.in_time_scaling)
             if self._groups is not None and self._groups[0] == key:
-                fused, staged = self._groups[1], self._groups[2]
+                fused, plain, staged = self._groups[1:]
             else:
-                fused = {}
+                fused, plain = {}, {}
                 staged = []
                 for i in range(len(params)):
                     if self._fusable(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i]):
                         fused.setdefault((int(params[i].qtype), int(grads[i].qtype), state_steps[i]), []).append(i)
+                    elif self._plain_fusable(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i]):
+                        plain.setdefault((params[i].dtype, grads[i].dtype, state_steps[i]), []).append(i)
                     else:
                         staged.append(i)
-                self._groups = (key, fused, staged)
+                self._groups = (key, fused, plain, staged)
             hyper = dict(beta1=beta1, beta2=beta2, lr=lr, weight_decay=weight_decay, eps=eps, maximize=maximize)
             for idx in fused.values():    # (one call per weight format, gradient format and step count)
                 self._fused_step(idx, params, grads, exp_avgs, exp_avg_sqs, state_steps[idx[0]], **hyper)
+            for idx in plain.values():    # (one call per parameter type, gradient type and step count)
+                self._plain_step(idx, params, grads, exp_avgs, exp_avg_sqs, state_steps[idx[0]], **hyper)
             self._staged_step(staged, params, grads, exp_avgs, exp_avg_sqs, state_steps, **hyper)
             return
         # float32 moments: whole-tensor float32 update, then requantize the parameter if it is low-bit

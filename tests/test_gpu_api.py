@@ -744,3 +744,76 @@ def test_empty_inputs_are_accepted_everywhere():
     # fused AdamW: no tensors at all
     be.adamw_fused(torch.zeros(0, be.ADAMW_DESC_WORDS, dtype=torch.int64, device=dev), 0,
                    torch.zeros(0, 2, dtype=torch.int32, device=dev), 0, 5, 6, 1e-3, 0.9, 0.95, 1e-8, 0.1, 1, True, False, False, True)
+
+
+@pytest.mark.parametrize('optimizer, kw', [
+    (LBAdamW, dict()),
+    (LBAdamW, dict(weight_decay=0.0, maximize=True)),
+    (LBAdamW, dict(tensor_scale=False, bias_correction=False)),
+    (LBAdam, dict(weight_decay=0.05)),
+])
+def test_small_plain_parameters_take_one_launch_with_the_bits_of_the_two_stages(monkeypatch, optimizer, kw):
+    """Parameters kept in float32 / float16 / bfloat16 with E4M3 and scaled-float16 moments (biases, norm weights) go
+    through both stages of the reference recipe (msamp/optim/adamw.py:148-199) in one launch for all of them: same
+    parameter, moment payloads and metas, bit for bit, as the two stages taken tensor by tensor, over several steps whose
+    gradients change size by orders of magnitude (so the moment scales move)."""
+    shapes = [(1, ), (70, ), (4099, ), (3, 1000), (LBAdamW._PLAIN_LIMIT, ), (LBAdamW._PLAIN_LIMIT + 1, )]
+    dtypes = [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+              (torch.float32, torch.bfloat16)]
+    runs = {}
+    for fused in (True, False):
+        gen = torch.Generator(device='cuda').manual_seed(31)
+        params = []
+        for p_dt, g_dt in dtypes:
+            for shape in shapes:
+                params.append((torch.nn.Parameter((torch.randn(shape, device='cuda', generator=gen) * 0.3).to(p_dt)), g_dt))
+                if g_dt != p_dt:
+                    params[-1][0].grad_dtype = g_dt
+        opt = optimizer([p for p, _ in params], lr=3e-3, **kw)
+        calls = []
+        if fused:
+            plain_step = LBAdamW._plain_step
+            monkeypatch.setattr(LBAdamW, '_plain_step', lambda self, idx, *a, **k: (calls.append(len(idx)), plain_step(self, idx, *a, **k)))
+        else:
+            monkeypatch.setattr(LBAdamW, '_plain_fusable', classmethod(lambda cls, *a: False))
+        history = []
+        for step, size in enumerate((1.0, 1e-3, 40.0, 1e-6, 0.0, 2.0)):
+            for p, g_dt in params:
+                p.grad = (torch.randn(p.shape, device='cuda', generator=gen) * size).to(g_dt)
+            opt.step()
+            history.append([(p.detach().clone(), ) + tuple(t.clone() for name in ('exp_avg', 'exp_avg_sq')
+                                                           for t in (opt.state[p][name].value, opt.state[p][name].meta.scale,
+                                                                     opt.state[p][name].meta.scale_inv, opt.state[p][name].meta.amax))
+                            for p, _ in params])
+        monkeypatch.undo()
+        if fused:
+            # one call per pair of types, each with all the shapes but the one over the limit
+            assert calls == [len(shapes) - 1] * len(dtypes) * 6
+        runs[fused] = history
+    for step, (a, b) in enumerate(zip(runs[True], runs[False])):
+        for t, (x, y) in enumerate(zip(a, b)):
+            for which, (u, v) in enumerate(zip(x, y)):
+                assert same_float(u, v) if u.is_floating_point() else torch.equal(u, v), (step, t, which)
+    # the moment scales did move
+    assert len({float(h[1][2]) for h in runs[True]}) > (2 if kw.get('tensor_scale', True) else 0)
+
+
+def test_plain_parameter_step_follows_gradients_that_move():
+    """The descriptor table of the one-launch step is kept from step to step; a gradient at a new address (grads set to
+    None between steps) is found again."""
+    torch.manual_seed(5)
+    p = torch.nn.Parameter(torch.randn(300, device='cuda'))
+    q = torch.nn.Parameter(p.detach().clone())
+    opt_p, opt_q = LBAdamW([p], lr=1e-2), LBAdamW([q], lr=1e-2)
+    keep = []
+    for step in range(4):
+        g = torch.randn(300, device='cuda')
+        keep.append(g)    # (held, so that the next gradient gets another address)
+        p.grad = g.clone()
+        if q.grad is None:
+            q.grad = torch.empty_like(g)
+        q.grad.copy_(g)
+        opt_p.step()
+        opt_q.step()
+        p.grad = None
+        assert torch.equal(p, q)
