@@ -543,6 +543,25 @@ def bench_adam(iters=10, total_params=1_000_000_000):
         out[name] = row
         del opt
         torch.cuda.empty_cache()
+    del params
+    torch.cuda.empty_cache()
+    # float32 moments (the reference's opt_level O1 keeps them so): 16 float32 parameters of 4096 x 4096 with float32
+    # gradients, stepped by the one-pass kernel and by the reference's chain of element-wise calls; 28 B/param (read p, g,
+    # m, v; write p, m, v)
+    plain = [torch.nn.Parameter(torch.randn(4096, 4096, device='cuda', generator=g) * 0.02) for _ in range(16)]
+    for p in plain:
+        p.grad = torch.randn(4096, 4096, device='cuda', generator=g) * 1e-3
+    n_plain = sum(p.numel() for p in plain)
+    opt = LBAdamW(plain, exp_avg_dtype=torch.float32, exp_avg_sq_dtype=torch.float32, **hyper)
+    row = {'params': n_plain, 'ms': _time_gpu(opt.step, iters, warm=3)}
+    kernel_step = LBAdamW._f32_step
+    LBAdamW._f32_step = lambda self, *a, **k: False
+    try:
+        row['ms_as_torch_calls'] = _time_gpu(opt.step, iters, warm=3)
+    finally:
+        LBAdamW._f32_step = kernel_step
+    row['hbm_frac'] = n_plain * 28 / (row['ms'] * 1e-3) / 8e12
+    out['float32_moments'] = row
     return out
 
 

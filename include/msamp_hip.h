@@ -409,6 +409,16 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
  * leaves them at zero).  `workspace`: the MSAMP_WORKSPACE_BYTES buffer of the other entry points; a wait that
  * runs out (msamp_set_spin_limit) or a layout that breaks the rule above sets its sticky error word, reported by
  * msamp_check_async_error: the state is then partly updated and must be restored from a copy. */
+/* The float32-moment branch of LBAdamW.adamw_fn (adamw.py:200-232) for one parameter in one pass: the reference runs it
+ * as about a dozen element-wise torch calls (its own one-pass kernel, adamw.cu:20-28 bound as adamw_compute :77-97, is
+ * never called from its Python).  `param`, `exp_avg`, `exp_avg_sq`: float32, updated in place; `grad`: F32 / F16 / BF16.
+ * Every intermediate is rounded where the torch chain rounds it on the GPU (add with alpha = one fused multiply-add,
+ * division by the Python number sqrt(bias_correction2) = multiplication by its narrowed reciprocal), so the results are
+ * the chain's, bit for bit.  adam_mode: weight decay as an L2 term on the gradient instead of a decay of the weight. */
+int msamp_adamw_f32(float* param, const void* grad, int grad_dtype, size_t n, float* exp_avg, float* exp_avg_sq, double lr,
+                    double beta1, double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
+                    int maximize, msamp_stream_t stream);
+
 /* The same step (adamw.py:148-199: stage 1, the scale rule on the two amaxs, stage 2) for parameters kept in high
  * precision -- biases, norm weights: a plain F32 / F16 / BF16 parameter and gradient, exp_avg in E4M3, exp_avg_sq in scaled
  * F16 -- for n_tensors of them in one launch, one workgroup per parameter, with nothing read back by the host (the

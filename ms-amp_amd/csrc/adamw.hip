@@ -1388,6 +1388,81 @@ __global__ __launch_bounds__(kAdamThreads) void plain_step_kernel(msamp_adamw_te
     }
 }
 
+// ---- float32 moments ------------------------------------------------------------------------------------------------
+// The branch of LBAdamW.adamw_fn for float32 exp_avg / exp_avg_sq (msamp/optim/adamw.py:200-232) is a chain of a dozen
+// element-wise torch calls per parameter; this kernel is that chain in one pass, with every intermediate rounded where
+// the chain rounds it on the GPU: a.add(b, alpha=c) is one fused multiply-add, a division by a Python number is a
+// multiplication by its reciprocal (taken in double, then narrowed), everything else rounds per operation.
+// (adamw.cu:20-28, the kernel the reference binds as adamw_compute but never calls, divides by sqrt(bc2) instead.)
+struct F32Consts {
+    float beta1, omb1, beta2, omb2, inv_sbc2, eps, neg_step, wd, decay;
+    int maximize;
+};
+
+template <bool L2>
+__device__ __forceinline__ void f32_element(float& p, float g, float& m, float& v, const F32Consts& k) {
+#pragma clang fp contract(off)
+    if (k.maximize) g = -g;
+    if constexpr (L2) g = fmaf(k.wd, p, g);
+    else p = p * k.decay;    // (1 when there is no decay)
+    const float m_scaled = k.beta1 * m;
+    m = fmaf(k.omb1, g, m_scaled);
+    const float v_scaled = k.beta2 * v;
+    const float gg = g * g;
+    v = fmaf(k.omb2, gg, v_scaled);
+    const float root = sqrtf(v);
+    const float q = root * k.inv_sbc2;
+    const float denom = q + k.eps;
+    const float r = m / denom;
+    p = fmaf(k.neg_step, r, p);
+}
+
+template <typename GT>
+__device__ __forceinline__ void load_grad4(const GT* g, float* f) {
+    if constexpr (sizeof(GT) == 4) {
+        const float4 t = *reinterpret_cast<const float4*>(g);
+        f[0] = t.x, f[1] = t.y, f[2] = t.z, f[3] = t.w;
+    } else {
+        const uint2 t = *reinterpret_cast<const uint2*>(g);
+        const GT* h = reinterpret_cast<const GT*>(&t);
+        for (int j = 0; j < 4; ++j) f[j] = Elem<GT>::load(h + j);
+    }
+}
+
+// VEC: every pointer is aligned for four elements
+template <typename GT, bool L2, bool VEC>
+__global__ __launch_bounds__(kAdamThreads) void f32_step_kernel(float* __restrict__ param, const GT* __restrict__ grad,
+                                                                 float* __restrict__ exp_avg, float* __restrict__ exp_avg_sq,
+                                                                 size_t n, F32Consts k) {
+    const size_t tid = static_cast<size_t>(blockIdx.x) * kAdamThreads + threadIdx.x;
+    const size_t threads = static_cast<size_t>(gridDim.x) * kAdamThreads;
+    size_t done = 0;
+    if constexpr (VEC) {
+        const size_t quads = n / 4;
+        for (size_t q = tid; q < quads; q += threads) {
+            const size_t i = q * 4;
+            float4 p4 = *reinterpret_cast<const float4*>(param + i);
+            float4 m4 = *reinterpret_cast<const float4*>(exp_avg + i);
+            float4 v4 = *reinterpret_cast<const float4*>(exp_avg_sq + i);
+            float g[4];
+            load_grad4<GT>(grad + i, g);
+            f32_element<L2>(p4.x, g[0], m4.x, v4.x, k);
+            f32_element<L2>(p4.y, g[1], m4.y, v4.y, k);
+            f32_element<L2>(p4.z, g[2], m4.z, v4.z, k);
+            f32_element<L2>(p4.w, g[3], m4.w, v4.w, k);
+            *reinterpret_cast<float4*>(param + i) = p4;
+            *reinterpret_cast<float4*>(exp_avg + i) = m4;
+            *reinterpret_cast<float4*>(exp_avg_sq + i) = v4;
+        }
+        done = quads * 4;
+    }
+    for (size_t i = done + tid; i < n; i += threads) {
+        float p = param[i], m = exp_avg[i], v = exp_avg_sq[i];
+        f32_element<L2>(p, Elem<GT>::load(grad + i), m, v, k);
+        param[i] = p, exp_avg[i] = m, exp_avg_sq[i] = v;
+    }
+}
+
 }    // namespace msamp
 
 using namespace msamp;
@@ -1566,6 +1641,50 @@ int msamp_adamw_fp8_fused_speculative(msamp_adamw_tensor* tensors, const msamp_a
     MSAMP_CHECK_LAUNCH("fused_write_kernel");
     return MSAMP_OK;
 }
+int msamp_adamw_f32(float* param, const void* grad, int grad_dtype, size_t n, float* exp_avg, float* exp_avg_sq, double lr,
+                    double beta1, double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
+                    int maximize, msamp_stream_t stream) {
+    if (n == 0) return MSAMP_OK;
+    MSAMP_REQUIRE(param && grad && exp_avg && exp_avg_sq, MSAMP_ERR_NULL, "msamp_adamw_f32: null pointer");
+    MSAMP_REQUIRE(is_hp(grad_dtype), MSAMP_ERR_DTYPE, "msamp_adamw_f32: grad dtype %d", grad_dtype);
+    // the Python numbers of the chain, each narrowed where torch narrows it (to the tensors' float32)
+    const double bc1 = bias_correction ? 1.0 - pow(beta1, step) : 1.0;
+    const double bc2 = bias_correction ? 1.0 - pow(beta2, step) : 1.0;
+    F32Consts k;
+    k.beta1 = static_cast<float>(beta1), k.omb1 = static_cast<float>(1.0 - beta1);
+    k.beta2 = static_cast<float>(beta2), k.omb2 = static_cast<float>(1.0 - beta2);
+    k.inv_sbc2 = static_cast<float>(1.0 / sqrt(bc2));
+    k.eps = static_cast<float>(eps);
+    k.neg_step = static_cast<float>(-(lr / bc1));
+    k.wd = static_cast<float>(weight_decay);
+    const bool l2 = weight_decay != 0.0 && adam_mode;
+    k.decay = (weight_decay != 0.0 && !adam_mode) ? static_cast<float>(1.0 - lr * weight_decay) : 1.0f;
+    k.maximize = maximize;
+    const size_t grad_bytes = grad_dtype == MSAMP_DT_F32 ? 4 : 2;
+    const bool vec = (reinterpret_cast<uintptr_t>(param) | reinterpret_cast<uintptr_t>(exp_avg) |
+                      reinterpret_cast<uintptr_t>(exp_avg_sq)) % 16 == 0 && reinterpret_cast<uintptr_t>(grad) % (4 * grad_bytes) == 0;
+    const size_t per_group = static_cast<size_t>(kAdamThreads) * 4;
+    const int grid = static_cast<int>(std::min<size_t>((n + per_group - 1) / per_group, static_cast<size_t>(cu_count()) * 16));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define F32_LAUNCH(GT, L2V, VECV)                                                                                          \
+    hipLaunchKernelGGL((f32_step_kernel<GT, L2V, VECV>), dim3(grid), dim3(kAdamThreads), 0, st, param, static_cast<const GT*>(grad), \
+                       exp_avg, exp_avg_sq, n, k)
+#define F32_FORMS(GT)                                 \
+    do {                                              \
+        if (l2 && vec) F32_LAUNCH(GT, true, true);    \
+        else if (l2) F32_LAUNCH(GT, true, false);     \
+        else if (vec) F32_LAUNCH(GT, false, true);    \
+        else F32_LAUNCH(GT, false, false);            \
+    } while (0)
+    if (grad_dtype == MSAMP_DT_F32) F32_FORMS(float);
+    else if (grad_dtype == MSAMP_DT_F16) F32_FORMS(f16_t);
+    else F32_FORMS(bf16_t);
+#undef F32_FORMS
+#undef F32_LAUNCH
+    MSAMP_CHECK_LAUNCH("f32_step_kernel");
+    return MSAMP_OK;
+}
+
 int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, int param_dtype, int grad_dtype, double lr, double beta1,
                             double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
                             int maximize, int tensor_scale, msamp_stream_t stream) {

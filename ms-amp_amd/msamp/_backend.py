@@ -62,6 +62,7 @@ _SIGNATURES = {
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_adamw_f32': ([_vp, _vp, _i, _sz, _vp, _vp, _d, _d, _d, _d, _d, _i, _i, _i, _i, _vp], _i),
     'msamp_adamw_plain_fused': ([_vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
     'msamp_adamw_fp8_fused_shift': ([_vp, _vp, _vp, _i, _vp, _i, ctypes.c_longlong, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _vp], _i),
     'msamp_adamw_fp8_fused_speculative': ([_vp, _vp, _vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
@@ -743,6 +744,25 @@ def adamw_fused(desc, n_tensors, block_map, n_blocks, weight_dt, grad_dt, lr, be
 def hp_dt(tensor):
     """Library code of a float32 / float16 / bfloat16 tensor's element type."""
     return _dt(tensor)
+
+
+def adamw_f32(param, grad, exp_avg, exp_avg_sq, lr, beta1, beta2, eps, weight_decay, step, bias_correction, adam_mode,
+              maximize):
+    """One AdamW / Adam step of a float32 parameter with float32 moments, in place, in one pass; `grad` may be float32,
+    float16 or bfloat16."""
+    lib = load()
+    for t, what in ((param, 'param'), (grad, 'grad'), (exp_avg, 'exp_avg'), (exp_avg_sq, 'exp_avg_sq')):
+        _gpu(t, what)
+        if not t.is_contiguous() or t.numel() != param.numel():
+            raise ValueError(f'adamw_f32: {what} must be contiguous and of the parameter\'s size')
+    if any(t.dtype != torch.float32 for t in (param, exp_avg, exp_avg_sq)):
+        raise TypeError('adamw_f32: param, exp_avg and exp_avg_sq must be float32')
+    _check(
+        lib.msamp_adamw_f32(
+            _ptr(param), _ptr(grad), _dt(grad), param.numel(), _ptr(exp_avg), _ptr(exp_avg_sq), lr, beta1, beta2, eps,
+            weight_decay, step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0, _stream()
+        ), 'msamp_adamw_f32'
+    )
 
 
 def adamw_plain_fused(desc, n_tensors, param_dt, grad_dt, lr, beta1, beta2, eps, weight_decay, step, bias_correction,

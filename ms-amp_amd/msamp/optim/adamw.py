@@ -372,6 +372,27 @@ class LBAdamW(LBAdamWBase):
         _backend.adamw_plain_fused(plan.desc, len(ps), _backend.hp_dt(ps[0]), _backend.hp_dt(gs[0]), lr, beta1, beta2, eps,
                                    weight_decay, step, self.bias_correction, self.use_adam, maximize, self.tensor_scale)
 
+    # ---- float32 moments ---------------------------------------------------------------------
+    def _f32_step(self, p, g, exp_avg, exp_avg_sq, step, *, beta1, beta2, lr, weight_decay, eps, maximize):
+        """The chain of element-wise calls of the reference's float32 branch (msamp/optim/adamw.py:200-232) as one kernel,
+        same bits; False where the kernel does not apply (the chain below then runs as written)."""
+        moments = (exp_avg, exp_avg_sq)
+        if any(isinstance(t, ScalingTensor) or t.dtype != torch.float32 or not t.is_cuda or not t.is_contiguous()
+               for t in moments):
+            return False
+        param = p.float()
+        grad = g.float() if isinstance(g, ScalingTensor) or g.dtype not in self._PLAIN_DTYPES else g
+        if not (param.is_cuda and grad.is_cuda) or any(t.numel() != param.numel() for t in (grad, ) + moments):
+            return False
+        param, grad = param.contiguous(), grad.contiguous()
+        _backend.adamw_f32(param, grad, exp_avg, exp_avg_sq, lr, beta1, beta2, eps, weight_decay, step, self.bias_correction,
+                           self.use_adam, maximize)
+        if isinstance(p, ScalingTensor):
+            p.copy_(param.cast(p.qtype, meta=p.meta))
+        elif param.data_ptr() != p.data_ptr():
+            p.copy_(param)
+        return True
+
     # ---- per-tensor path (reference recipe) -----------------------------------------------
     def _staged_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, state_steps, *, beta1, beta2, lr, weight_decay,
                      eps, maximize):
@@ -455,6 +476,9 @@ class LBAdamW(LBAdamWBase):
             return
         # float32 moments: whole-tensor float32 update, then requantize the parameter if it is low-bit
         for i, p in enumerate(params):
+            if self._f32_step(p, grads[i], exp_avgs[i], exp_avg_sqs[i], state_steps[i], beta1=beta1, beta2=beta2, lr=lr,
+                              weight_decay=weight_decay, eps=eps, maximize=maximize):
+                continue
             param = p.float()
             grad = grads[i].float() if not maximize else -grads[i].float()
             exp_avg, exp_avg_sq = exp_avgs[i], exp_avg_sqs[i]

@@ -817,3 +817,57 @@ def test_plain_parameter_step_follows_gradients_that_move():
         opt_q.step()
         p.grad = None
         assert torch.equal(p, q)
+
+
+@pytest.mark.parametrize('optimizer, kw', [
+    (LBAdamW, dict()),
+    (LBAdamW, dict(weight_decay=0.0, maximize=True)),
+    (LBAdamW, dict(bias_correction=False, betas=(0.8, 0.95), eps=1e-6)),
+    (LBAdam, dict(weight_decay=0.05)),
+])
+def test_float32_moment_step_in_one_kernel_has_the_bits_of_the_chain(monkeypatch, optimizer, kw):
+    """With float32 exp_avg / exp_avg_sq the reference's step is a chain of element-wise torch calls
+    (msamp/optim/adamw.py:200-232); the one-pass kernel that stands in for it leaves the same parameter and moments, bit
+    for bit, over several steps: float32 / bfloat16 / float16 parameters, gradients of another type, a parameter that
+    is a misaligned view (no vector loads), and a scaled-float16 ScalingTensor weight that is requantized after the step."""
+    shapes = [(1, ), (70, ), (4099, ), (1 << 20, ), (3, 349_527)]
+    dtypes = [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+              (torch.float32, torch.bfloat16)]
+    runs = {}
+    for fused in (True, False):
+        gen = torch.Generator(device='cuda').manual_seed(77)
+        params = []
+        for p_dt, g_dt in dtypes:
+            for shape in shapes:
+                params.append((torch.nn.Parameter((torch.randn(shape, device='cuda', generator=gen) * 0.3).to(p_dt)), g_dt))
+                if g_dt != p_dt:
+                    params[-1][0].grad_dtype = g_dt
+        base = torch.randn(5001, device='cuda', generator=gen)
+        params.append((torch.nn.Parameter(base[1:]), torch.float32))    # 4 bytes past a 16-byte boundary
+        weight = torch.nn.Parameter(torch.randn(64, 48, device='cuda', generator=gen) * 0.05)
+        scaled = ScalingParameter(weight.detach().cast(Dtypes.kfloat16))
+        opt = optimizer([p for p, _ in params] + [scaled], lr=3e-3, exp_avg_dtype=torch.float32, exp_avg_sq_dtype=torch.float32,
+                        **kw)
+        calls = []
+        f32_step = LBAdamW._f32_step
+        if fused:
+            monkeypatch.setattr(LBAdamW, '_f32_step', lambda self, *a, **k: (calls.append(1), f32_step(self, *a, **k))[1])
+        else:
+            monkeypatch.setattr(LBAdamW, '_f32_step', lambda self, *a, **k: False)
+        history = []
+        for step, size in enumerate((1.0, 1e-3, 40.0, 0.0, 2.0)):
+            for p, g_dt in params:
+                p.grad = (torch.randn(p.shape, device='cuda', generator=gen) * size).to(g_dt)
+            scaled.grad = (torch.randn(64, 48, device='cuda', generator=gen) * size).cast(Dtypes.kfloat8_e4m3)
+            opt.step()
+            history.append([(p.detach().clone(), opt.state[p]['exp_avg'].clone(), opt.state[p]['exp_avg_sq'].clone())
+                            for p, _ in params] +
+                           [(scaled.value.clone(), scaled.meta.scale.clone(), opt.state[scaled]['exp_avg'].clone(),
+                             opt.state[scaled]['exp_avg_sq'].clone())])
+        monkeypatch.undo()
+        assert len(calls) == (5 * (len(params) + 1) if fused else 0)
+        runs[fused] = history
+    for step, (a, b) in enumerate(zip(runs[True], runs[False])):
+        for t, (x, y) in enumerate(zip(a, b)):
+            for which, (u, v) in enumerate(zip(x, y)):
+                assert same_float(u, v), (step, t, which, (u.float() - v.float()).abs().max().item())
