@@ -562,6 +562,34 @@ def bench_adam(iters=10, total_params=1_000_000_000):
         LBAdamW._f32_step = kernel_step
     row['hbm_frac'] = n_plain * 28 / (row['ms'] * 1e-3) / 8e12
     out['float32_moments'] = row
+    del opt, plain
+    # what a model keeps in high precision beside its FP8 weights: 64 bfloat16 vectors of 4096 .. 11008 elements with E4M3 /
+    # scaled-float16 moments.  One launch for all of them against the reference's recipe tensor by tensor (two stages and
+    # two reads of the amaxs by the host per tensor); wall time, since the recipe is bound by the host
+    small = [torch.nn.Parameter(torch.randn(4096 if i % 2 else 11008, device='cuda', generator=g).bfloat16()) for i in range(64)]
+    for p in small:
+        p.grad = (torch.randn(p.shape, device='cuda', generator=g) * 1e-3).bfloat16()
+    opt = LBAdamW(small, **hyper)
+
+    def wall_ms(n=20):
+        for _ in range(3):
+            opt.step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            opt.step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    row = {'tensors': len(small), 'wall_ms': wall_ms()}
+    fusable = LBAdamW._plain_fusable
+    LBAdamW._plain_fusable = classmethod(lambda cls, *a: False)
+    opt._groups = None
+    try:
+        row['wall_ms_tensor_by_tensor'] = wall_ms()
+    finally:
+        LBAdamW._plain_fusable = fusable
+    out['small_plain_parameters'] = row
     return out
 
 
