@@ -362,12 +362,21 @@ class LBAdamW(LBAdamWBase):
                 rows[r, 8:14] = (m.meta.scale.data_ptr(), m.meta.scale_inv.data_ptr(), m.meta.amax.data_ptr(),
                                  v.meta.scale.data_ptr(), v.meta.scale_inv.data_ptr(), v.meta.amax.data_ptr())
                 rows[r, 14] = ps[r].numel()
-            plan.desc = torch.from_numpy(rows).to(ps[0].device)
+            # a pinned copy of the rows stays with the table: what a captured step sends its new addresses through
+            plan.stage = torch.from_numpy(rows).pin_memory()
+            plan.desc = plan.stage.to(ps[0].device)
             plan.static_sig, plan.sig = static, sig
         elif plan.sig != sig:
-            for col, (values, before) in enumerate(zip(sig, plan.sig)):
-                if values != before:
-                    plan.desc[:, col] = torch.tensor(values, dtype=torch.int64).to(plan.desc.device)
+            if torch.cuda.is_current_stream_capturing():
+                # (gradients made under capture come from the graph's own memory) the whole table again, from pinned
+                # memory: one copy that the graph can hold
+                for col, values in enumerate(sig):
+                    plan.stage[:, col] = torch.tensor(values, dtype=torch.int64)
+                plan.desc.copy_(plan.stage, non_blocking=True)
+            else:
+                for col, (values, before) in enumerate(zip(sig, plan.sig)):
+                    if values != before:
+                        plan.desc[:, col] = torch.tensor(values, dtype=torch.int64).to(plan.desc.device)
             plan.sig = sig
         _backend.adamw_plain_fused(plan.desc, len(ps), _backend.hp_dt(ps[0]), _backend.hp_dt(gs[0]), lr, beta1, beta2, eps,
                                    weight_decay, step, self.bias_correction, self.use_adam, maximize, self.tensor_scale)

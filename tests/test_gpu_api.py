@@ -436,12 +436,14 @@ def test_captured_forward_and_backward_see_the_weights_of_eager_steps():
         assert torch.equal(model.weight.value, want[i][1]), i
 
 
-def test_optimizer_step_under_capture_after_an_eager_step():
+@pytest.mark.parametrize('bias', [False, True])
+def test_optimizer_step_under_capture_after_an_eager_step(bias):
     """A fused step can be captured once an eager step has built the device tables: the gradients made under capture live
     elsewhere, their addresses reach the table through a pinned copy that the graph holds.  (Bias correction is
-    computed on the host from the step count, so a captured step repeats the one it was captured with: off here.)"""
+    computed on the host from the step count, so a captured step repeats the one it was captured with: off here.)
+    With a bias the step has a second launch, the one for parameters kept in high precision, with a table of its own."""
     torch.manual_seed(16)
-    lin = torch.nn.Linear(128, 256, bias=False).cuda().bfloat16()
+    lin = torch.nn.Linear(128, 256, bias=bias).cuda().bfloat16()
     xs = [torch.randn(256, 128, device='cuda').bfloat16() * (1 + i % 3) for i in range(5)]
     dy = (torch.randn(256, 256, device='cuda') * 1e-2).bfloat16()
 
@@ -457,7 +459,8 @@ def test_optimizer_step_under_capture_after_an_eager_step():
         opt.all_reduce_grads(model)
         opt.step()
         opt.zero_grad()
-        want.append((model.weight.value.clone(), opt.state[model.weight]['exp_avg'].value.clone()))
+        want.append((model.weight.value.clone(), opt.state[model.weight]['exp_avg'].value.clone(),
+                     model.bias.detach().clone() if bias else None))
     model, opt = build()
     x = xs[0].clone()
     side = torch.cuda.Stream()
@@ -467,6 +470,8 @@ def test_optimizer_step_under_capture_after_an_eager_step():
         opt.all_reduce_grads(model)
         opt.step()
         model.weight.grad = None
+        if bias:
+            model.bias.grad = None
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     assert torch.equal(model.weight.value, want[0][0])
@@ -476,12 +481,15 @@ def test_optimizer_step_under_capture_after_an_eager_step():
         model_state.ready_to_scale_tensor = True
         opt.step()
         model.weight.grad = None
+        if bias:
+            model.bias.grad = None
     for i in range(1, len(xs)):
         x.copy_(xs[i])
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(model.weight.value, want[i][0]), i
         assert torch.equal(opt.state[model.weight]['exp_avg'].value, want[i][1]), i
+        assert not bias or torch.equal(model.bias, want[i][2]), i
         assert torch.isfinite(xs[i].float().sum()).item()    # eager work between replays
 
 
