@@ -590,6 +590,21 @@ def bench_adam(iters=10, total_params=1_000_000_000):
     finally:
         LBAdamW._plain_fusable = fusable
     out['small_plain_parameters'] = row
+    del opt, small
+    # an embedding kept in bfloat16 (32000 x 4096) with E4M3 / scaled-float16 moments: the same step chunk by chunk in
+    # three launches (19 B/param: read p, g, m, v, write p; read g, m, v, write m, v) against the recipe tensor by tensor
+    emb = torch.nn.Parameter((torch.randn(32000, 4096, device='cuda', generator=g) * 0.02).bfloat16())
+    emb.grad = (torch.randn(32000, 4096, device='cuda', generator=g) * 1e-3).bfloat16()
+    opt = LBAdamW([emb], **hyper)
+    row = {'params': emb.numel(), 'ms': _time_gpu(opt.step, iters, warm=3)}
+    row['hbm_frac'] = emb.numel() * 19 / (row['ms'] * 1e-3) / 8e12
+    LBAdamW._plain_fusable = classmethod(lambda cls, *a: False)
+    opt._groups = None
+    try:
+        row['ms_tensor_by_tensor'] = _time_gpu(opt.step, iters, warm=3)
+    finally:
+        LBAdamW._plain_fusable = fusable
+    out['plain_embedding'] = row
     return out
 
 

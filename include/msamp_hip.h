@@ -420,15 +420,18 @@ int msamp_adamw_f32(float* param, const void* grad, int grad_dtype, size_t n, fl
                     int maximize, msamp_stream_t stream);
 
 /* The same step (adamw.py:148-199: stage 1, the scale rule on the two amaxs, stage 2) for parameters kept in high
- * precision -- biases, norm weights: a plain F32 / F16 / BF16 parameter and gradient, exp_avg in E4M3, exp_avg_sq in scaled
- * F16 -- for n_tensors of them in one launch, one workgroup per parameter, with nothing read back by the host (the
- * reference takes a dozen launches and two host round trips per parameter).  Uses the weight (the parameter, updated in
- * place in param_dtype), grad (grad_dtype, passed through the uint8_t pointer), exp_avg, exp_avg_sq, m_* and v_* fields
- * of the descriptors; meant for small tensors (a workgroup walks its whole parameter twice).  Same bits as
- * msamp_adamw_fp8_stage1 / _stage2 with the parameter rounded to its type in between. */
-int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, int param_dtype, int grad_dtype, double lr, double beta1,
-                            double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
-                            int maximize, int tensor_scale, msamp_stream_t stream);
+ * precision -- biases, norm weights, embeddings: a plain F32 / F16 / BF16 parameter and gradient, exp_avg in E4M3, exp_avg_sq
+ * in scaled F16 -- for n_tensors of them at once, with nothing read back by the host (the reference takes a dozen launches
+ * and two host round trips per parameter).  Uses the weight (the parameter, updated in place in param_dtype), grad
+ * (grad_dtype, passed through the uint8_t pointer), exp_avg, exp_avg_sq, m_* and v_* fields of the descriptors.
+ * block_map == NULL: one launch, one workgroup per parameter (which walks its parameter twice: for small tensors).
+ * Otherwise `block_map` / `n_blocks` as for msamp_adamw_fp8_fused and three launches over the chunks (stage 1, scales,
+ * stage 2), for tensors of any size; the four payload pointers of a tensor must then be aligned for four elements, and
+ * the descriptors' `acc` words zero between calls (the call leaves them so).  Same bits as msamp_adamw_fp8_stage1 /
+ * _stage2 with the parameter rounded to its type in between. */
+int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, const int32_t* block_map, int n_blocks, int param_dtype,
+                            int grad_dtype, double lr, double beta1, double beta2, double eps, double weight_decay, int step,
+                            int bias_correction, int adam_mode, int maximize, int tensor_scale, msamp_stream_t stream);
 
 #define MSAMP_ADAMW_POST_WORDS 8
 #define MSAMP_ADAMW_SYNC_BYTES(n_tensors, n_blocks) ((size_t)(n_tensors) * MSAMP_ADAMW_POST_WORDS * 8 + (size_t)(n_blocks) * 136)

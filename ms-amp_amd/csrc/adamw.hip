@@ -1388,6 +1388,136 @@ __global__ __launch_bounds__(kAdamThreads) void plain_step_kernel(msamp_adamw_te
     }
 }
 
+// The same step for parameters of any size, in three launches over 16 Ki-element chunks (`block_map` as in the fused FP8
+// step): stage 1 with its maxima into the descriptors' accumulators, the scale rule per tensor (the old dequantization
+// factors are kept in `saved` for the last launch), stage 2.  Payload pointers must be aligned for four elements.
+template <typename T>
+__device__ __forceinline__ void load4(const T* p, float* f) {
+    if constexpr (sizeof(T) == 4) {
+        const float4 t = *reinterpret_cast<const float4*>(p);
+        f[0] = t.x, f[1] = t.y, f[2] = t.z, f[3] = t.w;
+    } else {
+        const uint2 t = *reinterpret_cast<const uint2*>(p);
+        const T* h = reinterpret_cast<const T*>(&t);
+        for (int j = 0; j < 4; ++j) f[j] = Elem<T>::load(h + j);
+    }
+}
+template <typename T>
+__device__ __forceinline__ void store4(T* p, const float* f) {
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+    } else {
+        uint2 t;
+        T* h = reinterpret_cast<T*>(&t);
+        for (int j = 0; j < 4; ++j) Elem<T>::store(h + j, f[j]);
+        *reinterpret_cast<uint2*>(p) = t;
+    }
+}
+
+template <typename PT, typename GT, bool L2>
+__device__ __forceinline__ void plain_stage1(float& pj, float gj, float m_old, float v_old, float inv_m, float inv_v,
+                                             const AdamConsts& k, float& mxm, float& mxv) {
+#pragma clang fp contract(off)
+    if (k.maximize) gj = -gj;
+    if constexpr (L2) gj = fmaf(k.wd, pj, gj);    // as in plain_step_kernel
+    else pj = pj * k.decay;
+    float m_new, v_new;
+    moments(m_old, v_old, gj, inv_m, inv_v, k, m_new, v_new);
+    mxm = fmaxf(mxm, fabsf(m_new));
+    mxv = fmaxf(mxv, fabsf(v_new));
+    pj = param_update(pj, m_new, v_new, k);
+}
+
+template <typename PT, typename GT, bool L2>
+__global__ __launch_bounds__(kAdamThreads) void plain_amax_kernel(msamp_adamw_tensor* __restrict__ tensors,
+                                                                   const int32_t* __restrict__ block_map, AdamConsts k) {
+    __shared__ uint32_t red[kAdamThreads / kWave];
+    msamp_adamw_tensor& d = tensors[block_map[2 * blockIdx.x]];
+    const size_t n = d.numel, first = static_cast<size_t>(block_map[2 * blockIdx.x + 1]) * MSAMP_ADAMW_CHUNK;
+    const size_t last = first + MSAMP_ADAMW_CHUNK < n ? first + MSAMP_ADAMW_CHUNK : n;
+    PT* param = static_cast<PT*>(d.weight);
+    const GT* grad = reinterpret_cast<const GT*>(d.grad);
+    const float inv_m = 1.0f / *d.m_scale, inv_v = 1.0f / *d.v_scale;
+    float mxm = 0.0f, mxv = 0.0f;
+    for (size_t i = first + threadIdx.x * 4; i < last; i += kAdamThreads * 4) {
+        if (i + 4 <= last) {
+            float p[4], g[4], m[4];
+            load4<PT>(param + i, p);
+            load4<GT>(grad + i, g);
+            dequant4<MSAMP_DT_E4M3>(*reinterpret_cast<const uint32_t*>(d.exp_avg + i), m[0], m[1], m[2], m[3]);
+            const uint2 vv = *reinterpret_cast<const uint2*>(d.exp_avg_sq + i);
+            const float v[4] = {f16_bits_to_float(vv.x & 0xffffu), f16_bits_to_float(vv.x >> 16), f16_bits_to_float(vv.y & 0xffffu),
+                                f16_bits_to_float(vv.y >> 16)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) plain_stage1<PT, GT, L2>(p[j], g[j], m[j], v[j], inv_m, inv_v, k, mxm, mxv);
+            store4<PT>(param + i, p);
+        } else {
+            for (size_t e = i; e < last; ++e) {
+                float pj = Elem<PT>::load(param + e);
+                plain_stage1<PT, GT, L2>(pj, Elem<GT>::load(grad + e), dequant1<MSAMP_DT_E4M3>(d.exp_avg[e]),
+                                         f16_bits_to_float(d.exp_avg_sq[e]), inv_m, inv_v, k, mxm, mxv);
+                Elem<PT>::store(param + e, pj);
+            }
+        }
+    }
+    const uint32_t a = block_max_u32(__float_as_uint(mxm), red);
+    const uint32_t b = block_max_u32(__float_as_uint(mxv), red);
+    if (threadIdx.x == 0) {
+        atomicMax(&d.acc[1], a);
+        atomicMax(&d.acc[2], b);
+    }
+}
+
+__global__ void plain_scales_kernel(msamp_adamw_tensor* tensors, int n_tensors, int tensor_scale) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n_tensors) return;
+    msamp_adamw_tensor& d = tensors[t];
+    const float am = __uint_as_float(d.acc[1]), av = __uint_as_float(d.acc[2]);
+    d.acc[1] = 0u, d.acc[2] = 0u;
+    d.saved[1] = 1.0f / *d.m_scale;
+    d.saved[2] = 1.0f / *d.v_scale;
+    const float ms = tensor_scale ? scale_rule(am, 1.0f, 448.0f, 0) : 1.0f;
+    const float vs = tensor_scale ? scale_rule(av, 1.0f, 65504.0f, 0) : 1.0f;
+    *d.m_scale = ms, *d.m_scale_inv = 1.0f / ms, *d.m_amax = am;
+    *d.v_scale = vs, *d.v_scale_inv = 1.0f / vs, *d.v_amax = av;
+}
+
+template <typename GT>
+__global__ __launch_bounds__(kAdamThreads) void plain_write_kernel(msamp_adamw_tensor* __restrict__ tensors,
+                                                                    const int32_t* __restrict__ block_map, AdamConsts k) {
+    msamp_adamw_tensor& d = tensors[block_map[2 * blockIdx.x]];
+    const size_t n = d.numel, first = static_cast<size_t>(block_map[2 * blockIdx.x + 1]) * MSAMP_ADAMW_CHUNK;
+    const size_t last = first + MSAMP_ADAMW_CHUNK < n ? first + MSAMP_ADAMW_CHUNK : n;
+    const GT* grad = reinterpret_cast<const GT*>(d.grad);
+    const float inv_m = d.saved[1], inv_v = d.saved[2], ms = *d.m_scale, vs = *d.v_scale;
+    for (size_t i = first + threadIdx.x * 4; i < last; i += kAdamThreads * 4) {
+        if (i + 4 <= last) {
+            float g[4], m[4], mn[4], vn[4];
+            load4<GT>(grad + i, g);
+            dequant4<MSAMP_DT_E4M3>(*reinterpret_cast<const uint32_t*>(d.exp_avg + i), m[0], m[1], m[2], m[3]);
+            const uint2 vv = *reinterpret_cast<const uint2*>(d.exp_avg_sq + i);
+            const float v[4] = {f16_bits_to_float(vv.x & 0xffffu), f16_bits_to_float(vv.x >> 16), f16_bits_to_float(vv.y & 0xffffu),
+                                f16_bits_to_float(vv.y >> 16)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) moments(m[j], v[j], k.maximize ? -g[j] : g[j], inv_m, inv_v, k, mn[j], vn[j]);
+            *reinterpret_cast<uint32_t*>(d.exp_avg + i) = quant4<MSAMP_DT_E4M3>(mn[0] * ms, mn[1] * ms, mn[2] * ms, mn[3] * ms);
+            uint2 out;
+            out.x = float_to_f16_bits(vn[0] * vs) | (float_to_f16_bits(vn[1] * vs) << 16);
+            out.y = float_to_f16_bits(vn[2] * vs) | (float_to_f16_bits(vn[3] * vs) << 16);
+            *reinterpret_cast<uint2*>(d.exp_avg_sq + i) = out;
+        } else {
+            for (size_t e = i; e < last; ++e) {
+                const float gj = Elem<GT>::load(grad + e);
+                float m_new, v_new;
+                moments(dequant1<MSAMP_DT_E4M3>(d.exp_avg[e]), f16_bits_to_float(d.exp_avg_sq[e]), k.maximize ? -gj : gj, inv_m, inv_v, k,
+                        m_new, v_new);
+                d.exp_avg[e] = static_cast<uint8_t>(quant1<MSAMP_DT_E4M3>(m_new * ms));
+                d.exp_avg_sq[e] = static_cast<uint16_t>(float_to_f16_bits(v_new * vs));
+            }
+        }
+    }
+}
+
 // ---- float32 moments ------------------------------------------------------------------------------------------------
 // The branch of LBAdamW.adamw_fn for float32 exp_avg / exp_avg_sq (msamp/optim/adamw.py:200-232) is a chain of a dozen
 // element-wise torch calls per parameter; this kernel is that chain in one pass, with every intermediate rounded where
@@ -1417,18 +1547,6 @@ __device__ __forceinline__ void f32_element(float& p, float g, float& m, float& 
     p = fmaf(k.neg_step, r, p);
 }
 
-template <typename GT>
-__device__ __forceinline__ void load_grad4(const GT* g, float* f) {
-    if constexpr (sizeof(GT) == 4) {
-        const float4 t = *reinterpret_cast<const float4*>(g);
-        f[0] = t.x, f[1] = t.y, f[2] = t.z, f[3] = t.w;
-    } else {
-        const uint2 t = *reinterpret_cast<const uint2*>(g);
-        const GT* h = reinterpret_cast<const GT*>(&t);
-        for (int j = 0; j < 4; ++j) f[j] = Elem<GT>::load(h + j);
-    }
-}
-
 // VEC: every pointer is aligned for four elements
 template <typename GT, bool L2, bool VEC>
 __global__ __launch_bounds__(kAdamThreads) void f32_step_kernel(float* __restrict__ param, const GT* __restrict__ grad,
@@ -1445,7 +1563,7 @@ __global__ __launch_bounds__(kAdamThreads) void f32_step_kernel(float* __restric
             float4 m4 = *reinterpret_cast<const float4*>(exp_avg + i);
             float4 v4 = *reinterpret_cast<const float4*>(exp_avg_sq + i);
             float g[4];
-            load_grad4<GT>(grad + i, g);
+            load4<GT>(grad + i, g);
             f32_element<L2>(p4.x, g[0], m4.x, v4.x, k);
             f32_element<L2>(p4.y, g[1], m4.y, v4.y, k);
             f32_element<L2>(p4.z, g[2], m4.z, v4.z, k);
@@ -1685,11 +1803,12 @@ int msamp_adamw_f32(float* param, const void* grad, int grad_dtype, size_t n, fl
     return MSAMP_OK;
 }
 
-int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, int param_dtype, int grad_dtype, double lr, double beta1,
-                            double beta2, double eps, double weight_decay, int step, int bias_correction, int adam_mode,
-                            int maximize, int tensor_scale, msamp_stream_t stream) {
-    MSAMP_REQUIRE(n_tensors >= 0, MSAMP_ERR_SHAPE, "msamp_adamw_plain_fused: n_tensors=%d", n_tensors);
-    if (n_tensors == 0) return MSAMP_OK;
+int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, const int32_t* block_map, int n_blocks, int param_dtype,
+                            int grad_dtype, double lr, double beta1, double beta2, double eps, double weight_decay, int step,
+                            int bias_correction, int adam_mode, int maximize, int tensor_scale, msamp_stream_t stream) {
+    MSAMP_REQUIRE(n_tensors >= 0 && n_blocks >= 0, MSAMP_ERR_SHAPE, "msamp_adamw_plain_fused: n_tensors=%d n_blocks=%d", n_tensors,
+                  n_blocks);
+    if (n_tensors == 0 || (block_map && n_blocks == 0)) return MSAMP_OK;
     MSAMP_REQUIRE(tensors, MSAMP_ERR_NULL, "msamp_adamw_plain_fused: null pointer");
     MSAMP_REQUIRE(is_hp(param_dtype) && is_hp(grad_dtype), MSAMP_ERR_DTYPE, "msamp_adamw_plain_fused: dtypes %d, %d", param_dtype,
                   grad_dtype);
@@ -1697,10 +1816,18 @@ int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, int para
     const bool l2 = fused_consts(lr, beta1, beta2, eps, weight_decay, step, bias_correction, adam_mode, maximize, k);
     k.rule_scales = tensor_scale != 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-#define PLAIN_LAUNCH(PT, GT)                                                                                              \
-    do {                                                                                                                  \
-        if (l2) hipLaunchKernelGGL((plain_step_kernel<PT, GT, true>), dim3(n_tensors), dim3(kAdamThreads), 0, st, tensors, k); \
-        else hipLaunchKernelGGL((plain_step_kernel<PT, GT, false>), dim3(n_tensors), dim3(kAdamThreads), 0, st, tensors, k);   \
+    // block_map == NULL: one workgroup per tensor, one launch
+#define PLAIN_LAUNCH(PT, GT)                                                                                                    \
+    do {                                                                                                                        \
+        if (!block_map) {                                                                                                       \
+            if (l2) hipLaunchKernelGGL((plain_step_kernel<PT, GT, true>), dim3(n_tensors), dim3(kAdamThreads), 0, st, tensors, k);   \
+            else hipLaunchKernelGGL((plain_step_kernel<PT, GT, false>), dim3(n_tensors), dim3(kAdamThreads), 0, st, tensors, k);     \
+        } else {                                                                                                                \
+            if (l2) hipLaunchKernelGGL((plain_amax_kernel<PT, GT, true>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k);  \
+            else hipLaunchKernelGGL((plain_amax_kernel<PT, GT, false>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k);    \
+            hipLaunchKernelGGL(plain_scales_kernel, dim3((n_tensors + 63) / 64), dim3(64), 0, st, tensors, n_tensors, tensor_scale);  \
+            hipLaunchKernelGGL((plain_write_kernel<GT>), dim3(n_blocks), dim3(kAdamThreads), 0, st, tensors, block_map, k);     \
+        }                                                                                                                       \
     } while (0)
 #define PLAIN_GRAD(PT)                                                   \
     do {                                                                 \
@@ -1713,7 +1840,7 @@ int msamp_adamw_plain_fused(msamp_adamw_tensor* tensors, int n_tensors, int para
     else PLAIN_GRAD(bf16_t);
 #undef PLAIN_GRAD
 #undef PLAIN_LAUNCH
-    MSAMP_CHECK_LAUNCH("plain_step_kernel");
+    MSAMP_CHECK_LAUNCH("msamp_adamw_plain_fused");
     return MSAMP_OK;
 }
 

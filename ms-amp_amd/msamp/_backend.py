@@ -63,7 +63,7 @@ _SIGNATURES = {
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
     'msamp_adamw_f32': ([_vp, _vp, _i, _sz, _vp, _vp, _d, _d, _d, _d, _d, _i, _i, _i, _i, _vp], _i),
-    'msamp_adamw_plain_fused': ([_vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
+    'msamp_adamw_plain_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
     'msamp_adamw_fp8_fused_shift': ([_vp, _vp, _vp, _i, _vp, _i, ctypes.c_longlong, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _vp], _i),
     'msamp_adamw_fp8_fused_speculative': ([_vp, _vp, _vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
 }
@@ -766,18 +766,25 @@ def adamw_f32(param, grad, exp_avg, exp_avg_sq, lr, beta1, beta2, eps, weight_de
 
 
 def adamw_plain_fused(desc, n_tensors, param_dt, grad_dt, lr, beta1, beta2, eps, weight_decay, step, bias_correction,
-                      adam_mode, maximize, tensor_scale):
-    """Both stages of the step for n_tensors small high-precision parameters with E4M3 / scaled-fp16 moments, one launch.
-    `desc`: int64 device tensor [n_tensors, ADAMW_DESC_WORDS] with the parameter, gradient, moment payloads, moment metas
-    and numel columns filled in."""
+                      adam_mode, maximize, tensor_scale, block_map=None, n_blocks=0):
+    """Both stages of the step for n_tensors high-precision parameters with E4M3 / scaled-fp16 moments.  `desc`: int64
+    device tensor [n_tensors, ADAMW_DESC_WORDS] with the parameter, gradient, moment payloads, moment metas and numel
+    columns filled in.  Without `block_map`: one launch, one workgroup per tensor (small tensors); with it (int32 device
+    tensor of {tensor, chunk} pairs over chunks of ADAMW_CHUNK elements): three launches, any size, payloads aligned for
+    four elements."""
     lib = load()
     _gpu(desc, 'descriptor table')
     if desc.dtype != torch.int64 or desc.numel() != n_tensors * ADAMW_DESC_WORDS or not desc.is_contiguous():
         raise ValueError('desc must be a contiguous int64 tensor of n_tensors x %d words' % ADAMW_DESC_WORDS)
+    if block_map is not None:
+        _gpu(block_map, 'block map')
+        if block_map.dtype != torch.int32 or block_map.numel() != 2 * n_blocks or not block_map.is_contiguous():
+            raise ValueError('block_map must be a contiguous int32 tensor of n_blocks pairs')
     _check(
         lib.msamp_adamw_plain_fused(
-            _ptr(desc), n_tensors, param_dt, grad_dt, lr, beta1, beta2, eps, weight_decay, step, 1 if bias_correction else 0,
-            1 if adam_mode else 0, 1 if maximize else 0, 1 if tensor_scale else 0, _stream()
+            _ptr(desc), n_tensors, _ptr(block_map) if block_map is not None else None, n_blocks, param_dt, grad_dt, lr, beta1,
+            beta2, eps, weight_decay, step, 1 if bias_correction else 0, 1 if adam_mode else 0, 1 if maximize else 0,
+            1 if tensor_scale else 0, _stream()
         ), 'msamp_adamw_plain_fused'
     )
 

@@ -313,7 +313,7 @@ class LBAdamW(LBAdamWBase):
 
     # ---- parameters kept in high precision: one launch for all of them ---------------------
     _PLAIN_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
-    _PLAIN_LIMIT = 1 << 16    # elements; one workgroup walks a whole parameter, so only biases, norm weights and the like
+    _PLAIN_LIMIT = 1 << 16    # elements up to which one workgroup takes a whole parameter (biases, norm weights, ...)
 
     @classmethod
     def _plain_fusable(cls, p, g, m, v):
@@ -325,27 +325,37 @@ class LBAdamW(LBAdamWBase):
             return False
         if m.qtype != Dtypes.kfloat8_e4m3 or v.qtype != Dtypes.kfloat16 or v.value.dtype != torch.float16:
             return False
-        if not 0 < p.numel() <= cls._PLAIN_LIMIT or m.meta.amax.numel() != 1 or v.meta.amax.numel() != 1:
+        if p.numel() == 0 or m.meta.amax.numel() != 1 or v.meta.amax.numel() != 1:
             return False
         tensors = (p, g, m.value, v.value)
-        return all(t.is_cuda and t.is_contiguous() and t.numel() == p.numel() for t in tensors)
+        if not all(t.is_cuda and t.is_contiguous() and t.numel() == p.numel() for t in tensors):
+            return False
+        # larger ones go chunk by chunk, four elements at a time
+        return p.numel() <= cls._PLAIN_LIMIT or all(t.data_ptr() % 16 == 0 for t in tensors)
 
     def _plain_step(self, idx, params, grads, exp_avgs, exp_avg_sqs, step, *, beta1, beta2, lr, weight_decay, eps, maximize):
         """Both stages of the reference recipe (msamp/optim/adamw.py:148-199) for all plain parameters of one type in
-        one launch, nothing read back by the host."""
+        one launch (small ones) or three (the others, chunk by chunk), nothing read back by the host."""
         ps, gs = [params[i] for i in idx], [grads[i] for i in idx]
         ms, vs = [exp_avgs[i] for i in idx], [exp_avg_sqs[i] for i in idx]
-        if any(not g.is_contiguous() or g.numel() != p.numel() for p, g in zip(ps, gs)):
+        chunked = ps[0].numel() > self._PLAIN_LIMIT
+        if any(not g.is_contiguous() or g.numel() != p.numel() or (chunked and g.data_ptr() % 16) for p, g in zip(ps, gs)):
             self._groups = None    # (the grouping is kept from an earlier step) this step tensor by tensor
             self._staged_step(idx, params, grads, exp_avgs, exp_avg_sqs, [step] * len(params), beta1=beta1, beta2=beta2, lr=lr,
                               weight_decay=weight_decay, eps=eps, maximize=maximize)
             return
-        key = ('plain', ps[0].dtype, gs[0].dtype, id(ps[0]))
+        key = ('plain', ps[0].dtype, gs[0].dtype, chunked, id(ps[0]))
         plan = self._plans.get(key)
         ids = tuple(id(p) for p in ps)
         if plan is None or plan.params != ids:
             plan = _FusedPlan()
             plan.params = ids
+            if chunked:
+                plan.chunks = [(p.numel() + _backend.ADAMW_CHUNK - 1) // _backend.ADAMW_CHUNK for p in ps]
+                tensor_idx = np.repeat(np.arange(len(ps), dtype=np.int32), plan.chunks)
+                chunk_idx = np.concatenate([np.arange(c, dtype=np.int32) for c in plan.chunks])
+                plan.block_map = torch.from_numpy(np.stack([tensor_idx, chunk_idx], axis=1).copy()).to(ps[0].device)
+                plan.n_blocks = int(plan.block_map.shape[0])
             self._plans[key] = plan
         static = [id(t) for m, v in zip(ms, vs) for t in (m.meta.scale, m.meta.scale_inv, m.meta.amax, v.meta.scale,
                                                            v.meta.scale_inv, v.meta.amax)]
@@ -379,7 +389,8 @@ class LBAdamW(LBAdamWBase):
                         plan.desc[:, col] = torch.tensor(values, dtype=torch.int64).to(plan.desc.device)
             plan.sig = sig
         _backend.adamw_plain_fused(plan.desc, len(ps), _backend.hp_dt(ps[0]), _backend.hp_dt(gs[0]), lr, beta1, beta2, eps,
-                                   weight_decay, step, self.bias_correction, self.use_adam, maximize, self.tensor_scale)
+                                   weight_decay, step, self.bias_correction, self.use_adam, maximize, self.tensor_scale,
+                                   block_map=plan.block_map, n_blocks=plan.n_blocks)
 
     # ---- float32 moments ---------------------------------------------------------------------
     def _f32_step(self, p, g, exp_avg, exp_avg_sq, step, *, beta1, beta2, lr, weight_decay, eps, maximize):
@@ -472,7 +483,8 @@ class LBAdamW(LBAdamWBase):
                     if self._fusable(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i]):
                         fused.setdefault((int(params[i].qtype), int(grads[i].qtype), state_steps[i]), []).append(i)
                     elif self._plain_fusable(params[i], grads[i], exp_avgs[i], exp_avg_sqs[i]):
-                        plain.setdefault((params[i].dtype, grads[i].dtype, state_steps[i]), []).append(i)
+                        plain.setdefault((params[i].dtype, grads[i].dtype, state_steps[i],
+                                          params[i].numel() > self._PLAIN_LIMIT), []).append(i)
                     else:
                         staged.append(i)
                 self._groups = (key, fused, plain, staged)
