@@ -339,7 +339,10 @@ class LBAdamW(LBAdamWBase):
         ps, gs = [params[i] for i in idx], [grads[i] for i in idx]
         ms, vs = [exp_avgs[i] for i in idx], [exp_avg_sqs[i] for i in idx]
         chunked = ps[0].numel() > self._PLAIN_LIMIT
-        if any(not g.is_contiguous() or g.numel() != p.numel() or (chunked and g.data_ptr() % 16) for p, g in zip(ps, gs)):
+        payloads = [t for quad in zip(ps, gs, (m.value for m in ms), (v.value for v in vs)) for t in quad]
+        # (gradients are new tensors every step, and a parameter's storage may have been replaced)
+        if any(not g.is_contiguous() or g.numel() != p.numel() for p, g in zip(ps, gs)) or \
+                (chunked and any(t.data_ptr() % 16 for t in payloads)) or any(not t.is_contiguous() for t in payloads):
             self._groups = None    # (the grouping is kept from an earlier step) this step tensor by tensor
             self._staged_step(idx, params, grads, exp_avgs, exp_avg_sqs, [step] * len(params), beta1=beta1, beta2=beta2, lr=lr,
                               weight_decay=weight_decay, eps=eps, maximize=maximize)
