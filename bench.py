@@ -47,20 +47,31 @@ def _events():
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
-def _time_gpu(fn, iters, warm=3):
+def _time_gpu(fn, iters, warm=3, settle_ms=0.0, batches=1):
     """Average duration of one call, from HIP events around a batch of `iters` back-to-back calls on the
-    current stream (what a kernel sustains once the launch queue is primed)."""
+    current stream (what a kernel sustains once the launch queue is primed).  `settle_ms`: keep warming up until that
+    much wall time has passed (clocks, allocator pools and library heuristics settled); `batches`: time that many
+    batches and return the median one (a stall in one batch -- an allocation inside a library call -- does not
+    become the figure)."""
     import torch
-    for _ in range(warm):
+    t0 = time.perf_counter()
+    n = 0
+    while n < warm or (time.perf_counter() - t0) * 1e3 < settle_ms:
         fn()
+        n += 1
+        if settle_ms and n % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
-    s, e = _events()
-    s.record()
-    for _ in range(iters):
-        fn()
-    e.record()
-    e.synchronize()
-    return s.elapsed_time(e) / iters
+    times = []
+    for _ in range(batches):
+        s, e = _events()
+        s.record()
+        for _ in range(iters):
+            fn()
+        e.record()
+        e.synchronize()
+        times.append(s.elapsed_time(e) / iters)
+    return sorted(times)[len(times) // 2]
 
 
 # ---- synthetic inputs (bench-local: the GPU legs import nothing from tests/ or oracle/) ---------------------------
@@ -253,7 +264,7 @@ def bench_gemm_sweep(cfg, iters=10, accumulate_row=None, vendor=True):
                                                                                     lambda: x.t().contiguous())}
         mine = []
         for pname, fn, (m, n, k) in passes:
-            ms = _time_gpu(fn, iters)
+            ms = _time_gpu(fn, iters, settle_ms=30.0, batches=3)
             fl = 2.0 * m * n * k
             tf = fl / (ms * 1e-3) / 1e12
             row = {'proj': name, 'pass': pname, 'm': m, 'n': n, 'k': k, 'ms': round(ms, 4), 'tflops': round(tf, 1),
@@ -330,7 +341,7 @@ def _time_vendor(rows_op, cols_op, iters):
         fn = lambda: torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
         fn()
         torch.cuda.synchronize()
-        return _time_gpu(fn, iters)
+        return _time_gpu(fn, iters, settle_ms=30.0, batches=3)
     except (RuntimeError, AttributeError, TypeError):
         return None
 

@@ -429,10 +429,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     const bool strips_x = XT && strips(NR), strips_y = YT && strips(NC);
     bool wide = K >= 16384 && strips_x != strips_y && (strips_y ? !by_columns : by_columns);
     // Weight gradients (both operands K-major) over 16384 .. 24576 tokens: the longer operand gets the eight whenever its
-    // leading dimension is 10240 or more and a multiple of 512, whichever walk the cache rule above prefers.  Measured
+    // leading dimension is 10240 or more and a multiple of 256, whichever walk the cache rule above prefers.  Measured
     // at K = 16384 on 41 shapes (long side 5120 .. 28672, short side 4096 / 5120 / 8192, either way round) against
     // the three other walks: 10240 x 8192 +7 %, 8192 x 10240 +11 %, 14336 x 4096 +13 %, 4096 x 14336 +14 %,
-    // 8192 x 14336 +11 %, 8192 x 22016 +8 %, 13824 x 4096 +6 %, the multiples of 4096 that the rule above already turned
+    // 8192 x 14336 +11 %, 8192 x 22016 +8 %, 13824 x 4096 +6 %, 11008 x 4096 +3 %, the multiples of 4096 that the rule above already turned
     // unchanged, nothing below -2 % (5120 x 13824); +2 to 5 % at K = 20480, +1 to 3 % at 24576; nothing at K = 12288, and
     // at K = 32768 the turned patch loses 3 to 6 %.
     // Input gradients (only Y K-major) with 12288 or more columns and K of 8192 or more: Y gets the eight, walking
@@ -443,7 +443,7 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     if (XT && YT && K >= 16384 && K <= 24576 && NR != NC) {
         const bool x_long = NR > NC;
         const int long_n = x_long ? NR : NC, short_n = x_long ? NC : NR;
-        if (long_n >= 10240 && long_n % 512 == 0 && short_n <= 8192) by_columns = x_long, wide = true;
+        if (long_n >= 10240 && long_n % 256 == 0 && short_n <= 8192) by_columns = x_long, wide = true;
     }
     tile_of_id(blockIdx.x, tiles_r, tiles_c, by_columns, wide, tr, tc);
     const int row0 = tr * kDmaTile, col0 = tc * kDmaTile;
