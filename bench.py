@@ -987,6 +987,8 @@ def main():
         result['kernels'] = {
             'cast': _round_kernels(cast),
             'fused_adamw': fused,
+            'adamw_other_parameters': {k: {kk: (round(vv, 4) if isinstance(vv, float) else vv) for kk, vv in adam[k].items()}
+                                       for k in ('float32_moments', 'small_plain_parameters', 'plain_embedding')},
             'grad_side': _round_kernels(grad_side),
         }
     if not args.skip_cpu:
