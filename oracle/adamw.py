@@ -121,3 +121,35 @@ def stage2(g, m_q, inv_m, new_m_scale, v_q, inv_v, new_v_scale, *, beta1, beta2)
     m_out = fp8.encode(m_new * torch.tensor(new_m_scale, dtype=f32), fp8.E4M3)
     v_out = (v_new * torch.tensor(new_v_scale, dtype=f32)).to(v_q.dtype)
     return m_out, v_out
+
+
+def _fma(a, b, c):
+    """a * b + c with one rounding to float32: the product of two float32 is exact in float64, the sum is rounded to
+    float64 and then to float32 (a second rounding that can differ from a true fused multiply-add only when the float64
+    sum lands exactly on a float32 tie: about one element in 2**29)."""
+    return (np.float64(a) * np.asarray(b, dtype=np.float64) + np.asarray(c, dtype=np.float64)).astype(np.float32)
+
+
+def float32_step(p, g, m, v, *, lr, beta1, beta2, eps, weight_decay, step, bias_correction=True, adam_mode=False,
+                 maximize=False):
+    """The float32-moment branch of LBAdamW.adamw_fn (msamp/optim/adamw.py:200-232) on float32 numpy arrays: returns the
+    new (p, m, v).  The reference runs it as a chain of torch calls; on a GPU each `x.add(y, alpha=a)` of the chain
+    (lines 209, 223, 226, 232) evaluates x + a * y with one rounding, the division by the Python number
+    sqrt(bias_correction2) (line 228) is a multiplication by its reciprocal -- taken in double, narrowed to float32 --
+    and every other call rounds once; Python numbers are narrowed to float32 where they meet a tensor."""
+    f = np.float32
+    p, g, m, v = (np.asarray(t, dtype=np.float32) for t in (p, g, m, v))
+    if maximize:
+        g = -g
+    if weight_decay != 0:
+        if adam_mode:
+            g = _fma(f(weight_decay), p, g)                                   # :209
+        else:
+            p = p * f(1 - lr * weight_decay)                                  # :211
+    bc1 = 1 - beta1**step if bias_correction else 1.0                         # :213-217
+    bc2 = 1 - beta2**step if bias_correction else 1.0
+    m_new = _fma(f(1 - beta1), g, m * f(beta1))                               # :223
+    v_new = _fma(f(1 - beta2), g * g, v * f(beta2))                           # :226
+    denom = np.sqrt(v_new) * f(1.0 / math.sqrt(bc2)) + f(eps)                 # :228
+    p_new = _fma(f(-(lr / bc1)), m_new / denom, p)                            # :232
+    return p_new, m_new, v_new

@@ -485,3 +485,36 @@ def test_stage1_stage2_entry_points(be):
     m_want, v_want = oadam.stage2(g0, t['m'], inv_m, 4096.0, t['v'], inv_v, 2.0**20, beta1=0.9, beta2=0.999)
     be.adamw_stage2(g, m, 5, inv_m, 4096.0, 0.9, v, 3, inv_v, 2.0**20, 0.999)
     assert torch.equal(m.cpu(), m_want) and torch.equal(v.cpu(), v_want)
+
+
+@pytest.mark.parametrize('kw', [dict(), dict(adam_mode=True), dict(maximize=True, weight_decay=0.0), dict(bias_correction=False, eps=1e-6),
+                                dict(adam_mode=True, maximize=True, beta1=0.8, beta2=0.999)])
+@pytest.mark.parametrize('grad_dtype', [torch.float32, torch.bfloat16, torch.float16])
+def test_float32_moment_step_matches_the_oracle_to_the_bit(be, kw, grad_dtype):
+    """msamp_adamw_f32 against oracle.adamw.float32_step (the chain of msamp/optim/adamw.py:200-232 with the roundings it
+    has on a GPU): parameter and both moments bit-equal over three steps, on a size with a ragged tail and, offset by
+    one element, without vector loads; gradients of eight orders of magnitude, some zero, one infinite."""
+    hyper = dict(HYPER)
+    hyper.update(kw)
+    n = 3 * 65536 + 37
+    rng = np.random.default_rng(41)
+    for offset in (0, 1):
+        p = (rng.standard_normal(n) * 0.3).astype(np.float32)
+        m = np.zeros(n, np.float32)
+        v = np.zeros(n, np.float32)
+        dev = [torch.from_numpy(np.concatenate([np.zeros(offset, np.float32), t])).cuda()[offset:] for t in (p, m, v)]
+        for step in (1, 2, 3):
+            g = (rng.standard_normal(n) * 10.0 ** rng.uniform(-6, 2, n)).astype(np.float32)
+            g[::97] = 0.0
+            if step == 2:
+                g[1234] = np.inf
+            g_dev = torch.from_numpy(np.concatenate([np.zeros(offset, np.float32), g])).cuda().to(grad_dtype)[offset:].contiguous()
+            g = g_dev.float().cpu().numpy()
+            with np.errstate(all='ignore'):
+                p, m, v = oadam.float32_step(p, g, m, v, step=step, **hyper)
+            be.adamw_f32(dev[0], g_dev, dev[1], dev[2], hyper['lr'], hyper['beta1'], hyper['beta2'], hyper['eps'],
+                         hyper['weight_decay'], step, hyper.get('bias_correction', True), hyper.get('adam_mode', False),
+                         hyper.get('maximize', False))
+            torch.cuda.synchronize()
+            for got, want, name in zip(dev, (p, m, v), 'pmv'):
+                assert same_float(got, torch.from_numpy(want)), (offset, step, name)

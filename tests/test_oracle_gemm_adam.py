@@ -118,3 +118,38 @@ def test_host_constants():
 
 def test_scaling_helper_reexport():
     assert scaling.compute_scaling_factor(torch.tensor(10.0), torch.ones(()), 448.0).item() == 32.0
+
+
+def test_float32_moment_step_matches_textbook_adamw_and_adam():
+    """oracle.adamw.float32_step against torch.optim.AdamW / Adam in float64 from the same state (to float32 rounding),
+    decoupled decay and L2 mode, with and without maximize; and two closed forms: a zero gradient with zero moments
+    leaves the moments at zero and only decays the parameter, and at step 1 from zero moments the update is
+    lr * sign(g) for |g| far above eps."""
+    import numpy as np
+    rng = np.random.default_rng(3)
+    n = 5000
+    p0 = rng.standard_normal(n).astype(np.float32) * 0.3
+    g0 = rng.standard_normal(n).astype(np.float32) * 1e-2
+    m0 = rng.standard_normal(n).astype(np.float32) * 1e-2
+    v0 = (rng.standard_normal(n).astype(np.float32) * 1e-2) ** 2
+    for cls, adam_mode in ((torch.optim.AdamW, False), (torch.optim.Adam, True)):
+        for maximize in (False, True):
+            step = 7
+            got = adamw.float32_step(p0, g0, m0, v0, lr=3e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=step,
+                                     adam_mode=adam_mode, maximize=maximize)
+            param = torch.nn.Parameter(torch.from_numpy(p0).double())
+            opt = cls([param], lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1, maximize=maximize)
+            opt.state[param] = {'step': torch.tensor(float(step - 1)), 'exp_avg': torch.from_numpy(m0).double(),
+                                'exp_avg_sq': torch.from_numpy(v0).double()}
+            param.grad = torch.from_numpy(g0).double()
+            opt.step()
+            want = (param.detach(), opt.state[param]['exp_avg'], opt.state[param]['exp_avg_sq'])
+            for a, b, atol in zip(got, want, (3e-7, 1e-8, 1e-10)):
+                assert a.dtype == np.float32
+                assert torch.allclose(torch.from_numpy(a).double(), b, rtol=2e-6, atol=atol)
+    zero = np.zeros(n, np.float32)
+    p1, m1, v1 = adamw.float32_step(p0, zero, zero, zero, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.5, step=3)
+    assert not m1.any() and not v1.any() and np.array_equal(p1, p0 * np.float32(1 - 1e-2 * 0.5))
+    p1, m1, v1 = adamw.float32_step(p0, g0 + np.sign(g0), zero, zero, lr=1e-2, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.0,
+                                    step=1)
+    assert np.allclose(p0 - p1, 1e-2 * np.sign(g0), rtol=1e-5, atol=0)
