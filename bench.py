@@ -39,6 +39,9 @@ LLAMA_7B = {'tokens': 16384, 'proj': (('qkv', 12288, 4096), ('o', 4096, 4096), (
                                        ('up', 11008, 4096), ('down', 4096, 11008))}
 LLAMA_70B = {'tokens': 16384, 'proj': (('qkv', 10240, 8192), ('o', 8192, 8192), ('gate', 28672, 8192),
                                         ('up', 28672, 8192), ('down', 8192, 28672))}
+# not a BASELINE configuration: a Llama-3-8B layer (MLP width 14336), shapes on which the tile-walk rules were not measured
+LLAMA3_8B = {'tokens': 16384, 'proj': (('qkv', 6144, 4096), ('o', 4096, 4096), ('gate', 14336, 4096), ('up', 14336, 4096),
+                                       ('down', 4096, 14336))}
 CONFIG_2 = {'tokens': 8192, 'proj': (('linear', 4096, 4096), )}
 
 
@@ -850,7 +853,7 @@ def main():
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--skip-cpu', action='store_true', help='leave out the CPU-oracle baseline')
     ap.add_argument('--skip-extra', action='store_true', help='leave out the sweep, cast and Adam kernel sections')
-    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'gemm_small', 'cast', 'adam', 'grad_side', 'power'), default=None,
+    ap.add_argument('--only', choices=('gemm_c2', 'gemm_c4', 'gemm_c5', 'gemm_llama3_8b', 'gemm_small', 'cast', 'adam', 'grad_side', 'power'), default=None,
                     help='run one kernel section alone (after the calibration copy), for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
@@ -870,6 +873,8 @@ def main():
             out = bench_gemm_sweep(LLAMA_7B, iters=3, accumulate_row='gate')
         elif args.only == 'gemm_c5':
             out = bench_gemm_sweep(LLAMA_70B, iters=3)
+        elif args.only == 'gemm_llama3_8b':
+            out = bench_gemm_sweep(LLAMA3_8B, iters=3)
         elif args.only == 'cast':
             out = _round_kernels(bench_cast())
         elif args.only == 'grad_side':
@@ -880,7 +885,10 @@ def main():
             out = bench_small_gemms()
         else:
             out = bench_adam()
-        print(json.dumps({'only': args.only, 'result': out}))
+        from msamp import _backend as _be
+        walks = {'%dx%dx%d%s%s' % (k[0], k[1], k[2], ' aT' if k[3] else '', ' bT' if k[4] else ''): w
+                 for k, w in sorted(_be.gemm_walks().items())}
+        print(json.dumps({'only': args.only, 'result': out, 'gemm_walks_timed_at_first_use': walks}))
         return
 
     lin = bench_layer(LLAMA_7B, args.steps, args.warmup)
@@ -991,6 +999,10 @@ def main():
                                        for k in ('float32_moments', 'small_plain_parameters', 'plain_embedding')},
             'grad_side': _round_kernels(grad_side),
         }
+    # the tile walks that timing at first use registered in place of the rules' (m, n, k, a K-major, b K-major -> walk)
+    from msamp import _backend as _be
+    result['gemm_walks_timed_at_first_use'] = {'%dx%dx%d%s%s' % (k[0], k[1], k[2], ' aT' if k[3] else '', ' bT' if k[4] else ''): w
+                                               for k, w in sorted(_be.gemm_walks().items())}
     if not args.skip_cpu:
         result['cpu_baseline'] = cpu_baseline()
     print(json.dumps(result))

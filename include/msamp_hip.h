@@ -291,6 +291,24 @@ int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, 
                         float* scale, float* amax, float* scale_inv, int m, int n, int k, int margin, int flags,
                         void* workspace, msamp_stream_t stream);
 
+/* Tile walks of the 256 x 256-tile kernel (no counterpart in the reference, whose GEMM is cuBLASLt behind
+ * transformer_engine_wrapper.py:63-103).  Which workgroup takes which output tile decides what the 32 compute units of
+ * an XCD share through their L2; the library picks a walk from the shape by rules measured on Llama shapes, and the
+ * best one for another shape can be up to 13 % faster.  A walk is a number 0..3: bit 0 = groups of eight tile columns
+ * walked row by row (instead of groups of tile rows walked column by column), bit 1 = the XCD's patch of 32 tiles
+ * turned, 4 of the grouped dimension by 8 of the walked one.  Every walk gives the same output bits.
+ * msamp_fp8_gemm_set_walk registers a walk for one problem -- (m, n, k) and operand layouts as in msamp_fp8_gemm_kmajor --
+ * for all later calls of every GEMM entry point, walk = -1 removes it; msamp_fp8_gemm_get_walk returns it, -1 if none.
+ * msamp_fp8_gemm_tune computes the product like msamp_fp8_gemm_kmajor with accumulate = 0 and, when the problem has at
+ * least two rounds of tiles and `stream` is not being captured, times the rule's walk and the four explicit ones on the
+ * operands given (some forty launches between HIP events; it synchronises with the stream) and registers the fastest if
+ * it beats the rule's by more than 3 %; *chosen (nullable) receives the registered walk or -1.  Process-wide. */
+int msamp_fp8_gemm_set_walk(int m, int n, int k, int a_kmajor, int b_kmajor, int walk);
+int msamp_fp8_gemm_get_walk(int m, int n, int k, int a_kmajor, int b_kmajor);
+int msamp_fp8_gemm_tune(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b, int b_type,
+                        const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int m, int n, int k, const void* bias,
+                        int bias_dtype, int* chosen, msamp_stream_t stream);
+
 /* msamp_fp8_gemm with row-major operands runs 256 x 256 output tiles, one workgroup each; a problem with few of them
  * (a 2048 x 2048 output has 64, a quarter of the compute units) runs 128 x 128 tiles instead when it has at most
  * `big_tiles` of the large ones (at most half that many if K < 3072), K is a multiple of 128 and at least 512.  Same

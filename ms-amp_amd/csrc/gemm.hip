@@ -5,6 +5,9 @@
 #include "gemm_call.h"
 
 #include <atomic>
+#include <map>
+#include <mutex>
+#include <tuple>
 
 namespace msamp {
 
@@ -21,6 +24,18 @@ static bool kmajor_shape_ok(int NR, int NC, int K, bool xt, bool yt) {
     return K % kBK == 0 && K >= 2 * kBK && fits32 && (!xt || NR % kDmaTile == 0) && (!yt || NC % kDmaTile == 0);
 }
 
+// tile walks registered per problem (kernel-side naming: NR x NC output, K, which operands are K-major)
+static std::mutex g_walk_mutex;
+static std::map<std::tuple<int, int, int, int>, int> g_walks;
+static thread_local int t_forced_walk = -2;    // -2: none; msamp_fp8_gemm_tune times its candidates through this
+int registered_walk(int NR, int NC, int K, bool XT, bool YT) {
+    if (t_forced_walk != -2) return t_forced_walk;
+    std::lock_guard<std::mutex> lock(g_walk_mutex);
+    if (g_walks.empty()) return -1;
+    const auto it = g_walks.find(std::make_tuple(NR, NC, K, (XT ? 1 : 0) | (YT ? 2 : 0)));
+    return it == g_walks.end() ? -1 : it->second;
+}
+
 static std::atomic<int> g_small_tile_limit{128};
 int small_tile_limit() { return g_small_tile_limit.load(std::memory_order_relaxed); }
 
@@ -30,6 +45,78 @@ using namespace msamp;
 
 extern "C" void msamp_set_small_tile_limit(int big_tiles) {
     msamp::g_small_tile_limit.store(big_tiles < 0 ? 0 : big_tiles, std::memory_order_relaxed);
+}
+
+extern "C" int msamp_fp8_gemm_set_walk(int m, int n, int k, int a_kmajor, int b_kmajor, int walk) {
+    MSAMP_REQUIRE(walk >= -1 && walk <= 3, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_set_walk: walk=%d", walk);
+    // X = b (n rows of D), Y = a (m columns of D)
+    const auto key = std::make_tuple(n, m, k, (b_kmajor ? 1 : 0) | (a_kmajor ? 2 : 0));
+    std::lock_guard<std::mutex> lock(msamp::g_walk_mutex);
+    if (walk < 0) msamp::g_walks.erase(key);
+    else msamp::g_walks[key] = walk;
+    return MSAMP_OK;
+}
+
+extern "C" int msamp_fp8_gemm_get_walk(int m, int n, int k, int a_kmajor, int b_kmajor) {
+    std::lock_guard<std::mutex> lock(msamp::g_walk_mutex);
+    const auto it = msamp::g_walks.find(std::make_tuple(n, m, k, (b_kmajor ? 1 : 0) | (a_kmajor ? 2 : 0)));
+    return it == msamp::g_walks.end() ? -1 : it->second;
+}
+
+extern "C" int msamp_fp8_gemm_tune(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b,
+                                   int b_type, const float* b_scale_inv, int b_kmajor, void* d, int d_dtype, int m, int n,
+                                   int k, const void* bias, int bias_dtype, int* chosen, msamp_stream_t stream) {
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto run = [&]() {
+        return msamp_fp8_gemm_kmajor(a, a_type, a_scale_inv, a_kmajor, b, b_type, b_scale_inv, b_kmajor, d, d_dtype, m, n, k, 0, bias,
+                                     bias_dtype, stream);
+    };
+    if (chosen) *chosen = -1;
+    // Only problems of the 256 x 256-tile kernel with at least two rounds of tiles have a walk worth timing, and timing
+    // needs a stream that is not being captured; everything else is the plain product.
+    const long tiles = (static_cast<long>(n) + kDmaTile - 1) / kDmaTile * ((static_cast<long>(m) + kDmaTile - 1) / kDmaTile);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess) capturing = hipStreamCaptureStatusActive, (void)hipGetLastError();
+    const bool candidate = m > 0 && n > 0 && k >= 4 * kBK && k % kBK == 0 && tiles >= 2L * cu_count() && !takes_small_tiles(n, m, k) &&
+                           capturing == hipStreamCaptureStatusNone;
+    if (!candidate) return run();
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        if (e0) (void)hipEventDestroy(e0);
+        (void)hipGetLastError();
+        return run();
+    }
+    // the rule's walk first, then the four explicit ones: two untimed launches, then as many as fill about four
+    // milliseconds (at least four) between one pair of events
+    float best_ms = 0.0f, rule_ms = 0.0f;
+    int best = -1, rc = MSAMP_OK;
+    for (int walk = -1; walk <= 3 && rc == MSAMP_OK; ++walk) {
+        msamp::t_forced_walk = walk;
+        for (int i = 0; i < 2 && rc == MSAMP_OK; ++i) rc = run();
+        int reps = 4;
+        if (walk >= 0 && rule_ms > 0.0f) reps = std::max(4, std::min(64, static_cast<int>(4.0f / rule_ms)));
+        if (rc == MSAMP_OK && hipEventRecord(e0, st) != hipSuccess) rc = MSAMP_ERR_HIP;
+        for (int i = 0; i < reps && rc == MSAMP_OK; ++i) rc = run();
+        float ms = 0.0f;
+        if (rc == MSAMP_OK && (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+                               hipEventElapsedTime(&ms, e0, e1) != hipSuccess))
+            rc = MSAMP_ERR_HIP;
+        ms /= reps;
+        if (walk < 0) rule_ms = best_ms = ms;
+        else if (ms < best_ms) best_ms = ms, best = walk;
+    }
+    msamp::t_forced_walk = -2;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != MSAMP_OK) {
+        (void)hipGetLastError();
+        return run();
+    }
+    // an explicit walk is kept only where it beats the rule's by more than the timing's noise
+    if (best >= 0 && best_ms > 0.97f * rule_ms) best = -1;
+    msamp_fp8_gemm_set_walk(m, n, k, a_kmajor, b_kmajor, best);
+    if (chosen) *chosen = best;
+    return MSAMP_OK;    // (d holds the product: every timed launch wrote it)
 }
 
 // words of the workspace that the speculative form of msamp_fp8_gemm_cast uses: running maximum, ticket counter (both

@@ -21,6 +21,7 @@ struct QuantArgs {
     uint32_t spin_limit;
     uint32_t* error_word;    // sticky: set when a bounded wait runs out
     uint32_t* spec_words;    // speculative form: [0] running maximum, [1] ticket counter (both zero between calls), [2] out: 1 = cast again
+    int walk_plus_one;       // every form of the kernel: 0 = the tile walk the built-in rule picks, 1..4 = walk 0..3 (see registered_walk)
 };
 
 // One product D[NR][NC] = X[NR][K] . Y[NC][K]^T * *xs * *ys.  xt / yt: that operand is handed over K-major.
@@ -48,6 +49,11 @@ int run_gemm_pair(const GemmCall& c);
 
 // Problems of at most this many 256 x 256 tiles take the kernel with 128 x 128 tiles (msamp_set_small_tile_limit) ...
 int small_tile_limit();
+// The tile walk registered for this problem of the 256 x 256-tile kernel (msamp_fp8_gemm_set_walk / _tune), or -1: bit 0 =
+// groups of tile columns walked row by row instead of groups of tile rows, bit 1 = the XCD's patch of 32 tiles turned (4 of
+// the grouped dimension x 8 of the walked one).  Any walk gives the same output bits: it only decides which workgroup
+// takes which tile.
+int registered_walk(int NR, int NC, int K, bool XT, bool YT);
 // ... which is this rule: K in whole slices, at least four of them; up to half the limit always (one small tile per
 // compute unit with the default limit), up to the limit where K is long enough for the second round of small tiles to
 // pay (measured: 128 large tiles level at K = 2048, 15 % ahead at 4096).

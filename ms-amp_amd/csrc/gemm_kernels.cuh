@@ -445,6 +445,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         const int long_n = x_long ? NR : NC, short_n = x_long ? NC : NR;
         if (long_n >= 10240 && long_n % 256 == 0 && short_n <= 8192) by_columns = x_long, wide = true;
     }
+    // a walk registered for this problem (timed on this machine) overrides the rules
+    if (qa.walk_plus_one > 0) by_columns = (qa.walk_plus_one - 1) & 1, wide = ((qa.walk_plus_one - 1) >> 1) & 1;
     tile_of_id(blockIdx.x, tiles_r, tiles_c, by_columns, wide, tr, tc);
     const int row0 = tr * kDmaTile, col0 = tc * kDmaTile;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1081,8 +1083,10 @@ static int launch_gemm_dma_parity(const uint8_t* X, const uint8_t* Y, void* D, i
         configured.store(true, std::memory_order_release);
     }
     const int tiles = ((NR + kDmaTile - 1) / kDmaTile) * ((NC + kDmaTile - 1) / kDmaTile);
+    QuantArgs qa = {};
+    qa.walk_plus_one = registered_walk(NR, NC, K, XT, YT) + 1;
     hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys,
-                       accumulate, bias, bias_dt, QuantArgs{});
+                       accumulate, bias, bias_dt, qa);
     MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel");
     return MSAMP_OK;
 }
@@ -1117,8 +1121,10 @@ static int launch_gemm_dma_quant_parity(const uint8_t* X, const uint8_t* Y, int 
     }
     if (!fits) return MSAMP_NOT_FUSED;
     const int tiles = (NR / kDmaTile) * (NC / kDmaTile);
+    QuantArgs qw = qa;
+    qw.walk_plus_one = registered_walk(NR, NC, K, XT, YT) + 1;
     hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(nullptr), NR, NC, K, xs, ys, 0,
-                       static_cast<const void*>(nullptr), 0, qa);
+                       static_cast<const void*>(nullptr), 0, qw);
     MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel (fused cast)");
     return MSAMP_OK;
 }
@@ -1143,8 +1149,10 @@ static int launch_gemm_dma_spec_parity(const uint8_t* X, const uint8_t* Y, void*
         configured.store(true, std::memory_order_release);
     }
     const int tiles = (NR / kDmaTile) * (NC / kDmaTile);
+    QuantArgs qw = qa;
+    qw.walk_plus_one = registered_walk(NR, NC, K, XT, YT) + 1;
     hipLaunchKernelGGL(kern, dim3(tiles), dim3(kGemmThreads), smem, st, X, Y, static_cast<OT*>(D), NR, NC, K, xs, ys, accumulate,
-                       static_cast<const void*>(nullptr), 0, qa);
+                       static_cast<const void*>(nullptr), 0, qw);
     MSAMP_CHECK_LAUNCH("fp8_gemm_dma_kernel (speculative cast)");
     return MSAMP_OK;
 }

@@ -62,6 +62,9 @@ _SIGNATURES = {
     'msamp_adamw_fp8_stage1': ([_vp, _vp, _sz, _vp, _i, _f, _vp, _f, _vp, _i, _f, _vp, _f, _f, _i, _f, _i, _vp], _i),
     'msamp_adamw_fp8_stage2': ([_vp, _sz, _vp, _i, _f, _f, _f, _vp, _i, _f, _f, _f, _vp], _i),
     'msamp_adamw_fp8_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _i, _vp], _i),
+    'msamp_fp8_gemm_set_walk': ([_i, _i, _i, _i, _i, _i], _i),
+    'msamp_fp8_gemm_get_walk': ([_i, _i, _i, _i, _i], _i),
+    'msamp_fp8_gemm_tune': ([_vp, _i, _vp, _i, _vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _i, _vp, _vp], _i),
     'msamp_adamw_f32': ([_vp, _vp, _i, _sz, _vp, _vp, _d, _d, _d, _d, _d, _i, _i, _i, _i, _vp], _i),
     'msamp_adamw_plain_fused': ([_vp, _i, _vp, _i, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp], _i),
     'msamp_adamw_fp8_fused_shift': ([_vp, _vp, _vp, _i, _vp, _i, ctypes.c_longlong, _i, _i, _d, _d, _d, _d, _d, _i, _i, _i, _i, _i, _vp, _vp], _i),
@@ -488,12 +491,65 @@ def gemm_kmajor_supported(m, n, k, a_kmajor, b_kmajor):
         m * k < 2**32 and n * k < 2**32
 
 
+# ---- tile walks of the large GEMM, timed at first use ---------------------------------------------------------------
+_tune_walks = os.environ.get('MSAMP_GEMM_TUNE', '1') != '0'
+_walk_seen = set()
+_TUNE_MIN_TILES = 512    # two rounds of 256 x 256 tiles on 256 compute units: below that the library does not time anything
+
+
+def tune_gemm_walks(on=True):
+    """Whether a GEMM problem (sizes and operand layouts) seen for the first time has its tile walk timed: the product of
+    that call is computed some forty times over, and the fastest of the walks is used from then on (same bits whichever).
+    On by default; the environment variable MSAMP_GEMM_TUNE=0 switches it off from the start."""
+    global _tune_walks
+    _tune_walks = bool(on)
+
+
+def forget_gemm_walks():
+    """Drop every walk registered so far (the next call of each problem times again if tuning is on)."""
+    lib = load()
+    for m, n, k, a_kmajor, b_kmajor in _walk_seen:
+        lib.msamp_fp8_gemm_set_walk(m, n, k, int(a_kmajor), int(b_kmajor), -1)
+    _walk_seen.clear()
+
+
+def gemm_walks():
+    """{(m, n, k, a_kmajor, b_kmajor): walk} of the problems whose timing registered a walk other than the rule's."""
+    lib = load()
+    found = {key: lib.msamp_fp8_gemm_get_walk(key[0], key[1], key[2], int(key[3]), int(key[4])) for key in _walk_seen}
+    return {key: walk for key, walk in found.items() if walk >= 0}
+
+
+def _tune_walk(lib, a, a_dt, a_scale_inv, a_kmajor, b, b_dt, b_scale_inv, b_kmajor, out, m, n, k, bias):
+    """Times the walks of a problem not seen before on the operands given, writing the product to `out`; False (nothing
+    done) if the problem has been seen, is too small to matter, or the stream is being captured."""
+    key = (m, n, k, bool(a_kmajor), bool(b_kmajor))
+    if key in _walk_seen or ((n + 255) // 256) * ((m + 255) // 256) < _TUNE_MIN_TILES or k < 512 or k % 128:
+        return False
+    if torch.cuda.is_current_stream_capturing():
+        return False
+    _walk_seen.add(key)
+    _check(
+        lib.msamp_fp8_gemm_tune(
+            _ptr(a), a_dt, _ptr(a_scale_inv), 1 if a_kmajor else 0, _ptr(b), b_dt, _ptr(b_scale_inv), 1 if b_kmajor else 0,
+            _ptr(out), _dt(out), m, n, k, _ptr(bias), _dt(bias) if bias is not None else DT_F32, None, _stream()
+        ), 'msamp_fp8_gemm_tune'
+    )
+    return True
+
+
 def fp8_gemm(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, out, accumulate=False, bias=None, a_kmajor=False, b_kmajor=False):
     """out[N,M] (+)= (b[N,K] . a[M,K]^T) * a_scale_inv * b_scale_inv (+ bias[M]).
     With a_kmajor / b_kmajor the tensor handed over is the transpose, [K,M] / [K,N]."""
     lib = load()
     _gpu(a, 'mat_a')
     _gpu(b, 'mat_b')
+    if _tune_walks and not accumulate and a.dim() == 2 and b.dim() == 2 and (a_kmajor or not b_kmajor):
+        k, m = a.shape if a_kmajor else a.shape[::-1]
+        kb, n = b.shape if b_kmajor else b.shape[::-1]
+        if kb == k and tuple(out.shape) == (n, m) and out.is_contiguous() and \
+                _tune_walk(lib, a, a_dt, a_scale_inv, a_kmajor, b, b_dt, b_scale_inv, b_kmajor, out, m, n, k, bias):
+            return out
     if a_kmajor or b_kmajor:
         k, m = a.shape if a_kmajor else a.shape[::-1]
         kb, n = b.shape if b_kmajor else b.shape[::-1]
@@ -547,6 +603,13 @@ def fp8_gemm_cast(a, a_dt, a_scale_inv, b, b_dt, b_scale_inv, hp_dtype, q_dt, sc
         raise ValueError(f'hp_out must be a contiguous {hp_dtype} tensor of shape {(n, m)}')
     if hp_out is None and speculate and m % 256 == 0 and n % 256 == 0 and (n // 256) * (m // 256) > 0:
         hp_out = torch.empty(n, m, dtype=hp_dtype, device=a.device)
+    if _tune_walks and (a_kmajor or not b_kmajor):
+        # (the product into a scratch buffer of its own: hp_out may hold a sum that is being added to)
+        key = (m, n, k, bool(a_kmajor), bool(b_kmajor))
+        if key not in _walk_seen and ((n + 255) // 256) * ((m + 255) // 256) >= _TUNE_MIN_TILES and \
+                not torch.cuda.is_current_stream_capturing():
+            _tune_walk(lib, a, a_dt, a_scale_inv, a_kmajor, b, b_dt, b_scale_inv, b_kmajor,
+                       torch.empty(n, m, dtype=hp_dtype, device=a.device), m, n, k, None)
     out = torch.empty(n, m, dtype=torch.uint8, device=a.device)
     rc = lib.msamp_fp8_gemm_cast(
         _ptr(a), a_dt, _ptr(a_scale_inv), 1 if a_kmajor else 0, _ptr(b), b_dt, _ptr(b_scale_inv), 1 if b_kmajor else 0,

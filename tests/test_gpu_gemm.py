@@ -764,7 +764,78 @@ def test_every_tile_is_written_whatever_the_walk(be, nr, nc, k, a_kmajor, b_kmaj
     y = ys.view(1, nc).expand(k, nc).contiguous() if a_kmajor else ys.view(nc, 1).expand(nc, k).contiguous()
     out = torch.full((nr, nc), float('nan'), dtype=torch.bfloat16, device='cuda')
     one = torch.ones((), device='cuda')
-    be.fp8_gemm(y, 5, one, x, 5, one, out, a_kmajor=a_kmajor, b_kmajor=b_kmajor)
     want = (float(k) * torch.exp2((ex - 7).float()).view(nr, 1) * torch.exp2((ey - 7).float()).view(1, nc)).to(torch.bfloat16)
-    bad = (out != want) | out.isnan()
-    assert not bool(bad.any()), f'{int(bad.sum())} wrong outputs, first at {bad.nonzero()[0].tolist()}'
+    lib = be.load()
+    # the walk the rules pick, then each of the four registered by hand (what the timing at first use may choose)
+    be.tune_gemm_walks(False)
+    try:
+        for walk in (-1, 0, 1, 2, 3):
+            assert lib.msamp_fp8_gemm_set_walk(nc, nr, k, int(a_kmajor), int(b_kmajor), walk) == 0
+            assert lib.msamp_fp8_gemm_get_walk(nc, nr, k, int(a_kmajor), int(b_kmajor)) == walk
+            out.fill_(float('nan'))
+            be.fp8_gemm(y, 5, one, x, 5, one, out, a_kmajor=a_kmajor, b_kmajor=b_kmajor)
+            bad = (out != want) | out.isnan()
+            assert not bool(bad.any()), f'walk {walk}: {int(bad.sum())} wrong outputs, first at {bad.nonzero()[0].tolist()}'
+    finally:
+        lib.msamp_fp8_gemm_set_walk(nc, nr, k, int(a_kmajor), int(b_kmajor), -1)
+        be.tune_gemm_walks(True)
+
+
+def test_walk_timed_at_first_use_changes_no_bit(be):
+    """A problem with two rounds of tiles or more has its tile walks timed the first time it is seen (the call computes
+    the product some forty times over); whatever walk comes out, the product is the one of the rules' walk, bit for bit,
+    in that call and in the following ones, also through the entry point that casts on to E4M3; a problem met first
+    under stream capture, or a small one, is left to the rules."""
+    torch.manual_seed(21)
+    n, m, k = 8192, 4096, 1024    # 32 x 16 = 512 tiles
+    a = torch.randint(0, 0x78, (m, k), device='cuda', dtype=torch.uint8)
+    b = torch.randint(0, 0x78, (n, k), device='cuda', dtype=torch.uint8)
+    one = torch.ones((), device='cuda')
+    be.forget_gemm_walks()
+    be.tune_gemm_walks(False)
+    want = be.fp8_gemm(a, 5, one, b, 5, one, torch.empty(n, m, dtype=torch.bfloat16, device='cuda'))
+    assert be.load().msamp_fp8_gemm_get_walk(m, n, k, 0, 0) == -1
+    be.tune_gemm_walks(True)
+    try:
+        first = be.fp8_gemm(a, 5, one, b, 5, one, torch.full((n, m), float('nan'), dtype=torch.bfloat16, device='cuda'))
+        assert (m, n, k, False, False) in be._walk_seen
+        assert be.load().msamp_fp8_gemm_get_walk(m, n, k, 0, 0) in (-1, 0, 1, 2, 3)
+        second = be.fp8_gemm(a, 5, one, b, 5, one, torch.full((n, m), float('nan'), dtype=torch.bfloat16, device='cuda'))
+        assert torch.equal(first, want) and torch.equal(second, want)
+        # adding into an output never times (the timed launches would add forty times)
+        acc = want.clone()
+        be.forget_gemm_walks()
+        be.fp8_gemm(a, 5, one, b, 5, one, acc, accumulate=True)
+        assert not be._walk_seen
+        assert torch.equal(acc, (want.float() * 2).to(torch.bfloat16))
+        # the weight-gradient form: timed on a scratch product, then the fused call
+        at, bt = a.t().contiguous(), b.t().contiguous()
+        metas = [(torch.ones((), device='cuda'), torch.zeros(1, device='cuda'), torch.ones((), device='cuda')) for _ in range(2)]
+        be.tune_gemm_walks(False)
+        q0 = be.fp8_gemm_cast(at, 5, one, bt, 5, one, torch.bfloat16, 5, *metas[0], a_kmajor=True, b_kmajor=True)
+        be.tune_gemm_walks(True)
+        q1 = be.fp8_gemm_cast(at, 5, one, bt, 5, one, torch.bfloat16, 5, *metas[1], a_kmajor=True, b_kmajor=True)
+        assert (m, n, k, True, True) in be._walk_seen
+        assert q0 is not None and torch.equal(q0, q1) and all(torch.equal(u, v) for u, v in zip(metas[0], metas[1]))
+        # under capture nothing is timed and the problem stays unseen
+        be.forget_gemm_walks()
+        out = torch.empty(n, m, dtype=torch.bfloat16, device='cuda')
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            be.tune_gemm_walks(False)
+            be.fp8_gemm(a, 5, one, b, 5, one, out)    # (allocator and library warm-up on the side stream)
+            be.tune_gemm_walks(True)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            be.fp8_gemm(a, 5, one, b, 5, one, out)
+        assert not be._walk_seen
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+    finally:
+        be.forget_gemm_walks()
+        be.tune_gemm_walks(True)
