@@ -309,3 +309,30 @@ def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(gemm_a
     assert len(found) - len(small) >= 36 and len(small) == 9    # three output types x (row-major, Y K-major, both K-major)
     for name, (ours, compilers, scratch) in found.items():
         assert ours >= (320 if name in small else 512) and compilers == 0 and scratch == 0, (name, ours, compilers, scratch)
+
+
+def test_entry_points_refuse_bad_arguments_before_touching_a_gpu():
+    """Argument checks of the entry points run on the host before any HIP call: what they refuse, and the walk registry
+    (host data only), can be tried without a GPU."""
+    lib = _backend.load()
+    err = lambda: lib.msamp_last_error().decode()    # noqa: E731
+    # tile-walk registry: walks 0..3, -1 erases, anything else is refused
+    assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == -1
+    assert lib.msamp_fp8_gemm_set_walk(4096, 8192, 1024, 0, 0, 2) == 0
+    assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == 2
+    assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 1, 0) == -1 and lib.msamp_fp8_gemm_get_walk(8192, 4096, 1024, 0, 0) == -1
+    assert lib.msamp_fp8_gemm_set_walk(4096, 8192, 1024, 0, 0, 4) == -2 and 'walk=4' in err()
+    assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == 2
+    assert lib.msamp_fp8_gemm_set_walk(4096, 8192, 1024, 0, 0, -1) == 0
+    assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == -1
+    # the AdamW steps for float32 moments and for high-precision parameters
+    hyper = (1e-3, 0.9, 0.999, 1e-8, 0.01, 1, 1, 0, 0)
+    assert lib.msamp_adamw_f32(None, None, _backend.DT_F32, 0, None, None, *hyper, None) == 0          # nothing to do
+    assert lib.msamp_adamw_f32(None, None, _backend.DT_F32, 16, None, None, *hyper, None) == -3 and 'null' in err()
+    buf = (ctypes.c_float * 16)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.msamp_adamw_f32(p, p, _backend.DT_E4M3, 16, p, p, *hyper, None) == -1 and 'grad dtype' in err()
+    assert lib.msamp_adamw_plain_fused(None, 0, None, 0, _backend.DT_F32, _backend.DT_F32, *hyper, 1, None) == 0
+    assert lib.msamp_adamw_plain_fused(None, 3, None, 0, _backend.DT_F32, _backend.DT_F32, *hyper, 1, None) == -3
+    assert lib.msamp_adamw_plain_fused(p, 3, None, 0, _backend.DT_E5M2, _backend.DT_F32, *hyper, 1, None) == -1
+    assert lib.msamp_adamw_plain_fused(p, -1, None, 0, _backend.DT_F32, _backend.DT_F32, *hyper, 1, None) == -2
