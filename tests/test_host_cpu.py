@@ -336,3 +336,45 @@ def test_entry_points_refuse_bad_arguments_before_touching_a_gpu():
     assert lib.msamp_adamw_plain_fused(None, 3, None, 0, _backend.DT_F32, _backend.DT_F32, *hyper, 1, None) == -3
     assert lib.msamp_adamw_plain_fused(p, 3, None, 0, _backend.DT_E5M2, _backend.DT_F32, *hyper, 1, None) == -1
     assert lib.msamp_adamw_plain_fused(p, -1, None, 0, _backend.DT_F32, _backend.DT_F32, *hyper, 1, None) == -2
+
+
+def test_every_tile_walk_is_a_bijection(tmp_path):
+    """The function that maps a workgroup id to its output tile, taken as it stands in the kernel header and compiled for
+    the host: for every grid of 1..140 x 1..140 tiles and each of the four walks (groups of rows or of columns, the
+    XCD's patch turned or not -- the rules pick one, the timing at first use may pick any) every tile is taken exactly
+    once."""
+    import subprocess
+    src = open(os.path.join(os.path.dirname(_backend.library_path()), '..', 'csrc', 'gemm_kernels.cuh')).read()
+    start = src.index('__device__ __forceinline__ void tile_of_id(')
+    fn = src[start:src.index('\n}\n', start) + 3]
+    prog = '''#include <cstdio>
+#include <vector>
+#define __device__
+#define __forceinline__ inline
+''' + fn + '''
+int main() {
+    long checked = 0;
+    for (int tr = 1; tr <= 140; ++tr)
+        for (int tc = 1; tc <= 140; ++tc)
+            for (int walk = 0; walk < 4; ++walk) {
+                std::vector<char> seen(tr * tc, 0);
+                for (int id = 0; id < tr * tc; ++id) {
+                    int r = -1, c = -1;
+                    tile_of_id(id, tr, tc, walk & 1, (walk >> 1) & 1, r, c);
+                    if (r < 0 || r >= tr || c < 0 || c >= tc || seen[r * tc + c]) {
+                        printf("BAD %d x %d walk %d id %d -> %d %d\\n", tr, tc, walk, id, r, c);
+                        return 1;
+                    }
+                    seen[r * tc + c] = 1;
+                }
+                ++checked;
+            }
+    printf("OK %ld\\n", checked);
+    return 0;
+}
+'''
+    cpp, exe = tmp_path / 'walk.cpp', tmp_path / 'walk'
+    cpp.write_text(prog)
+    subprocess.run(['g++', '-O2', '-o', str(exe), str(cpp)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.strip() == 'OK 78400', out.stdout[-300:]
