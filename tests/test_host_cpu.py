@@ -344,7 +344,7 @@ def test_every_tile_walk_is_a_bijection(tmp_path):
     XCD's patch turned or not -- the rules pick one, the timing at first use may pick any) every tile is taken exactly
     once."""
     import subprocess
-    src = open(os.path.join(os.path.dirname(_backend.library_path()), '..', 'csrc', 'gemm_kernels.cuh')).read()
+    src = open(os.path.join(os.path.dirname(os.path.abspath(__file__)), '..', 'ms-amp_amd', 'csrc', 'gemm_kernels.cuh')).read()
     start = src.index('__device__ __forceinline__ void tile_of_id(')
     fn = src[start:src.index('\n}\n', start) + 3]
     prog = '''#include <cstdio>
