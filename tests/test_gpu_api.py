@@ -768,7 +768,7 @@ def test_small_plain_parameters_take_one_launch_with_the_bits_of_the_two_stages(
     moment scales move)."""
     shapes = [(1, ), (70, ), (4099, ), (3, 1000), (LBAdamW._PLAIN_LIMIT, ), (LBAdamW._PLAIN_LIMIT + 1, ), (3, 349_527), (1 << 20, )]
     dtypes = [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
-              (torch.float32, torch.bfloat16)]
+              (torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)]    # (the last: a bf16 module's bias)
     runs = {}
     for fused in (True, False):
         gen = torch.Generator(device='cuda').manual_seed(31)
