@@ -789,6 +789,18 @@ def bench_power(seconds=2.0):
     ms, row = sample_while(lambda: be.fp8_gemm(w, be.DT_E4M3, ws, x, be.DT_E4M3, xs, y), seconds)
     row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(2.0 * tokens * d_out * d_in / ms / 1e9, 1)})
     out['fp8_gemm_16384x28672x8192'] = row
+    # the vendor library on the same operands (hipBLASLt through torch._scaled_mm, its output allocated once): what it
+    # draws and at which clock, for the comparison of the two kernels' energy per flop
+    try:
+        x8, w8 = x.view(torch.float8_e4m3fn), w.view(torch.float8_e4m3fn)
+        one = torch.ones((), device='cuda')
+        vendor = lambda: torch._scaled_mm(x8, w8.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16, out=y)    # noqa: E731
+        vendor()
+        ms, row = sample_while(vendor, seconds)
+        row.update({'ms_per_call': round(ms, 4), 'TFLOPs': round(2.0 * tokens * d_out * d_in / ms / 1e9, 1)})
+        out['hipblaslt_16384x28672x8192'] = row
+    except (RuntimeError, AttributeError, TypeError) as exc:
+        out['hipblaslt_16384x28672x8192'] = {'skipped': str(exc)[:200]}
     del x, w, y
 
     # the forward GEMM of the Llama-7B QKV projection: K = 4096, where the time outside the K loop weighs most
