@@ -294,13 +294,15 @@ int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, 
 /* Tile walks of the 256 x 256-tile kernel (no counterpart in the reference, whose GEMM is cuBLASLt behind
  * transformer_engine_wrapper.py:63-103).  Which workgroup takes which output tile decides what the 32 compute units of
  * an XCD share through their L2; the library picks a walk from the shape by rules measured on Llama shapes, and the
- * best one for another shape can be up to 13 % faster.  A walk is a number 0..3: bit 0 = groups of eight tile columns
+ * best one for another shape can be up to 13 % faster.  A walk is a number 0..7: bit 0 = groups of eight tile columns
  * walked row by row (instead of groups of tile rows walked column by column), bit 1 = the XCD's patch of 32 tiles
- * turned, 4 of the grouped dimension by 8 of the walked one.  Every walk gives the same output bits.
+ * turned, 4 of the grouped dimension by 8 of the walked one; with both operands row-major a third bit (walks 4..7) makes
+ * the K loop await a slice's tile loads in two parts at two barriers instead of one (faster where the loads come from
+ * HBM, K of 24576 and more by the built-in rule; slower elsewhere).  Every walk gives the same output bits.
  * msamp_fp8_gemm_set_walk registers a walk for one problem -- (m, n, k) and operand layouts as in msamp_fp8_gemm_kmajor --
  * for all later calls of every GEMM entry point, walk = -1 removes it; msamp_fp8_gemm_get_walk returns it, -1 if none.
  * msamp_fp8_gemm_tune computes the product like msamp_fp8_gemm_kmajor with accumulate = 0 and, when the problem has at
- * least two rounds of tiles and `stream` is not being captured, times the rule's walk and the four explicit ones on the
+ * least two rounds of tiles and `stream` is not being captured, times the rule's walk and the explicit ones on the
  * operands given (some forty launches between HIP events; it synchronises with the stream) and registers the fastest if
  * it beats the rule's by more than 3 %; *chosen (nullable) receives the registered walk or -1.  Process-wide. */
 int msamp_fp8_gemm_set_walk(int m, int n, int k, int a_kmajor, int b_kmajor, int walk);

@@ -4,6 +4,7 @@
 // X (= B of the API, N rows) and the one that supplies D's columns is Y (= A of the API, M rows).
 #include "gemm_call.h"
 
+#include <algorithm>
 #include <atomic>
 #include <map>
 #include <mutex>
@@ -48,7 +49,7 @@ extern "C" void msamp_set_small_tile_limit(int big_tiles) {
 }
 
 extern "C" int msamp_fp8_gemm_set_walk(int m, int n, int k, int a_kmajor, int b_kmajor, int walk) {
-    MSAMP_REQUIRE(walk >= -1 && walk <= 3, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_set_walk: walk=%d", walk);
+    MSAMP_REQUIRE(walk >= -1 && walk <= 7, MSAMP_ERR_SHAPE, "msamp_fp8_gemm_set_walk: walk=%d", walk);
     // X = b (n rows of D), Y = a (m columns of D)
     const auto key = std::make_tuple(n, m, k, (b_kmajor ? 1 : 0) | (a_kmajor ? 2 : 0));
     std::lock_guard<std::mutex> lock(msamp::g_walk_mutex);
@@ -90,8 +91,14 @@ extern "C" int msamp_fp8_gemm_tune(const uint8_t* a, int a_type, const float* a_
     // milliseconds (at least four) between one pair of events
     float best_ms = 0.0f, rule_ms = 0.0f;
     int best = -1, rc = MSAMP_OK;
-    for (int turn = 0; turn < 6 && rc == MSAMP_OK; ++turn) {
-        const int walk = turn == 5 ? -1 : turn - 1;    // (the rule's walk once more at the end: a cold start must not cost it the comparison)
+    // (row-major operands: the fastest of the four once more with split waits, bit 2)
+    const bool can_split = !a_kmajor && !b_kmajor;
+    float explicit_ms[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int turns = can_split ? 7 : 6;
+    for (int turn = 0; turn < turns && rc == MSAMP_OK; ++turn) {
+        int walk = turn - 1;
+        if (turn == turns - 1) walk = -1;    // (the rule's walk once more at the end: a cold start must not cost it the comparison)
+        else if (turn == 5) walk = 4 + static_cast<int>(std::min_element(explicit_ms, explicit_ms + 4) - explicit_ms);
         msamp::t_forced_walk = walk;
         for (int i = 0; i < 2 && rc == MSAMP_OK; ++i) rc = run();
         int reps = 4;
@@ -103,6 +110,7 @@ extern "C" int msamp_fp8_gemm_tune(const uint8_t* a, int a_type, const float* a_
                                hipEventElapsedTime(&ms, e0, e1) != hipSuccess))
             rc = MSAMP_ERR_HIP;
         ms /= reps;
+        if (walk >= 0 && walk < 4) explicit_ms[walk] = ms;
         if (turn == 0) rule_ms = best_ms = ms;
         else if (walk < 0) rule_ms = std::min(rule_ms, ms);
         else if (ms < best_ms) best_ms = ms, best = walk;

@@ -52,7 +52,7 @@ int small_tile_limit();
 // The tile walk registered for this problem of the 256 x 256-tile kernel (msamp_fp8_gemm_set_walk / _tune), or -1: bit 0 =
 // groups of tile columns walked row by row instead of groups of tile rows, bit 1 = the XCD's patch of 32 tiles turned (4 of
 // the grouped dimension x 8 of the walked one).  Any walk gives the same output bits: it only decides which workgroup
-// takes which tile.
+// takes which tile.  Bit 2 (row-major operands only): the tile loads awaited in two parts, see the kernel.
 int registered_walk(int NR, int NC, int K, bool XT, bool YT);
 // ... which is this rule: K in whole slices, at least four of them; up to half the limit always (one small tile per
 // compute unit with the default limit), up to the limit where K is long enough for the second round of small tiles to

@@ -406,7 +406,8 @@ __device__ __forceinline__ v4f acc_quad(uint32_t token) {
     return r;
 }
 
-template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0, bool ODD_NK = false, bool QSPEC = false>
+template <int XF, int YF, typename OT, bool XT = false, bool YT = false, int QF = 0, bool ODD_NK = false, bool QSPEC = false,
+          bool SPLIT = false>
 __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_t* __restrict__ X,
                                                                      const uint8_t* __restrict__ Y, OT* __restrict__ D,
                                                                      int NR, int NC, int K,
@@ -445,6 +446,17 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         const int long_n = x_long ? NR : NC, short_n = x_long ? NC : NR;
         if (long_n >= 10240 && long_n % 256 == 0 && short_n <= 8192) by_columns = x_long, wide = true;
     }
+    // Split waits (template flag SPLIT, row-major operands only; the host picks the instantiation: bit 2 of a registered
+    // walk, else by rule).  A slice's sixteen tile loads are issued during the second half of a step and, in the plain
+    // form, all awaited at the one barrier in the middle of the next step: the last of them has half a step to
+    // arrive.  In the split form they are issued in the order of need -- X and Y blocks 0..3 of every wave's quadrant
+    // (read in the second half of the next step), then Y and X blocks 4..7 (read in the first half of the step after) --
+    // and awaited in two parts, the second at a barrier of its own at the start of that step: every load has three
+    // quarters of a step or more.  That pays where the loads miss the L2 and the memory-side cache (K = 28672 between
+    // 8192 x 8192 and 16384 x 8192 outputs: +4 to 5 %; 16384 cubed +3 %) and costs the second barrier elsewhere (-0.4 to
+    // -2 % at K of 4096 .. 16384), hence the rule on the host side.  (A flag read at run time instead of a second
+    // instantiation cost the plain form 3 to 7 %: the selects between the two orders sit in the K loop.)
+    static_assert(!SPLIT || (!XT && !YT && QF == 0 && !QSPEC), "split waits: plain row-major form only");
     // a walk registered for this problem (timed on this machine) overrides the rules
     if (qa.walk_plus_one > 0) by_columns = (qa.walk_plus_one - 1) & 1, wide = ((qa.walk_plus_one - 1) >> 1) & 1;
     tile_of_id(blockIdx.x, tiles_r, tiles_c, by_columns, wide, tr, tc);
@@ -485,7 +497,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
                      : static_cast<uint32_t>(gy) * static_cast<uint32_t>(K) + chunk * 16;
     }
     // one of the 16 loads of a slice (0..7: X rows, 8..15: Y rows), so they can be spread between MFMAs
-    auto dma = [&](int kt, int stage, int which) __attribute__((always_inline)) {
+    auto dma = [&](int kt, int stage, int i) __attribute__((always_inline)) {
+        // the i-th load of a slice is load i, or in the split form the i-th in order of need
+        constexpr int by_need[16] = {0, 1, 4, 5, 8, 9, 12, 13, 10, 11, 14, 15, 2, 3, 6, 7};
+        const int which = SPLIT ? by_need[i] : i;
         const bool is_x = which < 8;
         const size_t slice = static_cast<size_t>(kt) * kBK;
         const uint8_t* src = is_x ? X + (XT ? slice * NR : slice) : Y + (YT ? slice * NC : slice);
@@ -577,12 +592,21 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // slice kt is in registers now.  Barrier: slice kt + 1 has landed and nobody needs the LDS copy of slice kt.
     // Quarters 3, 4: X1 x Y0 while X half 0 of slice kt + 1 arrives, X1 x Y1 while its Y half 0 arrives; the stage of
     // slice kt is refilled with slice kt + 2 meanwhile.
-    auto slice = [&](int st, bool has_next, int ld_kt, bool do_load) __attribute__((always_inline)) {
+    // Split form: at the start of the step the second part of slice kt's loads has landed (behind it in the queue, if the
+    // step before issued loads -- prev_loaded --, the sixteen of slice kt + 1), and in the middle only the first part of
+    // slice kt + 1's is awaited.
+    auto slice = [&](int st, bool has_next, int ld_kt, bool do_load, bool prev_loaded = true) __attribute__((always_inline)) {
         constexpr std::integral_constant<int, 0> c0{};
         constexpr std::integral_constant<int, 1> c1{};
+        if constexpr (SPLIT) {
+            if (prev_loaded) wait_vmcnt<16>();
+            else wait_vmcnt<0>();
+            __syncthreads();
+        }
         quarter(c0, c0, fy[1], st, false, 1, true, 0, 0, 0, false);
         quarter(c0, c1, fx[1], st, true, 1, true, 0, 0, 0, false);
-        wait_vmcnt<0>();
+        if (SPLIT && has_next) wait_vmcnt<8>();
+        else wait_vmcnt<0>();
         __syncthreads();
         quarter(c1, c0, fx[0], st ^ 1, true, 0, has_next, ld_kt, st, 0, do_load);
         quarter(c1, c1, fy[0], st ^ 1, false, 0, has_next, ld_kt, st, 8, do_load);
@@ -611,10 +635,10 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     if constexpr (ODD_NK) {
         slice(0, true, kt + 2, true);
         slice(1, true, 0, false);
-        slice(0, false, 0, false);
+        slice(0, false, 0, false, false);
     } else {
         slice(0, true, 0, false);
-        slice(1, false, 0, false);
+        slice(1, false, 0, false, false);
     }
     // The workgroup that follows this one on the CU is, as a rule, the one 256 ids on (same XCD).  Touch the first two K
     // slices of its tile now -- one 4-byte load per 128-byte line, dropped into an LDS corner that nothing reads -- so that
@@ -1071,12 +1095,12 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
 
 // The kernel is built once for an even and once for an odd number of K slices (its last slices are straight-line
 // code); ODD picks the one that fits K.
-template <int XF, int YF, typename OT, bool XT, bool YT, bool ODD>
+template <int XF, int YF, typename OT, bool XT, bool YT, bool ODD, bool SPLIT = false>
 static int launch_gemm_dma_parity(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                                   const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     constexpr int smem = 2 * kDmaStage;
     static std::atomic<bool> configured{false};    // setting the attribute twice is harmless
-    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, 0, ODD>;
+    auto kern = fp8_gemm_dma_kernel<XF, YF, OT, XT, YT, 0, ODD, false, SPLIT>;
     if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(fp8_gemm_dma_kernel)");
@@ -1094,6 +1118,15 @@ static int launch_gemm_dma_parity(const uint8_t* X, const uint8_t* Y, void* D, i
 template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
 static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                            const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    if constexpr (!XT && !YT) {
+        // split waits: bit 2 of a walk registered for the problem, else from K = 24576 on (see the kernel)
+        const int walk = registered_walk(NR, NC, K, XT, YT);
+        if (walk >= 0 ? (walk & 4) != 0 : K >= 24576) {
+            if ((K / kBK) & 1)
+                return launch_gemm_dma_parity<XF, YF, OT, XT, YT, true, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+            return launch_gemm_dma_parity<XF, YF, OT, XT, YT, false, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+        }
+    }
     if ((K / kBK) & 1) return launch_gemm_dma_parity<XF, YF, OT, XT, YT, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
     return launch_gemm_dma_parity<XF, YF, OT, XT, YT, false>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
 }

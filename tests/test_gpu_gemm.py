@@ -769,7 +769,7 @@ def test_every_tile_is_written_whatever_the_walk(be, nr, nc, k, a_kmajor, b_kmaj
     # the walk the rules pick, then each of the four registered by hand (what the timing at first use may choose)
     be.tune_gemm_walks(False)
     try:
-        for walk in (-1, 0, 1, 2, 3):
+        for walk in (-1, 0, 1, 2, 3, 4, 7):    # (4..7: the split waits too; they apply to row-major operands only)
             assert lib.msamp_fp8_gemm_set_walk(nc, nr, k, int(a_kmajor), int(b_kmajor), walk) == 0
             assert lib.msamp_fp8_gemm_get_walk(nc, nr, k, int(a_kmajor), int(b_kmajor)) == walk
             out.fill_(float('nan'))
@@ -779,6 +779,40 @@ def test_every_tile_is_written_whatever_the_walk(be, nr, nc, k, a_kmajor, b_kmaj
     finally:
         lib.msamp_fp8_gemm_set_walk(nc, nr, k, int(a_kmajor), int(b_kmajor), -1)
         be.tune_gemm_walks(True)
+
+
+@pytest.mark.parametrize('n, m, k', [(1024, 768, 256), (2048, 1280, 384), (1536, 2048, 1152), (4096, 2048, 4096), (2304, 1792, 640),
+                                     (8192, 4096, 24576 + 128)])
+def test_split_waits_change_no_bit(be, large_tiles_only, n, m, k):
+    """With both operands row-major the K loop can await a slice's tile loads in two parts (bit 2 of a registered walk; by
+    rule from K = 24576 on): random codes, even and odd slice counts down to two and three, ragged edges, bias and sum
+    -- the same bits as the plain form and as the generic kernel."""
+    g = torch.Generator(device='cuda').manual_seed(n + m + k)
+    a = torch.randint(0, 0x7f, (m, k), device='cuda', dtype=torch.uint8, generator=g)
+    b = torch.randint(0, 0x7f, (n - 3, k), device='cuda', dtype=torch.uint8, generator=g)    # a ragged last tile row
+    a_si = torch.tensor(0.37, device='cuda')
+    b_si = torch.tensor(1.9, device='cuda')
+    bias = torch.randn(m, device='cuda', generator=g).bfloat16()
+    lib = be.load()
+    be.tune_gemm_walks(False)
+    outs = {}
+    try:
+        for walk in (0, 4, 1, 5, 6, 7, -1):
+            assert lib.msamp_fp8_gemm_set_walk(m, n - 3, k, 0, 0, walk) == 0
+            plain = be.fp8_gemm(a, 5, a_si, b, 6, b_si, torch.full((n - 3, m), float('nan'), dtype=torch.bfloat16, device='cuda'))
+            summed = be.fp8_gemm(a, 5, a_si, b, 6, b_si, plain.clone(), accumulate=True, bias=bias)
+            outs[walk] = (plain, summed)
+    finally:
+        lib.msamp_fp8_gemm_set_walk(m, n - 3, k, 0, 0, -1)
+        be.tune_gemm_walks(True)
+    for walk, (plain, summed) in outs.items():
+        assert torch.equal(plain.view(torch.int16), outs[0][0].view(torch.int16)), walk
+        assert torch.equal(summed.view(torch.int16), outs[0][1].view(torch.int16)), walk
+    if k <= 4096:
+        # the generic kernel (K made unfit for the direct-to-LDS kernel by 16 columns of zero codes)
+        pad = lambda t: torch.cat([t, torch.zeros(t.shape[0], 16, dtype=torch.uint8, device='cuda')], dim=1)    # noqa: E731
+        generic = be.fp8_gemm(pad(a), 5, a_si, pad(b), 6, b_si, torch.empty(n - 3, m, dtype=torch.bfloat16, device='cuda'))
+        assert torch.equal(generic.view(torch.int16), outs[0][0].view(torch.int16))
 
 
 def test_walk_timed_at_first_use_changes_no_bit(be):
@@ -799,7 +833,7 @@ def test_walk_timed_at_first_use_changes_no_bit(be):
     try:
         first = be.fp8_gemm(a, 5, one, b, 5, one, torch.full((n, m), float('nan'), dtype=torch.bfloat16, device='cuda'))
         assert (m, n, k, False, False) in be._walk_seen
-        assert be.load().msamp_fp8_gemm_get_walk(m, n, k, 0, 0) in (-1, 0, 1, 2, 3)
+        assert be.load().msamp_fp8_gemm_get_walk(m, n, k, 0, 0) in range(-1, 8)
         second = be.fp8_gemm(a, 5, one, b, 5, one, torch.full((n, m), float('nan'), dtype=torch.bfloat16, device='cuda'))
         assert torch.equal(first, want) and torch.equal(second, want)
         # adding into an output never times (the timed launches would add forty times)

@@ -316,12 +316,12 @@ def test_entry_points_refuse_bad_arguments_before_touching_a_gpu():
     (host data only), can be tried without a GPU."""
     lib = _backend.load()
     err = lambda: lib.msamp_last_error().decode()    # noqa: E731
-    # tile-walk registry: walks 0..3, -1 erases, anything else is refused
+    # tile-walk registry: walks 0..7, -1 erases, anything else is refused
     assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == -1
     assert lib.msamp_fp8_gemm_set_walk(4096, 8192, 1024, 0, 0, 2) == 0
     assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == 2
     assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 1, 0) == -1 and lib.msamp_fp8_gemm_get_walk(8192, 4096, 1024, 0, 0) == -1
-    assert lib.msamp_fp8_gemm_set_walk(4096, 8192, 1024, 0, 0, 4) == -2 and 'walk=4' in err()
+    assert lib.msamp_fp8_gemm_set_walk(4096, 8192, 1024, 0, 0, 8) == -2 and 'walk=8' in err()
     assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == 2
     assert lib.msamp_fp8_gemm_set_walk(4096, 8192, 1024, 0, 0, -1) == 0
     assert lib.msamp_fp8_gemm_get_walk(4096, 8192, 1024, 0, 0) == -1
