@@ -297,8 +297,8 @@ int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, 
  * best one for another shape can be up to 13 % faster.  A walk is a number 0..7: bit 0 = groups of eight tile columns
  * walked row by row (instead of groups of tile rows walked column by column), bit 1 = the XCD's patch of 32 tiles
  * turned, 4 of the grouped dimension by 8 of the walked one; with both operands row-major a third bit (walks 4..7) makes
- * the K loop await a slice's tile loads in two parts at two barriers instead of one (faster where the loads come from
- * HBM, K of 24576 and more by the built-in rule; slower elsewhere).  Every walk gives the same output bits.
+ * the K loop issue a slice's tile loads in the order of need over a whole step and await them in two parts at two
+ * barriers (1 to 8 % faster at K of 12288 and more, where the built-in rule takes it; level below).  Every walk gives the same output bits.
  * msamp_fp8_gemm_set_walk registers a walk for one problem -- (m, n, k) and operand layouts as in msamp_fp8_gemm_kmajor --
  * for all later calls of every GEMM entry point, walk = -1 removes it; msamp_fp8_gemm_get_walk returns it, -1 if none.
  * msamp_fp8_gemm_tune computes the product like msamp_fp8_gemm_kmajor with accumulate = 0 and, when the problem has at

@@ -447,15 +447,18 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
         if (long_n >= 10240 && long_n % 256 == 0 && short_n <= 8192) by_columns = x_long, wide = true;
     }
     // Split waits (template flag SPLIT, row-major operands only; the host picks the instantiation: bit 2 of a registered
-    // walk, else by rule).  A slice's sixteen tile loads are issued during the second half of a step and, in the plain
-    // form, all awaited at the one barrier in the middle of the next step: the last of them has half a step to
-    // arrive.  In the split form they are issued in the order of need -- X and Y blocks 0..3 of every wave's quadrant
-    // (read in the second half of the next step), then Y and X blocks 4..7 (read in the first half of the step after) --
-    // and awaited in two parts, the second at a barrier of its own at the start of that step: every load has three
-    // quarters of a step or more.  That pays where the loads miss the L2 and the memory-side cache (K = 28672 between
-    // 8192 x 8192 and 16384 x 8192 outputs: +4 to 5 %; 16384 cubed +3 %) and costs the second barrier elsewhere (-0.4 to
-    // -2 % at K of 4096 .. 16384), hence the rule on the host side.  (A flag read at run time instead of a second
-    // instantiation cost the plain form 3 to 7 %: the selects between the two orders sit in the K loop.)
+    // walk, else by rule).  In the plain form a slice's sixteen tile loads are issued during the second half of a step
+    // (the stage they fill is read until then) and all awaited at the one barrier in the middle of the next step: the
+    // last of them has half a step to arrive.  But a row-major load brings whole rows, and the rows of blocks 0..3 of
+    // every wave's quadrant were already read at the end of the step before.  In the split form the loads go out in the
+    // order of need, four per quarter of the step: X and Y blocks 0..3 of slice kt + 2 during the first half of step kt
+    // (after a barrier of its own at the start of the step: everybody has read those rows of slice kt), Y and X blocks
+    // 4..7 during the second half; the first part is awaited in the middle of step kt + 1, the second at the start of
+    // step kt + 2, each with sixteen younger loads in flight behind it: every load has one to one and a half steps.  That
+    // pays where the loads miss the L2 and the memory-side cache -- the longer K, the more: 16384 x 8192 x K at K = 12288
+    // +1 %, 14336 +5 %, 16384 +2 %, 20480 +5 %, 28672 +8 %, 16384 cubed +5 % -- and is level below (-0.8 to +0.8 % at K
+    // of 4096 .. 11008: the second barrier), hence the host's rule K >= 12288.  (A flag read at run time instead of a
+    // second instantiation cost the plain form 3 to 7 %: the selects between the two orders sat in the K loop.)
     static_assert(!SPLIT || (!XT && !YT && QF == 0 && !QSPEC), "split waits: plain row-major form only");
     // a walk registered for this problem (timed on this machine) overrides the rules
     if (qa.walk_plus_one > 0) by_columns = (qa.walk_plus_one - 1) & 1, wide = ((qa.walk_plus_one - 1) >> 1) & 1;
@@ -580,7 +583,11 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
 #pragma unroll
                     for (int p = n * np / 16; p < (n + 1) * np / 16; ++p) read_piece(rd_dst, rd_stage, rd_x, rd_half, p);
                 }
-                if (do_load && (n & 1)) dma(ld_kt, ld_stage, ld_first + (n >> 1));
+                if constexpr (SPLIT) {    // four loads per quarter, all four quarters
+                    if (do_load && (n & 3) == 3) dma(ld_kt, ld_stage, ld_first + (n >> 2));
+                } else {    // eight per quarter in the second half of the step
+                    if (do_load && (n & 1)) dma(ld_kt, ld_stage, ld_first + (n >> 1));
+                }
                 // Nothing moves across: one MFMA, then the reads and the load that go with it, so that the LDS reads and
                 // the tile loads stay spread evenly between the MFMAs as written.
                 __builtin_amdgcn_sched_barrier(0);
@@ -593,8 +600,8 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
     // Quarters 3, 4: X1 x Y0 while X half 0 of slice kt + 1 arrives, X1 x Y1 while its Y half 0 arrives; the stage of
     // slice kt is refilled with slice kt + 2 meanwhile.
     // Split form: at the start of the step the second part of slice kt's loads has landed (behind it in the queue, if the
-    // step before issued loads -- prev_loaded --, the sixteen of slice kt + 1), and in the middle only the first part of
-    // slice kt + 1's is awaited.
+    // step before issued loads -- prev_loaded --, the sixteen of slice kt + 1) and everybody is past the reads of the
+    // step before; the first part of slice kt + 2 then goes out during quarters 1 and 2, into the rows of blocks 0..3.
     auto slice = [&](int st, bool has_next, int ld_kt, bool do_load, bool prev_loaded = true) __attribute__((always_inline)) {
         constexpr std::integral_constant<int, 0> c0{};
         constexpr std::integral_constant<int, 1> c1{};
@@ -603,13 +610,18 @@ __global__ __launch_bounds__(kGemmThreads) void fp8_gemm_dma_kernel(const uint8_
             else wait_vmcnt<0>();
             __syncthreads();
         }
-        quarter(c0, c0, fy[1], st, false, 1, true, 0, 0, 0, false);
-        quarter(c0, c1, fx[1], st, true, 1, true, 0, 0, 0, false);
-        if (SPLIT && has_next) wait_vmcnt<8>();
-        else wait_vmcnt<0>();
+        quarter(c0, c0, fy[1], st, false, 1, true, ld_kt, st, 0, SPLIT && do_load);
+        quarter(c0, c1, fx[1], st, true, 1, true, ld_kt, st, 4, SPLIT && do_load);
+        if (SPLIT && has_next) {
+            // the first part of slice kt + 1; behind it its second part and, if this step loads, the first of slice kt + 2
+            if (do_load) wait_vmcnt<16>();
+            else wait_vmcnt<8>();
+        } else {
+            wait_vmcnt<0>();
+        }
         __syncthreads();
-        quarter(c1, c0, fx[0], st ^ 1, true, 0, has_next, ld_kt, st, 0, do_load);
-        quarter(c1, c1, fy[0], st ^ 1, false, 0, has_next, ld_kt, st, 8, do_load);
+        quarter(c1, c0, fx[0], st ^ 1, true, 0, has_next, ld_kt, st, SPLIT ? 8 : 0, do_load);
+        quarter(c1, c1, fy[0], st ^ 1, false, 0, has_next, ld_kt, st, SPLIT ? 12 : 8, do_load);
     };
 
     // prologue: slices 0 and 1 (the host sends no problem with fewer than two slices here); wait for slice 0; read
@@ -1119,9 +1131,9 @@ template <int XF, int YF, typename OT, bool XT = false, bool YT = false>
 static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, int NC, int K, const float* xs,
                            const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
     if constexpr (!XT && !YT) {
-        // split waits: bit 2 of a walk registered for the problem, else from K = 24576 on (see the kernel)
+        // split waits: bit 2 of a walk registered for the problem, else from K = 12288 on (see the kernel)
         const int walk = registered_walk(NR, NC, K, XT, YT);
-        if (walk >= 0 ? (walk & 4) != 0 : K >= 24576) {
+        if (walk >= 0 ? (walk & 4) != 0 : K >= 12288) {
             if ((K / kBK) & 1)
                 return launch_gemm_dma_parity<XF, YF, OT, XT, YT, true, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
             return launch_gemm_dma_parity<XF, YF, OT, XT, YT, false, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
