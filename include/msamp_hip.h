@@ -304,7 +304,7 @@ int msamp_fp8_gemm_cast(const uint8_t* a, int a_type, const float* a_scale_inv, 
  * msamp_fp8_gemm_tune computes the product like msamp_fp8_gemm_kmajor with accumulate = 0 and, when the problem has at
  * least two rounds of tiles and `stream` is not being captured, times the rule's walk and the explicit ones on the
  * operands given (some forty launches between HIP events; it synchronises with the stream) and registers the fastest if
- * it beats the rule's by more than 3 %; *chosen (nullable) receives the registered walk or -1.  Process-wide. */
+ * it beats the rule's by more than 5 %; *chosen (nullable) receives the registered walk or -1.  Process-wide. */
 int msamp_fp8_gemm_set_walk(int m, int n, int k, int a_kmajor, int b_kmajor, int walk);
 int msamp_fp8_gemm_get_walk(int m, int n, int k, int a_kmajor, int b_kmajor);
 int msamp_fp8_gemm_tune(const uint8_t* a, int a_type, const float* a_scale_inv, int a_kmajor, const uint8_t* b, int b_type,

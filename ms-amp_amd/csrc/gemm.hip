@@ -123,7 +123,7 @@ extern "C" int msamp_fp8_gemm_tune(const uint8_t* a, int a_type, const float* a_
         return run();
     }
     // an explicit walk is kept only where it beats the rule's by more than the timing's noise
-    if (best >= 0 && best_ms > 0.97f * rule_ms) best = -1;
+    if (best >= 0 && best_ms > 0.95f * rule_ms) best = -1;
     msamp_fp8_gemm_set_walk(m, n, k, a_kmajor, b_kmajor, best);
     if (chosen) *chosen = best;
     return MSAMP_OK;    // (d holds the product: every timed launch wrote it)
