@@ -46,6 +46,12 @@ struct GemmCall {
 
 template <int XF, int YF>
 int run_gemm_pair(const GemmCall& c);
+// The split-wait instantiations of the 256 x 256-tile kernel for one pair of formats (row-major operands, all three
+// output types, both parities of the slice count).  They live in translation units of their own (gemm_inst.hip built
+// with -DMSAMP_GEMM_SPLIT_UNIT) so that they compile beside the others instead of after them.
+template <int XF, int YF>
+int run_gemm_split(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, int NR, int NC, int K, const float* xs,
+                   const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st);
 
 // Problems of at most this many 256 x 256 tiles take the kernel with 128 x 128 tiles (msamp_set_small_tile_limit) ...
 int small_tile_limit();
@@ -71,5 +77,10 @@ extern template int run_gemm_pair<MSAMP_DT_E4M3, MSAMP_DT_E4M3>(const GemmCall&)
 extern template int run_gemm_pair<MSAMP_DT_E4M3, MSAMP_DT_E5M2>(const GemmCall&);
 extern template int run_gemm_pair<MSAMP_DT_E5M2, MSAMP_DT_E4M3>(const GemmCall&);
 extern template int run_gemm_pair<MSAMP_DT_E5M2, MSAMP_DT_E5M2>(const GemmCall&);
+#define MSAMP_SPLIT_ARGS const uint8_t*, const uint8_t*, void*, int, int, int, int, const float*, const float*, int, const void*, int, hipStream_t
+extern template int run_gemm_split<MSAMP_DT_E4M3, MSAMP_DT_E4M3>(MSAMP_SPLIT_ARGS);
+extern template int run_gemm_split<MSAMP_DT_E4M3, MSAMP_DT_E5M2>(MSAMP_SPLIT_ARGS);
+extern template int run_gemm_split<MSAMP_DT_E5M2, MSAMP_DT_E4M3>(MSAMP_SPLIT_ARGS);
+extern template int run_gemm_split<MSAMP_DT_E5M2, MSAMP_DT_E5M2>(MSAMP_SPLIT_ARGS);
 
 }    // namespace msamp

@@ -1134,9 +1134,8 @@ static int launch_gemm_dma(const uint8_t* X, const uint8_t* Y, void* D, int NR, 
         // split waits: bit 2 of a walk registered for the problem, else from K = 12288 on (see the kernel)
         const int walk = registered_walk(NR, NC, K, XT, YT);
         if (walk >= 0 ? (walk & 4) != 0 : K >= 12288) {
-            if ((K / kBK) & 1)
-                return launch_gemm_dma_parity<XF, YF, OT, XT, YT, true, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
-            return launch_gemm_dma_parity<XF, YF, OT, XT, YT, false, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
+            constexpr int d_dtype = std::is_same<OT, float>::value ? MSAMP_DT_F32 : std::is_same<OT, f16_t>::value ? MSAMP_DT_F16 : MSAMP_DT_BF16;
+            return run_gemm_split<XF, YF>(X, Y, D, d_dtype, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
         }
     }
     if ((K / kBK) & 1) return launch_gemm_dma_parity<XF, YF, OT, XT, YT, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st);
@@ -1316,6 +1315,23 @@ static int pick_out_spec(const uint8_t* X, const uint8_t* Y, void* D, int d_dtyp
             return launch_gemm_dma_spec<XF, YF, bf16_t, T, T>(X, Y, D, NR, NC, K, xs, ys, accumulate, qa, st);
     }
 }
+
+#ifdef MSAMP_GEMM_SPLIT_UNIT
+template <int XF, int YF>
+int run_gemm_split(const uint8_t* X, const uint8_t* Y, void* D, int d_dtype, int NR, int NC, int K, const float* xs,
+                   const float* ys, int accumulate, const void* bias, int bias_dt, hipStream_t st) {
+    const bool odd = (K / kBK) & 1;
+#define MSAMP_SPLIT_LAUNCH(OT)                                                                                                         \
+    return odd ? launch_gemm_dma_parity<XF, YF, OT, false, false, true, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st) \
+               : launch_gemm_dma_parity<XF, YF, OT, false, false, false, true>(X, Y, D, NR, NC, K, xs, ys, accumulate, bias, bias_dt, st)
+    switch (d_dtype) {
+        case MSAMP_DT_F32: MSAMP_SPLIT_LAUNCH(float);
+        case MSAMP_DT_F16: MSAMP_SPLIT_LAUNCH(f16_t);
+        default: MSAMP_SPLIT_LAUNCH(bf16_t);
+    }
+#undef MSAMP_SPLIT_LAUNCH
+}
+#endif
 
 // Everything behind the C entry points for one pair of operand formats.  gemm_inst.hip instantiates it once per
 // pair (four translation units, so that they compile side by side).

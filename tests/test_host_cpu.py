@@ -2,6 +2,7 @@
 error behaviour, and that the C-ABI library loads and exports every declared symbol."""
 
 import ctypes
+import itertools
 import json
 import os
 import re
@@ -267,18 +268,20 @@ def gemm_assembly(tmp_path_factory):
         pytest.skip('no hipcc here')
     src = os.path.join(os.path.dirname(_backend.__file__), '..', 'csrc')
     tmp = tmp_path_factory.mktemp('gemm_asm')
-    procs = {}
+    procs = []
     for xf, yf in GEMM_PAIRS:
-        out = str(tmp / f'gemm_inst_{xf}{yf}.s')
-        cmd = [hipcc, '--offload-arch=gfx950', '-O3', '-std=c++17', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
-               '-Wno-unused-command-line-argument', '-Wno-inline-asm', f'-DMSAMP_XF={xf}', f'-DMSAMP_YF={yf}',
-               '--cuda-device-only', '-S', '-o', out, os.path.join(src, 'gemm_inst.hip')]
-        procs[(xf, yf)] = (out, subprocess.Popen(cmd, cwd=src, stdout=subprocess.PIPE, stderr=subprocess.STDOUT))
+        # (each pair is two translation units: everything but the split-wait instantiations, and those)
+        for unit, extra in (('inst', []), ('split', ['-DMSAMP_GEMM_SPLIT_UNIT'])):
+            out = str(tmp / f'gemm_{unit}_{xf}{yf}.s')
+            cmd = [hipcc, '--offload-arch=gfx950', '-O3', '-std=c++17', '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+                   '-Wno-unused-command-line-argument', '-Wno-inline-asm', f'-DMSAMP_XF={xf}', f'-DMSAMP_YF={yf}', *extra,
+                   '--cuda-device-only', '-S', '-o', out, os.path.join(src, 'gemm_inst.hip')]
+            procs.append(((xf, yf), out, subprocess.Popen(cmd, cwd=src, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
     paths = {}
-    for pair, (out, proc) in procs.items():
+    for pair, out, proc in procs:
         log = proc.communicate()[0]
         assert proc.returncode == 0, log.decode(errors='replace')[-2000:]
-        paths[pair] = out
+        paths.setdefault(pair, []).append(out)
     return paths
 
 
@@ -289,7 +292,7 @@ def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(gemm_a
     memory.  Each pair of operand formats is a translation unit of its own with its own register allocation: look at
     the assembly of all four."""
     kernel, in_asm, found = None, False, {}
-    for line in open(gemm_assembly[pair]):
+    for line in itertools.chain.from_iterable(open(path) for path in gemm_assembly[pair]):
         m = re.match(r'^(_Z\w+):', line)
         if m:
             kernel = m.group(1)
@@ -306,7 +309,8 @@ def test_direct_to_lds_gemm_kernels_leave_the_accumulator_registers_alone(gemm_a
     # bf16 / f16 / float outputs, row- and K-major operands, both parities, the fused and the speculative cast; and the
     # kernel with 128 x 128 tiles, which keeps 64 accumulator registers the same way
     small = [k for k in found if 'fp8_gemm_dma128_kernel' in k]
-    assert len(found) - len(small) >= 36 and len(small) == 9    # three output types x (row-major, Y K-major, both K-major)
+    assert len(found) - len(small) >= 42 and len(small) == 9    # three output types x (row-major, Y K-major, both K-major)
+    assert sum('Lb1EEEv' in k for k in found if k not in small) == 6    # the split-wait instantiations: three output types, two parities
     for name, (ours, compilers, scratch) in found.items():
         assert ours >= (320 if name in small else 512) and compilers == 0 and scratch == 0, (name, ours, compilers, scratch)
 
